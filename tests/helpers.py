@@ -1,0 +1,67 @@
+"""Shared by the tests: the tiny configurations, model folders, the oracle."""
+from __future__ import annotations
+
+import functools
+import json
+import os
+
+import torch
+
+# Two tiny configurations that differ in every size and option.
+TINY_A = dict(
+    architectures=["Qwen3ForCausalLM"], hidden_size=64, num_hidden_layers=2,
+    num_attention_heads=4, num_key_value_heads=2, head_dim=16, intermediate_size=128,
+    vocab_size=256, max_position_embeddings=128, rms_norm_eps=1e-6, rope_theta=10000.0,
+    tie_word_embeddings=True, use_sliding_window=False,
+)
+TINY_B = dict(
+    architectures=["Qwen3ForCausalLM"], hidden_size=96, num_hidden_layers=3,
+    num_attention_heads=8, num_key_value_heads=2, head_dim=32, intermediate_size=200,
+    vocab_size=320, max_position_embeddings=256, rms_norm_eps=1e-5, rope_theta=1000000.0,
+    tie_word_embeddings=False, use_sliding_window=True, sliding_window=24, max_window_layers=1,
+)
+TINY_CONFIGS = {"A": (TINY_A, 11), "B": (TINY_B, 23)}
+PAGE_SIZE = {"A": 16, "B": 8}
+
+
+def make_model_dir(path: str, cfg: dict, seed: int, dtype: str = "bfloat16") -> str:
+    from tffinfer_amd.weights import write_random_model
+    write_random_model(path, dict(cfg), seed, dtype=dtype)
+    return path
+
+
+def random_tokens(n: int, vocab: int, seed: int) -> list[int]:
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+@functools.lru_cache(maxsize=64)
+def _oracle_cached(model_dir: str, tokens: tuple) -> torch.Tensor:
+    from plain_qwen3 import fast_forward, load_plain_model
+    cfg, raw = load_plain_model(model_dir, torch.float64)
+    return fast_forward(cfg, raw, list(tokens))
+
+
+def oracle_logits(model_dir: str, tokens) -> torch.Tensor:
+    """float64 logits [T, V] of the plain implementation for a whole sequence."""
+    return _oracle_cached(model_dir, tuple(int(t) for t in tokens))
+
+
+def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
+    """Largest absolute difference over the largest reference magnitude."""
+    got = got.double().cpu()
+    ref = ref.double().cpu()
+    return float((got - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+
+
+# Tolerances on rel_err.  float32: the engine differs from a float64 run by
+# rounding only.  bfloat16: weights are the same bfloat16 values in both runs;
+# the engine rounds activations to bfloat16 between kernels (relative step
+# 2^-8), which over a few layers stays within a few percent of the logits'
+# range.  A fault of the cache or a kernel moves logits by tens of percent.
+TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+
+
+def read_config(model_dir: str) -> dict:
+    with open(os.path.join(model_dir, "config.json")) as f:
+        return json.load(f)

@@ -1,0 +1,311 @@
+"""Each kernel alone against a plain float64 computation of the same op, at
+sizes other than the engine's."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _ops():
+    from tffinfer_amd.kernels import ops
+    return ops
+
+
+def _close(got, ref, tol, what=""):
+    got, ref = got.double().cpu(), ref.double().cpu()
+    err = float((got - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+    assert err <= tol, f"{what}: rel. error {err:.3e} > {tol:.1e}"
+    return err
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(dtype):
+    ops = _ops()
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn(77, 40, generator=g).to(dtype)
+    ids = torch.tensor([0, 76, 5, 5, 33], dtype=torch.int32)
+    out = ops.embed(table.to(DEV), ids.to(DEV))
+    assert out.dtype == torch.float32
+    assert torch.equal(out.cpu(), table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("H", [40, 96, 1000, 4096, 5120])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_add_rmsnorm(H, out_dtype):
+    ops = _ops()
+    g = torch.Generator().manual_seed(H)
+    n = 7
+    resid = torch.randn(n, H, generator=g) * 3
+    delta = torch.randn(n, H, generator=g)
+    w = 1 + 0.1 * torch.randn(H, generator=g)
+    eps = 1e-3
+    v = (resid + delta).double()
+    ref = v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps) * w.double()
+    r = resid.to(DEV).clone()
+    out = ops.add_rmsnorm(r, delta.to(DEV), w.to(DEV), eps, out_dtype)
+    _close(out, ref, 1e-6 if out_dtype == torch.float32 else 8e-3, "norm")
+    _close(r, v, 1e-6, "residual sum stored back")
+    # gathered rows: residual untouched, norm of resid + delta of those rows
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32)
+    r2 = resid.to(DEV).clone()
+    out2 = ops.add_rmsnorm(r2, delta.to(DEV), w.to(DEV), eps, out_dtype, rows=rows.to(DEV))
+    _close(out2, ref[rows.long()], 1e-6 if out_dtype == torch.float32 else 8e-3, "gathered norm")
+    assert torch.equal(r2.cpu(), resid)
+    # no delta
+    out3 = ops.add_rmsnorm(r2, None, w.to(DEV), eps, out_dtype)
+    v3 = resid.double()
+    _close(out3, v3 * torch.rsqrt((v3 * v3).mean(-1, keepdim=True) + eps) * w.double(),
+           1e-6 if out_dtype == torch.float32 else 8e-3, "norm without delta")
+
+
+def test_rmsnorm_eps_position():
+    """eps is added to the mean inside the root: a row of tiny values tells it
+    from eps added to the sum or outside the root."""
+    ops = _ops()
+    H = 64
+    x = torch.full((1, H), 1e-3)
+    w = torch.ones(H)
+    eps = 1e-5
+    out = ops.add_rmsnorm(x.to(DEV).clone(), None, w.to(DEV), eps, torch.float32)
+    want = 1e-3 / math.sqrt(1e-6 + eps)
+    assert abs(float(out[0, 0]) - want) / want < 1e-5
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 320, 96), (33, 200, 200), (130, 130, 72), (257, 96, 256),
+                                    (64, 4096, 512), (300, 1000, 1024)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear(M, N, K, dtype):
+    ops = _ops()
+    g = torch.Generator().manual_seed(M * 1000 + N)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) * 0.1).to(dtype)
+    ref = x.double() @ w.double().T
+    out = ops.linear(x.to(DEV), w.to(DEV), out_dtype=torch.float32)
+    _close(out, ref, 2e-6 if dtype == torch.float32 else 2e-5, f"linear {M}x{N}x{K} f32 out")
+    if dtype == torch.bfloat16:
+        out_b = ops.linear(x.to(DEV), w.to(DEV))
+        assert out_b.dtype == torch.bfloat16
+        _close(out_b, ref, 6e-3, "linear bf16 out")
+    # strided rows (a slice of a wider matrix)
+    wide = torch.randn(M, K + 16, generator=g).to(dtype).to(DEV)
+    out_s = ops.linear(wide[:, :K], w.to(DEV), out_dtype=torch.float32)
+    _close(out_s, wide[:, :K].double().cpu() @ w.double().T, 2e-6 if dtype == torch.float32 else 2e-5, "strided")
+
+
+def test_linear_identity_and_layout():
+    """[out, in] layout: a non-square weight picks input columns."""
+    ops = _ops()
+    x = torch.arange(24, dtype=torch.float32).reshape(3, 8)
+    w = torch.zeros(2, 8)
+    w[0, 3] = 1.0
+    w[1, 7] = 2.0
+    out = ops.linear(x.to(DEV), w.to(DEV)).cpu()
+    assert torch.equal(out[:, 0], x[:, 3]) and torch.equal(out[:, 1], 2 * x[:, 7])
+
+
+def test_linear_refuses_bad_inner_size():
+    from tffinfer_amd.kernels.lib import KernelError
+    ops = _ops()
+    x = torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(8, 12, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(KernelError, match="multiple of 8"):
+        ops.linear(x, w)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("I", [200, 64, 1023])
+def test_swiglu(dtype, I):
+    ops = _ops()
+    g = torch.Generator().manual_seed(I)
+    gu = (torch.randn(5, 2 * I, generator=g) * 3).to(dtype)
+    gt, up = gu[:, :I].double(), gu[:, I:].double()
+    ref = gt / (1 + torch.exp(-gt)) * up
+    out = ops.swiglu(gu.to(DEV))
+    _close(out, ref, 1e-6 if dtype == torch.float32 else 8e-3, "swiglu")
+    # roles: zero up gives zero, zero gate gives zero; silu(x) -> x for large x
+    z = torch.zeros(1, 2 * I, dtype=dtype)
+    z[:, :I] = 30.0
+    z[:, I:] = 1.0
+    assert torch.allclose(ops.swiglu(z.to(DEV)).float().cpu(), torch.full((1, I), 30.0), rtol=1e-2)
+
+
+def _paged_setup(T_ctx, nkv, d, ps, dtype, seed, extra_pages=3):
+    """A cache whose pages are deliberately out of order."""
+    g = torch.Generator().manual_seed(seed)
+    nblk = -(-T_ctx // ps)
+    num_pages = nblk + extra_pages
+    perm = torch.randperm(num_pages, generator=g)[:nblk]
+    k = torch.randn(T_ctx, nkv, d, generator=g).to(dtype)
+    v = torch.randn(T_ctx, nkv, d, generator=g).to(dtype)
+    kc = torch.zeros(num_pages, nkv, ps, d, dtype=dtype)
+    vc = torch.zeros(num_pages, nkv, ps, d, dtype=dtype)
+    for j in range(T_ctx):
+        kc[perm[j // ps], :, j % ps] = k[j]
+        vc[perm[j // ps], :, j % ps] = v[j]
+    return k, v, kc, vc, perm.to(torch.int32)
+
+
+def _attn_ref(q, k, v, positions, window, scale):
+    T, nq, d = q.shape
+    G = nq // k.shape[1]
+    out = torch.zeros(T, nq, d, dtype=torch.float64)
+    for t in range(T):
+        p = int(positions[t])
+        lo = 0 if window <= 0 else max(0, p - window + 1)
+        for h in range(nq):
+            s = (k[lo:p + 1, h // G].double() @ q[t, h].double()) * scale
+            w = torch.softmax(s, 0)
+            out[t, h] = w @ v[lo:p + 1, h // G].double()
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,d,ps,window", [(4, 2, 16, 16, 0), (6, 3, 48, 8, 0), (8, 2, 32, 8, 24),
+                                                (5, 5, 80, 32, 0), (16, 2, 128, 16, 100), (3, 1, 256, 64, 0)])
+def test_attention_generic(dtype, nq, nkv, d, ps, window):
+    ops = _ops()
+    ctx = 150
+    k, v, kc, vc, table = _paged_setup(ctx, nkv, d, ps, dtype, seed=nq * d)
+    g = torch.Generator().manual_seed(1)
+    # queries at scattered positions of one request, including the first and the last
+    positions = torch.tensor([0, 1, ps - 1, ps, 63, 64, 65, 100, ctx - 1], dtype=torch.int32)
+    T = positions.numel()
+    q = torch.randn(T, nq, d, generator=g).to(dtype)
+    scale = 1 / math.sqrt(d)
+    ref = _attn_ref(q, k, v, positions, window, scale)
+    out = ops.attention_generic(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kc.to(DEV), vc.to(DEV),
+                                table[None].contiguous().to(DEV), torch.zeros(T, dtype=torch.int32, device=DEV),
+                                positions.to(DEV), window, scale)
+    _close(out.reshape(T, nq, d), ref, 2e-6 if dtype == torch.float32 else 1e-2, "attention")
+
+
+def test_attention_far_key_stands_out():
+    """One key among hundreds is made to dominate: the output must be its value."""
+    ops = _ops()
+    nq, nkv, d, ps, ctx = 4, 2, 32, 16, 700
+    k, v, kc, vc, table = _paged_setup(ctx, nkv, d, ps, torch.float32, seed=5)
+    far = 3
+    q = torch.randn(1, nq, d)
+    q[0, 1] = q[0, 0]   # the two heads of a group share a query, so one key can serve both
+    q[0, 3] = q[0, 2]
+    for gidx, h in ((0, 0), (1, 2)):
+        kc[table[far // ps], gidx, far % ps] = 200 * q[0, h] / q[0, h].norm()
+    out = ops.attention_generic(q.reshape(1, nq * d).to(DEV), nq, nkv, d, kc.to(DEV), vc.to(DEV),
+                                table[None].contiguous().to(DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
+                                torch.tensor([ctx - 1], dtype=torch.int32, device=DEV), 0, 1 / math.sqrt(d))
+    out = out.reshape(nq, d).cpu()
+    for h in range(nq):
+        assert torch.allclose(out[h], v[far, h // 2], atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("pairing", ["half", "interleaved"])
+@pytest.mark.parametrize("nq,nkv,d,rot", [(4, 2, 16, 16), (3, 1, 48, 48), (8, 2, 128, 128), (2, 2, 64, 32)])
+def test_qk_norm_rope_kv(dtype, pairing, nq, nkv, d, rot):
+    ops = _ops()
+    from tffinfer_amd.parts.position import RotaryEmbedding
+    T, ps, num_pages, eps, theta = 9, 8, 6, 1e-5, 5000.0
+    g = torch.Generator().manual_seed(d)
+    qkv = torch.randn(T, (nq + 2 * nkv) * d, generator=g).to(dtype)
+    qw = 1 + 0.1 * torch.randn(d, generator=g)
+    kw = 1 + 0.1 * torch.randn(d, generator=g)
+    positions = torch.tensor([0, 1, 2, 17, 18, 40, 41, 42, 99], dtype=torch.int32)
+    slots = torch.tensor([3, 47, 8, 9, 10, -1, 0, 1, 2], dtype=torch.int32)
+    rope = RotaryEmbedding(d, theta, pairing, rotary_dim=rot)
+    table = rope.table(128, DEV)
+    kc = torch.zeros(num_pages, nkv, ps, d, dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    dq = qkv.to(DEV).clone()
+    ops.qk_norm_rope_kv(dq, nq, nkv, d, qw.to(DEV), kw.to(DEV), eps, table, 1 if pairing == "interleaved" else 0,
+                        positions.to(DEV), slots.to(DEV), kc, vc)
+    x = qkv.double()
+    q = x[:, :nq * d].reshape(T, nq, d)
+    k = x[:, nq * d:(nq + nkv) * d].reshape(T, nkv, d)
+    v = x[:, (nq + nkv) * d:].reshape(T, nkv, d)
+
+    def norm(a, w):
+        return a * torch.rsqrt((a * a).mean(-1, keepdim=True) + eps) * w.double()
+
+    def rotate(a):
+        ang = positions.double()[:, None] * torch.exp(-(2.0 * torch.arange(rot // 2).double() / rot) * math.log(theta))
+        c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        out = a.clone()
+        if pairing == "half":
+            lo, hi = a[..., :rot // 2], a[..., rot // 2:rot]
+            out[..., :rot // 2] = lo * c - hi * s
+            out[..., rot // 2:rot] = lo * s + hi * c
+        else:
+            ev, od = a[..., 0:rot:2], a[..., 1:rot:2]
+            out[..., 0:rot:2] = ev * c - od * s
+            out[..., 1:rot:2] = ev * s + od * c
+        return out
+
+    tol = 2e-6 if dtype == torch.float32 else 8e-3
+    qr, kr = rotate(norm(q, qw)), rotate(norm(k, kw))
+    _close(dq[:, :nq * d].reshape(T, nq, d), qr, tol, "q")
+    kc_h, vc_h = kc.cpu(), vc.cpu()
+    written = set()
+    for t in range(T):
+        s = int(slots[t])
+        if s < 0:
+            continue
+        written.add(s)
+        _close(kc_h[s // ps, :, s % ps], kr[t], tol, f"k of token {t}")
+        _close(vc_h[s // ps, :, s % ps], v[t], tol if dtype == torch.bfloat16 else 0.0, f"v of token {t}")
+    for s in range(num_pages * ps):
+        if s not in written:
+            assert float(kc_h[s // ps, :, s % ps].abs().max()) == 0.0, f"slot {s} was written"
+
+
+def test_argmax_first_maximum():
+    ops = _ops()
+    x = torch.randn(6, 5000)
+    x[0, 77] = x[0, 4000] = 100.0
+    x[1, 4999] = 50.0
+    x[2, 0] = 50.0
+    out = ops.argmax(x.to(DEV)).cpu()
+    assert out[0] == 77 and out[1] == 4999 and out[2] == 0
+    assert torch.equal(out[3:].long(), x[3:].argmax(-1))
+
+
+@pytest.mark.parametrize("V", [320, 5000, 151936])
+def test_sample_distribution_and_draw(V):
+    from plain_qwen3 import plain_inverse_cdf, plain_probs
+    ops = _ops()
+    g = torch.Generator().manual_seed(V)
+    R = 6
+    logits = torch.randn(R, V, generator=g) * 3
+    temp = torch.tensor([0.8, 1.0, 0.5, 1.3, 0.0, 0.7])
+    top_k = torch.tensor([0, 50, 0, 10, 5, 0], dtype=torch.int32)
+    top_p = torch.tensor([1.0, 1.0, 0.9, 0.8, 0.5, 1.0])
+    min_p = torch.tensor([0.0, 0.0, 0.0, 0.0, 0.0, 0.05])
+    u = torch.tensor([0.3, 0.999, 0.0, 0.5, 0.7, 0.42])
+    tok, probs = ops.sample(logits.to(DEV), temp.to(DEV), u.to(DEV), top_k.to(DEV), top_p.to(DEV),
+                            min_p.to(DEV), return_probs=True)
+    tok, probs = tok.cpu(), probs.cpu()
+    for r in range(R):
+        if temp[r] == 0:
+            assert tok[r] == logits[r].argmax()
+            continue
+        ref = plain_probs(logits[r], float(temp[r]), int(top_k[r]), float(top_p[r]), float(min_p[r]))
+        assert int((ref > 0).sum()) == int((probs[r] > 0).sum()), f"row {r}: kept sets differ"
+        assert float((probs[r].double() - ref).abs().max()) < 1e-6
+        assert tok[r] == plain_inverse_cdf(ref, float(u[r]))
+
+
+def test_repetition_penalty():
+    from plain_qwen3 import plain_repetition_penalty
+    ops = _ops()
+    logits = torch.randn(2, 100)
+    seen = [[3, 7, 50], [99, 0]]
+    flat = torch.tensor(seen[0] + seen[1], dtype=torch.int32)
+    cu = torch.tensor([0, 3, 5], dtype=torch.int32)
+    pen = torch.tensor([1.3, 2.0])
+    d = logits.to(DEV).clone()
+    ops.repetition_penalty(d, flat.to(DEV), cu.to(DEV), pen.to(DEV))
+    for r in range(2):
+        assert torch.allclose(d[r].cpu(), plain_repetition_penalty(logits[r], seen[r], float(pen[r])))

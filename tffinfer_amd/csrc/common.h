@@ -1,0 +1,72 @@
+// Shared helpers of the gfx950 kernels: element types, wave and block
+// reductions, the error channel of the C entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16_t;
+
+// Element type codes of the C entry points.
+enum { TFF_F32 = 0, TFF_BF16 = 1 };
+
+#define TFF_WAVE 64
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return (float)v; }
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return (bf16_t)v; }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// Sum over a block of up to 1024 threads; `red` holds at least 17 floats.
+// Every thread gets the result.  The order of the additions is fixed.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nwave = (blockDim.x + 63) >> 6;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float s = 0.f;
+        for (int i = 0; i < nwave; ++i) s += red[i];
+        red[16] = s;
+    }
+    __syncthreads();
+    return red[16];
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nwave = (blockDim.x + 63) >> 6;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float s = red[0];
+        for (int i = 1; i < nwave; ++i) s = fmaxf(s, red[i]);
+        red[16] = s;
+    }
+    __syncthreads();
+    return red[16];
+}
+
+// Host side: the entry points return 0 or a negative code and leave a message
+// that tff_last_error() hands out.
+int tff_fail(const char* fmt, ...);
+int tff_check_launch(const char* what);
+
+#define TFF_REQUIRE(cond, ...)                     \
+    do {                                           \
+        if (!(cond)) return tff_fail(__VA_ARGS__); \
+    } while (0)

@@ -1,0 +1,309 @@
+// Row-wise and element-wise kernels: embedding gather, fused residual sum and
+// RMS norm, per-head q/k norm with rotation and the cache write, SwiGLU, casts.
+// All arithmetic is float32; only loads and stores see bfloat16.
+#include "common.h"
+#include "tffinfer_kernels.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+// ---------------------------------------------------------------- errors ---
+static thread_local char g_error[1024] = "";
+
+int tff_fail(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return -1;
+}
+int tff_check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return tff_fail("%s: launch failed: %s", what, hipGetErrorString(e));
+    return 0;
+}
+TFF_API const char* tff_last_error() { return g_error; }
+TFF_API int tff_abi_version() { return 3; }
+
+// ----------------------------------------------------------------- embed ---
+// x[t, :] = E[token[t], :]   (reference: src/kernel/cpu/embedding.cpp:34-49,
+// done there on the CPU; here a gather on the device into the float32
+// residual stream).
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
+                             float* __restrict__ out, int H, int V) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    const bool bad = id < 0 || id >= V;
+    if (bad) id = 0;
+    const T* row = table + (size_t)id * H;
+    float* o = out + (size_t)t * H;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) o[j] = bad ? __builtin_nanf("") : to_f32(row[j]);
+}
+
+TFF_API int tff_embed(const void* table, const int32_t* ids, float* out, int T, int H, int V,
+                      int dtype, tff_stream_t stream) {
+    TFF_REQUIRE(table && ids && out, "embed: null pointer");
+    TFF_REQUIRE(T >= 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TFF_F32)
+        embed_kernel<float><<<T, 256, 0, s>>>((const float*)table, ids, out, H, V);
+    else if (dtype == TFF_BF16)
+        embed_kernel<bf16_t><<<T, 256, 0, s>>>((const bf16_t*)table, ids, out, H, V);
+    else
+        return tff_fail("embed: unknown dtype %d", dtype);
+    return tff_check_launch("embed");
+}
+
+// ----------------------------------------------------------- add+rmsnorm ---
+// y_j = v_j * rsqrt(mean(v^2) + eps) * w_j, v = resid (+ delta)
+// (reference: src/kernel/cuda/norm.cu:31-48; the residual sum of
+// src/kernel/cuda/binary.cu:16-29 is folded in).
+template <typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __restrict__ delta,
+                                   const float* __restrict__ w, float eps, TO* __restrict__ out,
+                                   const int32_t* __restrict__ rows, int H) {
+    __shared__ float red[17];
+    const int i = blockIdx.x;
+    const int r = rows ? rows[i] : i;
+    float* x = resid + (size_t)r * H;
+    const float* dl = delta ? delta + (size_t)r * H : nullptr;
+    const bool store = rows == nullptr && dl != nullptr;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) {
+        float v = x[j];
+        if (dl) v += dl[j];
+        if (store) x[j] = v;
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_sum(ss, red);
+    const float rr = rsqrtf(ss / (float)H + eps);
+    TO* o = out + (size_t)i * H;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) {
+        float v = x[j];
+        if (dl && !store) v += dl[j];
+        o[j] = from_f32<TO>(v * rr * w[j]);
+    }
+}
+
+TFF_API int tff_add_rmsnorm(float* resid, const float* delta, const float* weight, float eps,
+                            void* out, const int32_t* rows, int n, int H, int out_dtype,
+                            tff_stream_t stream) {
+    TFF_REQUIRE(resid && weight && out, "add_rmsnorm: null pointer");
+    TFF_REQUIRE(n >= 0 && H > 0, "add_rmsnorm: bad sizes n=%d H=%d", n, H);
+    if (n == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = H >= 2048 ? 1024 : 256;
+    if (out_dtype == TFF_F32)
+        add_rmsnorm_kernel<float><<<n, threads, 0, s>>>(resid, delta, weight, eps, (float*)out, rows, H);
+    else if (out_dtype == TFF_BF16)
+        add_rmsnorm_kernel<bf16_t><<<n, threads, 0, s>>>(resid, delta, weight, eps, (bf16_t*)out, rows, H);
+    else
+        return tff_fail("add_rmsnorm: unknown dtype %d", out_dtype);
+    return tff_check_launch("add_rmsnorm");
+}
+
+template <typename T>
+__global__ void rmsnorm_kernel(const T* __restrict__ x, const float* __restrict__ w, float eps,
+                               T* __restrict__ out, int H) {
+    __shared__ float red[17];
+    const T* xr = x + (size_t)blockIdx.x * H;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) {
+        const float v = to_f32(xr[j]);
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_sum(ss, red);
+    const float rr = rsqrtf(ss / (float)H + eps);
+    T* o = out + (size_t)blockIdx.x * H;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) o[j] = from_f32<T>(to_f32(xr[j]) * rr * w[j]);
+}
+
+TFF_API int tff_rmsnorm(const void* x, const float* weight, float eps, void* out, int n, int H,
+                        int dtype, tff_stream_t stream) {
+    TFF_REQUIRE(x && weight && out, "rmsnorm: null pointer");
+    TFF_REQUIRE(n >= 0 && H > 0, "rmsnorm: bad sizes n=%d H=%d", n, H);
+    if (n == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TFF_F32)
+        rmsnorm_kernel<float><<<n, 256, 0, s>>>((const float*)x, weight, eps, (float*)out, H);
+    else if (dtype == TFF_BF16)
+        rmsnorm_kernel<bf16_t><<<n, 256, 0, s>>>((const bf16_t*)x, weight, eps, (bf16_t*)out, H);
+    else
+        return tff_fail("rmsnorm: unknown dtype %d", dtype);
+    return tff_check_launch("rmsnorm");
+}
+
+// ------------------------------------------------- q/k norm, rotation, kv ---
+// One wave per (token, head).  q and k heads: RMS norm over d with a [d]
+// weight shared by all heads (reference: src/core/model/qwen3/QWen3Creator.cpp:93-101),
+// then the rotation x'_a = x_a cos - x_b sin, x'_b = x_a sin + x_b cos
+// (src/kernel/cuda/paged_flash_attention.cu:343-355) with (cos, sin) from a
+// table indexed by the token's position (src/kernel/cuda/rope_table.cu:32-36).
+// The reference stores k before the rotation and rotates at every read
+// (QWen3Creator.cpp:104-120); storing it rotated once is the same product.
+#define QK_MAX_D 512
+template <typename T, typename TC>
+__global__ void qk_norm_rope_kv_kernel(T* __restrict__ qkv, int nq, int nkv, int d,
+                                       const float* __restrict__ qw, const float* __restrict__ kw,
+                                       float eps, const float* __restrict__ cos_sin, int rot,
+                                       int pairing, const int32_t* __restrict__ positions,
+                                       const int32_t* __restrict__ slot_mapping,
+                                       TC* __restrict__ k_cache, TC* __restrict__ v_cache,
+                                       int page_size) {
+    __shared__ float xs[QK_MAX_D];
+    const int t = blockIdx.x;
+    const int hh = blockIdx.y;
+    const int lane = threadIdx.x;
+    const int width = (nq + 2 * nkv) * d;
+    T* x = qkv + (size_t)t * width + (size_t)hh * d;
+    const int kind = hh < nq ? 0 : (hh < nq + nkv ? 1 : 2);  // q, k, v
+    const int slot = slot_mapping[t];
+    if (kind != 0 && slot < 0) return;
+
+    TC* dst = nullptr;
+    if (kind != 0) {
+        const int head = kind == 1 ? hh - nq : hh - nq - nkv;
+        const int page = slot / page_size, off = slot % page_size;
+        TC* base = kind == 1 ? k_cache : v_cache;
+        dst = base + (((size_t)page * nkv + head) * page_size + off) * d;
+    }
+    if (kind == 2) {
+        for (int e = lane; e < d; e += 64) dst[e] = from_f32<TC>(to_f32(x[e]));
+        return;
+    }
+    const float* w = kind == 0 ? qw : kw;
+    float ss = 0.f;
+    for (int e = lane; e < d; e += 64) {
+        const float v = to_f32(x[e]);
+        xs[e] = v;
+        ss = fmaf(v, v, ss);
+    }
+    ss = wave_sum(ss);
+    __syncthreads();
+    if (w) {
+        const float rr = rsqrtf(ss / (float)d + eps);
+        for (int e = lane; e < d; e += 64) xs[e] = xs[e] * rr * w[e];
+        __syncthreads();
+    }
+    if (cos_sin) {
+        const int pos = positions[t];
+        const int half = rot >> 1;
+        const float* cs = cos_sin + (size_t)pos * rot;  // [pos][pair][cos, sin]
+        for (int p = lane; p < half; p += 64) {
+            const int a = pairing == 0 ? p : 2 * p;
+            const int b = pairing == 0 ? p + half : 2 * p + 1;
+            const float c = cs[2 * p], s = cs[2 * p + 1];
+            const float xa = xs[a], xb = xs[b];
+            xs[a] = xa * c - xb * s;
+            xs[b] = xa * s + xb * c;
+        }
+        __syncthreads();
+    }
+    if (kind == 0) {
+        for (int e = lane; e < d; e += 64) x[e] = from_f32<T>(xs[e]);
+    } else {
+        for (int e = lane; e < d; e += 64) dst[e] = from_f32<TC>(xs[e]);
+    }
+}
+
+TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d, const float* q_weight,
+                                const float* k_weight, float eps, const float* cos_sin,
+                                int rot_dim, int pairing, int max_pos, const int32_t* positions,
+                                const int32_t* slot_mapping, void* k_cache, void* v_cache,
+                                int page_size, int num_pages, int dtype, int cache_dtype,
+                                tff_stream_t stream) {
+    TFF_REQUIRE(qkv && positions && slot_mapping && k_cache && v_cache,
+                "qk_norm_rope_kv: null pointer");
+    TFF_REQUIRE(T >= 0 && nq > 0 && nkv > 0 && page_size > 0 && num_pages > 0,
+                "qk_norm_rope_kv: bad sizes T=%d nq=%d nkv=%d page_size=%d pages=%d", T, nq, nkv,
+                page_size, num_pages);
+    TFF_REQUIRE(d > 0 && d <= QK_MAX_D && d % 2 == 0,
+                "qk_norm_rope_kv: head size %d not supported (even, at most %d)", d, QK_MAX_D);
+    TFF_REQUIRE((q_weight == nullptr) == (k_weight == nullptr),
+                "qk_norm_rope_kv: q and k norm weights must both be given or both be absent");
+    if (cos_sin) {
+        TFF_REQUIRE(rot_dim > 0 && rot_dim <= d && rot_dim % 2 == 0,
+                    "qk_norm_rope_kv: rotary size %d must be even and at most the head size %d",
+                    rot_dim, d);
+        TFF_REQUIRE(pairing == 0 || pairing == 1, "qk_norm_rope_kv: unknown pairing %d", pairing);
+        TFF_REQUIRE(max_pos > 0, "qk_norm_rope_kv: empty rotation table");
+    }
+    TFF_REQUIRE(dtype == cache_dtype, "qk_norm_rope_kv: cache type %d differs from activation type %d",
+                cache_dtype, dtype);
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid(T, nq + 2 * nkv);
+    if (dtype == TFF_F32)
+        qk_norm_rope_kv_kernel<float, float><<<grid, 64, 0, s>>>(
+            (float*)qkv, nq, nkv, d, q_weight, k_weight, eps, cos_sin, rot_dim, pairing, positions,
+            slot_mapping, (float*)k_cache, (float*)v_cache, page_size);
+    else if (dtype == TFF_BF16)
+        qk_norm_rope_kv_kernel<bf16_t, bf16_t><<<grid, 64, 0, s>>>(
+            (bf16_t*)qkv, nq, nkv, d, q_weight, k_weight, eps, cos_sin, rot_dim, pairing, positions,
+            slot_mapping, (bf16_t*)k_cache, (bf16_t*)v_cache, page_size);
+    else
+        return tff_fail("qk_norm_rope_kv: unknown dtype %d", dtype);
+    return tff_check_launch("qk_norm_rope_kv");
+}
+
+// ---------------------------------------------------------------- swiglu ---
+// m = silu(g) * u, silu(x) = x / (1 + exp(-x))  (reference:
+// src/kernel/cuda/unary.cu:10-27, x1 = gate, x2 = up).
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int64_t total, int I) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int64_t t = idx / I;
+    const int i = (int)(idx - t * I);
+    const float g = to_f32(gu[t * 2 * I + i]);
+    const float u = to_f32(gu[t * 2 * I + I + i]);
+    out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+}
+
+TFF_API int tff_swiglu(const void* gu, void* out, int T, int I, int dtype, tff_stream_t stream) {
+    TFF_REQUIRE(gu && out, "swiglu: null pointer");
+    TFF_REQUIRE(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
+    if (T == 0) return 0;
+    const int64_t total = (int64_t)T * I;
+    const int64_t blocks = (total + 255) / 256;
+    TFF_REQUIRE(blocks < 2147483647LL, "swiglu: too many elements");
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TFF_F32)
+        swiglu_kernel<float><<<(unsigned)blocks, 256, 0, s>>>((const float*)gu, (float*)out, total, I);
+    else if (dtype == TFF_BF16)
+        swiglu_kernel<bf16_t><<<(unsigned)blocks, 256, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, total, I);
+    else
+        return tff_fail("swiglu: unknown dtype %d", dtype);
+    return tff_check_launch("swiglu");
+}
+
+// ------------------------------------------------------------------ cast ---
+template <typename TS, typename TD>
+__global__ void cast_kernel(const TS* __restrict__ src, TD* __restrict__ dst, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        dst[i] = from_f32<TD>(to_f32(src[i]));
+}
+
+TFF_API int tff_cast(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n,
+                     tff_stream_t stream) {
+    TFF_REQUIRE(src && dst, "cast: null pointer");
+    TFF_REQUIRE(n >= 0, "cast: negative count");
+    if (n == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (src_dtype == TFF_F32 && dst_dtype == TFF_BF16)
+        cast_kernel<float, bf16_t><<<(unsigned)blocks, 256, 0, s>>>((const float*)src, (bf16_t*)dst, n);
+    else if (src_dtype == TFF_BF16 && dst_dtype == TFF_F32)
+        cast_kernel<bf16_t, float><<<(unsigned)blocks, 256, 0, s>>>((const bf16_t*)src, (float*)dst, n);
+    else if (src_dtype == TFF_F32 && dst_dtype == TFF_F32)
+        cast_kernel<float, float><<<(unsigned)blocks, 256, 0, s>>>((const float*)src, (float*)dst, n);
+    else if (src_dtype == TFF_BF16 && dst_dtype == TFF_BF16)
+        cast_kernel<bf16_t, bf16_t><<<(unsigned)blocks, 256, 0, s>>>((const bf16_t*)src, (bf16_t*)dst, n);
+    else
+        return tff_fail("cast: unknown dtypes %d -> %d", src_dtype, dst_dtype);
+    return tff_check_launch("cast");
+}

@@ -1,0 +1,88 @@
+// C entry points of the gfx950 kernel library.  Every function takes device
+// pointers, checks its arguments on the host, launches on `stream` and returns
+// 0, or a negative code after leaving a message for tff_last_error().
+// Element type codes: 0 = float32, 1 = bfloat16.
+//
+// The export macro plays the part of the reference's DEEP_TFF_API
+// (include/ExportInc.h:6-16).
+#pragma once
+#include <stdint.h>
+
+#define TFF_API extern "C" __attribute__((visibility("default")))
+
+typedef void* tff_stream_t;
+
+TFF_API const char* tff_last_error();
+TFF_API int tff_abi_version();
+
+// out[t, :] = float(table[ids[t], :]).  table [V, H] of `dtype`, out float32.
+TFF_API int tff_embed(const void* table, const int32_t* ids, float* out,
+                      int T, int H, int V, int dtype, tff_stream_t stream);
+
+// Fused residual sum and RMS norm over rows of width H:
+//   v = resid[r] + (delta ? delta[r] : 0);  out[i] = v * rsqrt(mean(v^2)+eps) * w
+// rows == null: r = i for i < n, and resid[r] = v is stored back.
+// rows != null: r = rows[i]; resid is left as it is (norm of gathered rows).
+TFF_API int tff_add_rmsnorm(float* resid, const float* delta, const float* weight,
+                            float eps, void* out, const int32_t* rows, int n, int H,
+                            int out_dtype, tff_stream_t stream);
+
+// RMS norm of a plain [n, H] tensor of `dtype` with a float32 weight.
+TFF_API int tff_rmsnorm(const void* x, const float* weight, float eps, void* out,
+                        int n, int H, int dtype, tff_stream_t stream);
+
+// C[M, N] = A[M, K] . W[N, K]^T.  A has row stride lda (elements), W and C are
+// dense.  A and W are of ab_dtype; C is of c_dtype.  float32 runs on plain FMA
+// in a fixed summation order, bfloat16 on MFMA with float32 accumulation.
+TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K,
+                     int lda, int ab_dtype, int c_dtype, tff_stream_t stream);
+
+// Per (token, head) of a fused projection output qkv [T, (nq + 2 nkv) d]:
+// q and k heads get an RMS norm over d (q_weight / k_weight, skipped if null),
+// then the rotation of pairs by cos_sin[pos, pair] (skipped if null); q is
+// written back in place, k and v go to their page slot slot_mapping[t]
+// (skipped if negative).  pairing 0: pairs (i, i + rot/2); 1: pairs (2i, 2i+1).
+// Cache layout: [pages, nkv, page_size, d].
+TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d,
+                                const float* q_weight, const float* k_weight, float eps,
+                                const float* cos_sin, int rot_dim, int pairing, int max_pos,
+                                const int32_t* positions, const int32_t* slot_mapping,
+                                void* k_cache, void* v_cache, int page_size, int num_pages,
+                                int dtype, int cache_dtype, tff_stream_t stream);
+
+// Attention of every token of a step over its request's cached keys.
+// q: [T, q_stride] with nq heads of d at the start of each row; out [T, nq*d].
+// token_req[t] names the row of block_tables; token t sees keys at positions
+// max(0, pos-window+1) .. pos of that request (window 0: from 0).
+// Works for every head size that is a multiple of 8 up to 512.
+TFF_API int tff_attention_generic(const void* q, int q_stride, void* out,
+                                  const void* k_cache, const void* v_cache,
+                                  const int32_t* block_tables, int bt_stride,
+                                  const int32_t* token_req, const int32_t* positions,
+                                  int T, int nq, int nkv, int d, int page_size, int num_pages,
+                                  int window, float scale, int dtype, int cache_dtype,
+                                  tff_stream_t stream);
+
+// out[t, i] = silu(gu[t, i]) * gu[t, I + i]
+TFF_API int tff_swiglu(const void* gu, void* out, int T, int I, int dtype, tff_stream_t stream);
+
+// Element type conversion of n elements.
+TFF_API int tff_cast(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n,
+                     tff_stream_t stream);
+
+// out[r] = lowest index among the maxima of logits[r, :].
+TFF_API int tff_argmax(const float* logits, int32_t* out, int rows, int V, tff_stream_t stream);
+
+// logits[r, seen] is divided by penalty[r] if positive, multiplied otherwise,
+// for the distinct token ids seen[cu_seen[r] .. cu_seen[r+1]).
+TFF_API int tff_repetition_penalty(float* logits, int rows, int V, const int32_t* seen,
+                                   const int32_t* cu_seen, const float* penalty,
+                                   tff_stream_t stream);
+
+// Draw from softmax(logits / temperature) restricted by top_k (0: off), top_p
+// (1: off) and min_p (0: off), by inverse CDF in index order with the given
+// uniform number per row.  temperature[r] <= 0 selects the argmax.
+TFF_API int tff_sample(const float* logits, int32_t* out, int rows, int V,
+                       const float* temperature, const int32_t* top_k, const float* top_p,
+                       const float* min_p, const float* uniform, float* probs_out,
+                       tff_stream_t stream);

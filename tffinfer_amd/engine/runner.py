@@ -1,0 +1,142 @@
+"""The step function: runs a batch of (request, its next tokens) through the
+model from the cache and returns the logits at the wanted places.
+
+It replaces the reference's ``prefill()`` + the body of ``decode()``'s loop +
+``update_kv_cache`` (src/core/runtime/InferRuntime.cu:294-323, :348-375,
+:523-529) and its kernel-launch task graph (src/core/runtime/TaskFlowManager.cu:15-56)
+by straight-line code on one stream.  A step runs only the tokens it is given;
+everything earlier comes from the cache.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..cache.block_pool import OutOfPages
+from ..cache.manager import CacheManager
+from ..kernels import ops as _ops
+from .batch import KVView, StepBatch, StepEntry, build_step_batch
+
+
+class StepError(ValueError):
+    """A batch the step function cannot run as given."""
+
+
+class LayerContext:
+    """What a part sees during one layer call of one step."""
+    __slots__ = ("ops", "act_dtype", "batch", "max_positions", "kv", "state", "call_index")
+
+    def __init__(self, ops, act_dtype, batch, max_positions):
+        self.ops = ops
+        self.act_dtype = act_dtype
+        self.batch = batch
+        self.max_positions = max_positions
+        self.kv = None
+        self.state = None
+        self.call_index = -1
+
+
+class StepContext(LayerContext):
+    __slots__ = ("_calls", "_cache")
+
+    def __init__(self, ops, act_dtype, batch, max_positions, calls, cache):
+        super().__init__(ops, act_dtype, batch, max_positions)
+        self._calls = calls
+        self._cache = cache
+
+    def for_call(self, idx: int) -> LayerContext:
+        c = LayerContext(self.ops, self.act_dtype, self.batch, self.max_positions)
+        c.call_index = idx
+        cache_id, writes, group, k, v, state = self._calls[idx]
+        if group is not None:
+            gt = self.batch.groups[group]
+            c.kv = KVView(k, v, gt.block_tables, gt.slot_mapping if writes else gt.no_slot_mapping,
+                          self._cache.page_size, group)
+        c.state = state
+        return c
+
+
+class ModelRunner:
+    def __init__(self, model, page_size: int = 16, num_pages=256, max_seqs: int = 8,
+                 max_model_len: int | None = None, ops=_ops):
+        if model.device is None or model.device.type != "cuda":
+            raise StepError("the model has no weights on a GPU; there is no CPU path")
+        self.model = model
+        self.ops = ops
+        self.device = model.device
+        self.act_dtype = model.dtype
+        cfg = model.config
+        self.max_model_len = min(int(max_model_len or cfg.max_position_embeddings),
+                                 cfg.max_position_embeddings)
+        self.vocab_size = cfg.vocab_size
+        reqs = model.call_requirements()
+        self.cache = CacheManager(reqs, page_size, num_pages, max_seqs, dtype=self.act_dtype,
+                                  device=self.device)
+        self._calls = []
+        for cache_id, writes, kv_spec, state_spec in reqs:
+            group = self.cache.group_index(cache_id) if kv_spec is not None else None
+            k = v = None
+            if group is not None:
+                k, v = self.cache.kv_tensors(cache_id)
+            self._calls.append((cache_id, writes, group, k, v, self.cache.state_tensors.get(cache_id)))
+
+    # ---- requests --------------------------------------------------------
+    def add_request(self, req) -> int:
+        return self.cache.add_request(req)
+
+    def free_request(self, req) -> None:
+        self.cache.release(req)
+
+    def has_request(self, req) -> bool:
+        return self.cache.has_request(req)
+
+    # ---- the step --------------------------------------------------------
+    def _validate(self, entries) -> None:
+        seen = set()
+        for e in entries:
+            if not self.cache.has_request(e.req):
+                raise StepError(f"request {e.req!r} is not live (add_request first)")
+            if e.req in seen:
+                raise StepError(f"request {e.req!r} appears twice in one step")
+            seen.add(e.req)
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"request {e.req!r} brings no tokens")
+            for t in e.tokens:
+                if not isinstance(t, int) or not 0 <= t < self.vocab_size:
+                    raise StepError(f"request {e.req!r}: token id {t!r} is outside the vocabulary "
+                                    f"of {self.vocab_size}")
+            for w in e.want:
+                if not isinstance(w, int) or not 0 <= w < n:
+                    raise StepError(f"request {e.req!r}: wanted place {w!r} is not among its {n} tokens")
+            end = self.cache.num_tokens(e.req) + n
+            if end > self.max_model_len:
+                raise StepError(f"request {e.req!r} would reach {end} tokens, the limit is {self.max_model_len}")
+
+    def reserve(self, entries) -> None:
+        """Takes the pages the step's new tokens need, for all entries or none."""
+        free = [g.pool.num_free for g in self.cache.groups]
+        for e in entries:
+            need = self.cache.pages_needed(e.req, len(e.tokens))
+            for i, n in enumerate(need):
+                free[i] -= n
+        if any(f < 0 for f in free):
+            short = [-f for f in free if f < 0]
+            raise OutOfPages(f"the step needs {max(short)} more pages than the pool has free")
+        for e in entries:
+            self.cache.reserve(e.req, len(e.tokens))
+
+    @torch.no_grad()
+    def step(self, entries: list[StepEntry]) -> torch.Tensor:
+        """Logits (float32 [wanted, vocab], on the device) at the wanted places,
+        in the order of the entries and of their ``want``."""
+        if not entries:
+            return torch.empty(0, self.vocab_size, dtype=torch.float32, device=self.device)
+        self._validate(entries)
+        self.reserve(entries)
+        with torch.cuda.device(self.device):
+            batch = build_step_batch(entries, self.cache, self.device)
+            ctx = StepContext(self.ops, self.act_dtype, batch, self.max_model_len, self._calls, self.cache)
+            logits = self.model.forward(ctx)
+        for e in entries:
+            self.cache.commit(e.req, len(e.tokens))
+        return logits

@@ -1,0 +1,159 @@
+"""Builds the gfx950 kernel library from ``csrc/*.hip`` with hipcc.
+
+The library is one shared object with C entry points, kept in the tree under
+``tffinfer_amd/lib`` (or, if the tree cannot be written, under the temporary
+folder).  ``ensure_built`` builds only when there is no library for the present
+sources; ``build`` always compiles.
+"""
+from __future__ import annotations
+
+import hashlib
+import json
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from concurrent.futures import ThreadPoolExecutor
+
+PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC_DIR = os.path.join(PKG_DIR, "csrc")
+LIB_NAME = "libtffinfer_hip.so"
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-fvisibility=hidden",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+class BuildError(RuntimeError):
+    pass
+
+
+def _sources() -> list[str]:
+    return sorted(
+        os.path.join(CSRC_DIR, f) for f in os.listdir(CSRC_DIR) if f.endswith(".hip")
+    )
+
+
+def _headers() -> list[str]:
+    return sorted(os.path.join(CSRC_DIR, f) for f in os.listdir(CSRC_DIR) if f.endswith(".h"))
+
+
+def source_digest() -> str:
+    h = hashlib.sha256()
+    for path in _sources() + _headers():
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(HIPCC_FLAGS).encode())
+    return h.hexdigest()[:16]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise BuildError("hipcc was not found (looked at $HIPCC, PATH and /opt/rocm/bin)")
+
+
+def _writable(d: str) -> bool:
+    try:
+        os.makedirs(d, exist_ok=True)
+        probe = os.path.join(d, f".probe_{os.getpid()}")
+        with open(probe, "w"):
+            pass
+        os.remove(probe)
+        return True
+    except OSError:
+        return False
+
+
+def lib_dirs() -> list[str]:
+    """Folders a library may live in, in order of preference."""
+    fallback = os.path.join(tempfile.gettempdir(), f"tffinfer_amd_{os.getuid()}")
+    return [os.path.join(PKG_DIR, "lib"), fallback]
+
+
+def find_library() -> str | None:
+    """Path of a library built from the present sources, or None."""
+    digest = source_digest()
+    for d in lib_dirs():
+        info = os.path.join(d, "build_info.json")
+        lib = os.path.join(d, LIB_NAME)
+        if os.path.exists(lib) and os.path.exists(info):
+            try:
+                with open(info) as f:
+                    if json.load(f).get("digest") == digest:
+                        return lib
+            except (OSError, ValueError):
+                pass
+    return None
+
+
+def build(verbose: bool = True) -> str:
+    """Compiles every source for gfx950 and links the library; returns its path."""
+    hipcc = _hipcc()
+    out_dir = next((d for d in lib_dirs() if _writable(d)), None)
+    if out_dir is None:
+        raise BuildError("no writable folder for the kernel library: " + ", ".join(lib_dirs()))
+    obj_dir = os.path.join(out_dir, "obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    sources = _sources()
+    t0 = time.time()
+    done = threading.Event()
+
+    def say(msg):
+        if verbose:
+            print(f"[tffinfer_amd build] {msg}", file=sys.stderr, flush=True)
+
+    def ticker():
+        while not done.wait(10.0):
+            say(f"still compiling ... {time.time() - t0:.0f} s")
+
+    def compile_one(src):
+        obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
+        cmd = [hipcc, *HIPCC_FLAGS, "-I", CSRC_DIR, "-c", src, "-o", obj]
+        p = subprocess.run(cmd, capture_output=True, text=True)
+        if p.returncode != 0:
+            raise BuildError(f"hipcc failed on {os.path.basename(src)}:\n{p.stderr[-4000:]}")
+        say(f"compiled {os.path.basename(src)} ({time.time() - t0:.0f} s)")
+        return obj
+
+    say(f"compiling {len(sources)} files for gfx950 into {out_dir}")
+    th = threading.Thread(target=ticker, daemon=True)
+    th.start()
+    try:
+        workers = max(1, min(len(sources), int(os.environ.get("MAX_JOBS", "8")), 16))
+        with ThreadPoolExecutor(workers) as pool:
+            objs = list(pool.map(compile_one, sources))
+        tmp_lib = os.path.join(out_dir, f".{LIB_NAME}.{os.getpid()}")
+        cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp_lib]
+        p = subprocess.run(cmd, capture_output=True, text=True)
+        if p.returncode != 0:
+            raise BuildError(f"link failed:\n{p.stderr[-4000:]}")
+        os.replace(tmp_lib, os.path.join(out_dir, LIB_NAME))
+        with open(os.path.join(out_dir, "build_info.json"), "w") as f:
+            json.dump({"digest": source_digest(), "flags": HIPCC_FLAGS}, f)
+    finally:
+        done.set()
+    say(f"built {LIB_NAME} in {time.time() - t0:.0f} s")
+    return os.path.join(out_dir, LIB_NAME)
+
+
+def ensure_built(verbose: bool = True) -> str:
+    lib = find_library()
+    if lib is None:
+        lib = build(verbose=verbose)
+    return lib
+
+
+if __name__ == "__main__":
+    print(build())

@@ -1,0 +1,308 @@
+"""The op table: every operation of the engine bound to exactly one HIP kernel.
+
+Each function checks on the host that its operands have the device, element
+type, contiguity and shape the kernel assumes (a kernel is never launched on
+operands it cannot address), allocates the result with torch's allocator and
+launches on torch's current stream.  There is no CPU path and no library
+fallback: without the compiled library every call raises.
+
+The reference binds ops to kernels by name in its FunctionFactory
+(include/FunctionFactory.h:18-116, kernel/include/TFFOPCreatorBase.h:73-97)
+with a device dispatch; here the table has one entry per op and no dispatch.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import lib as _lib
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DT[dt]
+    except KeyError:
+        raise _lib.KernelError(f"element type {dt} is not supported (float32 or bfloat16)") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _req(t: torch.Tensor, name: str, dtype=None, ndim=None):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise _lib.KernelError(f"{name}: expected a tensor on the GPU")
+    if not t.is_contiguous():
+        raise _lib.KernelError(f"{name}: tensor is not contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise _lib.KernelError(f"{name}: expected {dtype}, got {t.dtype}")
+    if ndim is not None and t.dim() != ndim:
+        raise _lib.KernelError(f"{name}: expected {ndim} dimensions, got shape {tuple(t.shape)}")
+    return t
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Rows of ``table`` [V, H] for int32 ``ids`` [T] as float32 [T, H]."""
+    _req(table, "embed table", ndim=2)
+    _req(ids, "embed ids", torch.int32, 1)
+    V, H = table.shape
+    T = ids.numel()
+    if out is None:
+        out = torch.empty(T, H, dtype=torch.float32, device=table.device)
+    else:
+        _req(out, "embed out", torch.float32, 2)
+        if tuple(out.shape) != (T, H):
+            raise _lib.KernelError(f"embed out: shape {tuple(out.shape)} is not {(T, H)}")
+    L = _lib.load()
+    _lib.check(L.tff_embed(table.data_ptr(), ids.data_ptr(), out.data_ptr(), T, H, V,
+                           dtype_code(table.dtype), _stream()))
+    return out
+
+
+def add_rmsnorm(resid: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, rows: torch.Tensor | None = None,
+                out: torch.Tensor | None = None) -> torch.Tensor:
+    """``resid += delta`` (when given and ``rows`` is None) and the RMS norm of
+    the sum; with ``rows`` the norm of those rows only, ``resid`` untouched."""
+    _req(resid, "add_rmsnorm resid", torch.float32, 2)
+    H = resid.shape[1]
+    _req(weight, "add_rmsnorm weight", torch.float32, 1)
+    if weight.numel() != H:
+        raise _lib.KernelError(f"add_rmsnorm: weight has {weight.numel()} elements, rows have {H}")
+    if delta is not None:
+        _req(delta, "add_rmsnorm delta", torch.float32, 2)
+        if delta.shape != resid.shape:
+            raise _lib.KernelError(
+                f"add_rmsnorm: delta {tuple(delta.shape)} does not match resid {tuple(resid.shape)}")
+    if rows is not None:
+        _req(rows, "add_rmsnorm rows", torch.int32, 1)
+        n = rows.numel()
+    else:
+        n = resid.shape[0]
+    if out is None:
+        out = torch.empty(n, H, dtype=out_dtype, device=resid.device)
+    else:
+        _req(out, "add_rmsnorm out", out_dtype, 2)
+        if tuple(out.shape) != (n, H):
+            raise _lib.KernelError(f"add_rmsnorm out: shape {tuple(out.shape)} is not {(n, H)}")
+    L = _lib.load()
+    _lib.check(L.tff_add_rmsnorm(resid.data_ptr(), _ptr(delta), weight.data_ptr(), float(eps),
+                                 out.data_ptr(), _ptr(rows), n, H, dtype_code(out_dtype), _stream()))
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """RMS norm over the last dimension of a dense tensor, float32 weight."""
+    _req(x, "rmsnorm x")
+    H = x.shape[-1]
+    _req(weight, "rmsnorm weight", torch.float32, 1)
+    if weight.numel() != H:
+        raise _lib.KernelError(f"rmsnorm: weight has {weight.numel()} elements, rows have {H}")
+    out = torch.empty_like(x)
+    L = _lib.load()
+    _lib.check(L.tff_rmsnorm(x.data_ptr(), weight.data_ptr(), float(eps), out.data_ptr(),
+                             x.numel() // H, H, dtype_code(x.dtype), _stream()))
+    return out
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None = None,
+           out: torch.Tensor | None = None) -> torch.Tensor:
+    """``x . weight^T`` for x [M, K] (rows may be strided) and weight [N, K]."""
+    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
+        raise _lib.KernelError("linear x: expected a GPU matrix with unit inner stride")
+    _req(weight, "linear weight", x.dtype, 2)
+    M, K = x.shape
+    N, K2 = weight.shape
+    if K != K2:
+        raise _lib.KernelError(f"linear: x has inner size {K}, weight [out, in] = {tuple(weight.shape)}")
+    lda = x.stride(0) if M > 1 else K
+    if lda < K:
+        raise _lib.KernelError("linear x: rows overlap")
+    out_dtype = out_dtype or x.dtype
+    if out is None:
+        out = torch.empty(M, N, dtype=out_dtype, device=x.device)
+    else:
+        _req(out, "linear out", out_dtype, 2)
+        if tuple(out.shape) != (M, N):
+            raise _lib.KernelError(f"linear out: shape {tuple(out.shape)} is not {(M, N)}")
+    L = _lib.load()
+    _lib.check(L.tff_gemm(x.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K, lda,
+                          dtype_code(x.dtype), dtype_code(out_dtype), _stream()))
+    return out
+
+
+def qk_norm_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int,
+                    q_weight: torch.Tensor | None, k_weight: torch.Tensor | None, eps: float,
+                    cos_sin: torch.Tensor | None, pairing: int,
+                    positions: torch.Tensor, slot_mapping: torch.Tensor,
+                    k_cache: torch.Tensor, v_cache: torch.Tensor) -> None:
+    """In place on the fused projection output ``qkv`` [T, (nq + 2 nkv) d]; see
+    the entry point's comment.  ``cos_sin`` is [max_pos, rot/2, 2] float32."""
+    _req(qkv, "qk_norm_rope_kv qkv", ndim=2)
+    T = qkv.shape[0]
+    if qkv.shape[1] != (nq + 2 * nkv) * d:
+        raise _lib.KernelError(
+            f"qk_norm_rope_kv: rows of {qkv.shape[1]} are not (nq + 2 nkv) d = {(nq + 2 * nkv) * d}")
+    for w, nm in ((q_weight, "q norm weight"), (k_weight, "k norm weight")):
+        if w is not None:
+            _req(w, nm, torch.float32, 1)
+            if w.numel() != d:
+                raise _lib.KernelError(f"{nm}: {w.numel()} elements, head size {d}")
+    rot, max_pos = 0, 0
+    if cos_sin is not None:
+        _req(cos_sin, "rotation table", torch.float32, 3)
+        max_pos, half, two = cos_sin.shape
+        if two != 2:
+            raise _lib.KernelError("rotation table: last dimension must hold (cos, sin)")
+        rot = 2 * half
+    _req(positions, "positions", torch.int32, 1)
+    _req(slot_mapping, "slot_mapping", torch.int32, 1)
+    if positions.numel() != T or slot_mapping.numel() != T:
+        raise _lib.KernelError("qk_norm_rope_kv: positions and slot_mapping need one entry per token")
+    _req(k_cache, "k cache", ndim=4)
+    _req(v_cache, "v cache", ndim=4)
+    if k_cache.shape != v_cache.shape or k_cache.shape[1] != nkv or k_cache.shape[3] != d:
+        raise _lib.KernelError(
+            f"qk_norm_rope_kv: cache {tuple(k_cache.shape)} is not [pages, {nkv}, page_size, {d}]")
+    L = _lib.load()
+    _lib.check(L.tff_qk_norm_rope_kv(
+        qkv.data_ptr(), T, nq, nkv, d, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin),
+        rot, int(pairing), max_pos, positions.data_ptr(), slot_mapping.data_ptr(),
+        k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[2], k_cache.shape[0],
+        dtype_code(qkv.dtype), dtype_code(k_cache.dtype), _stream()))
+
+
+def attention_generic(q: torch.Tensor, nq: int, nkv: int, d: int, k_cache: torch.Tensor,
+                      v_cache: torch.Tensor, block_tables: torch.Tensor, token_req: torch.Tensor,
+                      positions: torch.Tensor, window: int = 0, scale: float | None = None,
+                      out: torch.Tensor | None = None) -> torch.Tensor:
+    """Attention of each token over its request's pages; q is [T, >= nq*d]
+    with the query heads at the start of each row.  Returns [T, nq*d]."""
+    _req(q, "attention q", ndim=2)
+    T = q.shape[0]
+    if q.shape[1] < nq * d:
+        raise _lib.KernelError(f"attention q: rows of {q.shape[1]} hold fewer than nq*d = {nq * d}")
+    _req(k_cache, "k cache", q.dtype, 4)
+    _req(v_cache, "v cache", q.dtype, 4)
+    if k_cache.shape != v_cache.shape or k_cache.shape[1] != nkv or k_cache.shape[3] != d:
+        raise _lib.KernelError(
+            f"attention: cache {tuple(k_cache.shape)} is not [pages, {nkv}, page_size, {d}]")
+    _req(block_tables, "block tables", torch.int32, 2)
+    _req(token_req, "token_req", torch.int32, 1)
+    _req(positions, "positions", torch.int32, 1)
+    if token_req.numel() != T or positions.numel() != T:
+        raise _lib.KernelError("attention: token_req and positions need one entry per token")
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    if out is None:
+        out = torch.empty(T, nq * d, dtype=q.dtype, device=q.device)
+    L = _lib.load()
+    _lib.check(L.tff_attention_generic(
+        q.data_ptr(), q.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+        block_tables.data_ptr(), block_tables.stride(0), token_req.data_ptr(), positions.data_ptr(),
+        T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale),
+        dtype_code(q.dtype), dtype_code(k_cache.dtype), _stream()))
+    return out
+
+
+def paged_attention(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,
+                    scale: float | None = None) -> torch.Tensor:
+    """Attention of a step's tokens over the cache view ``kv`` (k_cache,
+    v_cache, block_tables) with the step's ``batch`` (token_req, positions).
+    Picks the kernel for the element type and the shape of the step."""
+    return attention_generic(q, nq, nkv, d, kv.k_cache, kv.v_cache, kv.block_tables,
+                             batch.token_req, batch.positions, window, scale)
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``silu(gate) * up`` for gate_up [T, 2I] = [gate | up]."""
+    _req(gate_up, "swiglu input", ndim=2)
+    T, two_i = gate_up.shape
+    if two_i % 2:
+        raise _lib.KernelError("swiglu: odd row width")
+    I = two_i // 2
+    if out is None:
+        out = torch.empty(T, I, dtype=gate_up.dtype, device=gate_up.device)
+    L = _lib.load()
+    _lib.check(L.tff_swiglu(gate_up.data_ptr(), out.data_ptr(), T, I, dtype_code(gate_up.dtype), _stream()))
+    return out
+
+
+def cast(src: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    _req(src, "cast src")
+    out = torch.empty(src.shape, dtype=dtype, device=src.device)
+    L = _lib.load()
+    _lib.check(L.tff_cast(src.data_ptr(), dtype_code(src.dtype), out.data_ptr(), dtype_code(dtype),
+                          src.numel(), _stream()))
+    return out
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """Lowest index among the maxima of each row of float32 logits [R, V]."""
+    _req(logits, "argmax logits", torch.float32, 2)
+    R, V = logits.shape
+    out = torch.empty(R, dtype=torch.int32, device=logits.device)
+    L = _lib.load()
+    _lib.check(L.tff_argmax(logits.data_ptr(), out.data_ptr(), R, V, _stream()))
+    return out
+
+
+def repetition_penalty(logits: torch.Tensor, seen: torch.Tensor, cu_seen: torch.Tensor,
+                       penalty: torch.Tensor) -> None:
+    _req(logits, "repetition_penalty logits", torch.float32, 2)
+    R, V = logits.shape
+    _req(seen, "seen", torch.int32, 1)
+    _req(cu_seen, "cu_seen", torch.int32, 1)
+    _req(penalty, "penalty", torch.float32, 1)
+    if cu_seen.numel() != R + 1 or penalty.numel() != R:
+        raise _lib.KernelError("repetition_penalty: cu_seen needs rows + 1 entries, penalty one per row")
+    L = _lib.load()
+    _lib.check(L.tff_repetition_penalty(logits.data_ptr(), R, V, seen.data_ptr(), cu_seen.data_ptr(),
+                                        penalty.data_ptr(), _stream()))
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,
+           top_k: torch.Tensor | None = None, top_p: torch.Tensor | None = None,
+           min_p: torch.Tensor | None = None, return_probs: bool = False):
+    """One token per row of float32 logits [R, V]; see the entry point."""
+    _req(logits, "sample logits", torch.float32, 2)
+    R, V = logits.shape
+    _req(temperature, "temperature", torch.float32, 1)
+    _req(uniform, "uniform", torch.float32, 1)
+    for t, nm, dt in ((top_k, "top_k", torch.int32), (top_p, "top_p", torch.float32),
+                      (min_p, "min_p", torch.float32)):
+        if t is not None:
+            _req(t, nm, dt, 1)
+            if t.numel() != R:
+                raise _lib.KernelError(f"sample: {nm} needs one entry per row")
+    if temperature.numel() != R or uniform.numel() != R:
+        raise _lib.KernelError("sample: temperature and uniform need one entry per row")
+    out = torch.empty(R, dtype=torch.int32, device=logits.device)
+    probs = torch.empty(R, V, dtype=torch.float32, device=logits.device) if return_probs else None
+    L = _lib.load()
+    _lib.check(L.tff_sample(logits.data_ptr(), out.data_ptr(), R, V, temperature.data_ptr(),
+                            _ptr(top_k), _ptr(top_p), _ptr(min_p), uniform.data_ptr(), _ptr(probs),
+                            _stream()))
+    return (out, probs) if return_probs else out
+
+
+OP_TABLE = {
+    "embed": embed,
+    "add_rmsnorm": add_rmsnorm,
+    "rmsnorm": rmsnorm,
+    "linear": linear,
+    "qk_norm_rope_kv": qk_norm_rope_kv,
+    "attention": attention_generic,
+    "swiglu": swiglu,
+    "cast": cast,
+    "argmax": argmax,
+    "repetition_penalty": repetition_penalty,
+    "sample": sample,
+}

@@ -1,0 +1,131 @@
+"""The model skeleton every decoder architecture shares: embedding, a list of
+blocks run in the order the configuration gives, final norm, output head.
+
+What a layer is made of and in which order layers run is data from the typed
+configuration (``layer_specs``, ``layer_schedule``); this file holds no size
+and no constant of any architecture.  The reference wires the same sequence as
+graph nodes in src/core/model/qwen3/QWen3Creator.cpp:43-165.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+from ..config.base import ModelConfig
+from ..parts.base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Part, WeightSpec
+from ..parts.embedding import Embedding, OutputHead
+from ..weights.loader import check_weights, normalize_stored
+from ..weights.random_init import random_tensor
+
+
+@dataclass
+class TensorNames:
+    """How an architecture's files name the tensors of the skeleton's parts."""
+    embedding: str = "model.embed_tokens"
+    layer: str = "model.layers.{i}"
+    final_norm: str = "model.norm"
+    head: str = "lm_head"
+    #: the block's children by the name the files use
+    children: dict = field(default_factory=dict)
+    #: tensors a file may hold that the model has no use for
+    ignorable: tuple = ()
+
+
+def _leaves(prefix: str, part: Part, rename: dict):
+    """(global name prefix, part) for a part and all its sub-parts."""
+    yield prefix, part
+    for child_name, child in part.children().items():
+        yield from _leaves(f"{prefix}.{rename.get(child_name, child_name)}", child, rename)
+
+
+class DecoderModel:
+    def __init__(self, config: ModelConfig, names: TensorNames):
+        self.config = config
+        self.names = names
+        self.dtype = None
+        self.device = None
+        H, V = config.hidden_size, config.vocab_size
+        self.embedding = Embedding(V, H)
+        self.blocks = []
+        for spec in config.layer_specs():
+            mixer = MIXERS.build(spec.mixer)
+            ffn = FEED_FORWARDS.build(spec.feed_forward)
+            norm_spec = spec.norm
+            block = BLOCKS.build(spec.block, mixer=mixer, feed_forward=ffn,
+                                 make_norm=lambda s=norm_spec: NORMS.build(s))
+            self.blocks.append(block)
+        self.schedule = list(config.layer_schedule())
+        for call in self.schedule:
+            if not 0 <= call.layer < len(self.blocks):
+                raise ValueError(f"layer schedule names layer {call.layer}, the model has {len(self.blocks)}")
+        self.final_norm = NORMS.build(config.final_norm_spec())
+        self.head = OutputHead(V, H, self.embedding if config.tie_word_embeddings else None)
+
+    # ---- weights ---------------------------------------------------------
+    def _weighted_parts(self):
+        yield self.names.embedding, self.embedding
+        for i, block in enumerate(self.blocks):
+            yield from _leaves(self.names.layer.format(i=i), block, self.names.children)
+        yield self.names.final_norm, self.final_norm
+        yield self.names.head, self.head
+
+    def expected_tensors(self) -> dict[str, WeightSpec]:
+        out = {}
+        for prefix, part in self._weighted_parts():
+            for local, spec in part.weight_specs().items():
+                out[f"{prefix}.{local}"] = spec
+        return out
+
+    def load_tensors(self, found: dict[str, torch.Tensor], dtype: torch.dtype, device,
+                     where: str = "") -> None:
+        """Checks ``found`` against what the parts expect (one error for all
+        that is wrong) and hands every part its tensors."""
+        ignorable = set(self.names.ignorable)
+        if self.config.tie_word_embeddings:
+            ignorable.add(f"{self.names.head}.weight")  # a stored copy of the tied head is not used
+        check_weights(self.expected_tensors(), found, ignorable, where)
+        self.dtype, self.device = dtype, torch.device(device)
+        for prefix, part in self._weighted_parts():
+            specs = part.weight_specs()
+            if specs:
+                part.load_weights({local: normalize_stored(found[f"{prefix}.{local}"]) for local in specs},
+                                  dtype, self.device)
+
+    def init_random(self, seed: int, dtype: torch.dtype, device, on_device: bool = False) -> None:
+        """Seeded random weights without a file.  ``on_device`` draws on the GPU
+        (another stream of numbers than the host's, for large models)."""
+        self.dtype, self.device = dtype, torch.device(device)
+        gen_dev = self.device if on_device else "cpu"
+        for prefix, part in self._weighted_parts():
+            specs = part.weight_specs()
+            if specs:
+                ws = {}
+                for local, spec in specs.items():
+                    t = random_tensor(spec, seed, f"{prefix}.{local}", device=gen_dev)
+                    ws[local] = t if spec.init == "norm" else t.to(torch.bfloat16)
+                part.load_weights(ws, dtype, self.device)
+
+    # ---- cache needs -----------------------------------------------------
+    def call_requirements(self):
+        """For every entry of the run order: (cache id, writes, KVCacheSpec or
+        None, StateSpec or None)."""
+        out = []
+        for call in self.schedule:
+            mixer = self.blocks[call.layer].mixer
+            out.append((call.cache, call.writes_cache, mixer.cache_spec(), mixer.state_spec()))
+        return out
+
+    # ---- one step --------------------------------------------------------
+    def forward(self, ctx) -> torch.Tensor:
+        """Runs the tokens of ``ctx.batch`` and returns float32 logits
+        [len(logit_rows), vocab]."""
+        b = ctx.batch
+        resid = self.embedding.forward(ctx, b.token_ids)
+        pending = None
+        for idx, call in enumerate(self.schedule):
+            pending = self.blocks[call.layer].forward(ctx.for_call(idx), resid, pending)
+        if b.num_logit_rows == 0:
+            return torch.empty(0, self.config.vocab_size, dtype=torch.float32, device=resid.device)
+        y = self.final_norm.forward(ctx, resid, pending, rows=b.logit_rows)
+        return self.head.forward(ctx, y)
