@@ -1,0 +1,143 @@
+"""Generation through the entry points against the plain implementation."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from helpers import TOL, oracle_logits, random_tokens, read_config, rel_err
+from plain_qwen3 import plain_greedy, plain_inverse_cdf, plain_probs
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def plain_generate_greedy(model_dir, prompt, n):
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(plain_greedy(oracle_logits(model_dir, toks)[-1]))
+    return toks[len(prompt):]
+
+
+def check_choices(model_dir, result, dtype, sampling=None):
+    """Every kept logits row matches the plain logits of the engine's own
+    sequence at that place, and the chosen token is what the plain sampler
+    picks from that row."""
+    from tffinfer_amd.sampling import uniform_at
+    seq = result.prompt + result.output
+    ref = oracle_logits(model_dir, seq)
+    assert len(result.logits) == len(result.output)
+    for i, (row, tok) in enumerate(zip(result.logits, result.output)):
+        pos = len(result.prompt) + i - 1
+        assert rel_err(row, ref[pos]) <= TOL[dtype], f"output {i}"
+        if sampling is None or sampling.greedy:
+            assert tok == plain_greedy(row)
+        else:
+            t, k, p, m = sampling.effective()
+            assert tok == plain_inverse_cdf(plain_probs(row, t, k, p, m), uniform_at(sampling.seed, i))
+
+
+def test_greedy_through_the_reference_style_entry_point_fp32(model_dirs):
+    from tffinfer_amd import LLMInferRuntime, ModelConfig
+    d = model_dirs["A"]
+    V = read_config(d)["vocab_size"]
+    prompts = [random_tokens(n, V, 50 + n) for n in (1, 9, 40)]
+    cfg = ModelConfig()
+    cfg._use_f16 = False
+    cfg._n_ctx = 128
+    rt = LLMInferRuntime()
+    assert rt.load_model([d], cfg) and rt.init_runtime_context()
+    assert rt.encode(prompts) == 50
+    out = []
+    assert rt.infer(16, out)
+    assert out == [plain_generate_greedy(d, p, 16) for p in prompts]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_engine(model_dirs, dtype):
+    from tffinfer_amd import EngineOptions, LLMEngine
+    d = model_dirs["A"]
+    V = read_config(d)["vocab_size"]
+    prompts = [random_tokens(n, V, 60 + n) for n in (1, 9, 40)]
+    eng = LLMEngine.from_model_dir(d, EngineOptions(dtype=dtype, page_size=16, kv_tokens=256, max_num_seqs=4))
+    eng.keep_logits = True
+    res = eng.generate(prompts, max_new_tokens=16, ignore_eos=True)
+    for r in res:
+        assert len(r.output) == 16 and r.finish_reason == "length"
+        check_choices(d, r, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_chunked_prefill_mixed_with_decode_temperature_small_pool(model_dirs, dtype):
+    """Tiny B's workload: 5 requests, portions of 24 tokens beside decoding,
+    24 tokens at temperature 0.8 with a fixed seed, on a pool so small that
+    requests are preempted and computed again."""
+    from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
+    d = model_dirs["B"]
+    V = read_config(d)["vocab_size"]
+    prompts = [random_tokens(n, V, 70 + n) for n in (3, 17, 31, 64, 100)]
+    sc = [SamplingConfig("random", temperature=0.8, seed=100 + i) for i in range(5)]
+    opt = EngineOptions(dtype=dtype, page_size=8, num_pages=20, max_num_seqs=4, max_num_batched_tokens=48,
+                        prefill_chunk=24)
+    eng = LLMEngine.from_model_dir(d, opt)
+    eng.keep_logits = True
+    res = eng.generate(prompts, sc, max_new_tokens=24, ignore_eos=True)
+    assert eng.scheduler.stats.preemptions > 0, "the pool was meant to run out"
+    for r, s in zip(res, sc):
+        assert len(r.output) == 24
+        # logits kept before a preemption stay valid: the recomputation feeds the same tokens
+        r.logits = r.logits[:len(r.output)]
+        check_choices(d, r, dtype, s)
+    assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
+    if dtype == "float32":
+        # each request alone gives the same tokens as in the crowd
+        for p, s, r in zip(prompts, sc, res):
+            alone = LLMEngine(eng.model, EngineOptions(dtype=dtype, page_size=8, num_pages=40, max_num_seqs=1))
+            assert alone.generate([p], s, max_new_tokens=24, ignore_eos=True)[0].output == r.output
+
+
+def test_sampling_filters_and_penalty_through_engine(model_dirs):
+    from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
+    d = model_dirs["A"]
+    prompts = [[5, 6, 7, 8], [9, 10]]
+    sc = [SamplingConfig("top_k", 0.9, top_k=7, top_p=0.9, seed=4), SamplingConfig("top_p", 1.2, top_p=0.6, min_p=0.01, seed=5)]
+    eng = LLMEngine.from_model_dir(d, EngineOptions(dtype="float32", kv_tokens=128, max_num_seqs=2))
+    eng.keep_logits = True
+    res = eng.generate(prompts, sc, max_new_tokens=12, ignore_eos=True)
+    for r, s in zip(res, sc):
+        check_choices(d, r, "float32", s)
+    # repetition penalty: the kept rows are the logits before the penalty
+    from plain_qwen3 import plain_repetition_penalty
+    r = eng.generate([[1, 2, 3]], SamplingConfig("greedy", repetition_penalty=5.0), max_new_tokens=20,
+                     ignore_eos=True)[0]
+    for i, (row, tok) in enumerate(zip(r.logits, r.output)):
+        seen = r.prompt + r.output[:i]
+        assert tok == plain_greedy(plain_repetition_penalty(row, seen, 5.0))
+    plain = eng.generate([[1, 2, 3]], SamplingConfig("greedy"), max_new_tokens=20, ignore_eos=True)[0].output
+    assert plain != r.output, "a penalty of 5 was expected to change a tiny model's greedy loop"
+
+
+def test_eos_stops(model_dirs):
+    from tffinfer_amd import EngineOptions, LLMEngine
+    d = model_dirs["A"]
+    eng = LLMEngine.from_model_dir(d, EngineOptions(dtype="float32", kv_tokens=128, max_num_seqs=2))
+    full = eng.generate([[3, 4, 5]], max_new_tokens=10, ignore_eos=True)[0].output
+    stop = eng.generate([[3, 4, 5]], max_new_tokens=10, eos_token_id=full[4])[0]
+    cut = full.index(full[4]) + 1
+    assert stop.output == full[:cut] and stop.finish_reason == "stop"
+
+
+def test_command_line(model_dirs):
+    d = model_dirs["A"]
+    prompt = [7, 8, 9, 10, 11]
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "tffinfer"), d, "--fp32", "--prompt-ids",
+           ",".join(map(str, prompt)), "--n-predict", "8", "--n-ctx", "128", "--json", "--ignore-eos"]
+    p = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr
+    rec = json.loads(p.stdout.strip().splitlines()[-1])
+    assert rec["prompt"] == prompt and rec["output"] == plain_generate_greedy(d, prompt, 8)
+    p = subprocess.run([sys.executable, "-m", "tffinfer_amd", d, "--load-only"], capture_output=True, text=True,
+                       timeout=300, cwd=ROOT)
+    assert p.returncode == 0 and "loaded" in p.stderr

@@ -57,11 +57,12 @@ class StepContext(LayerContext):
 
 class ModelRunner:
     def __init__(self, model, page_size: int = 16, num_pages=256, max_seqs: int = 8,
-                 max_model_len: int | None = None, ops=_ops):
+                 max_model_len: int | None = None, ops=_ops, use_graphs: bool = False):
         if model.device is None or model.device.type != "cuda":
             raise StepError("the model has no weights on a GPU; there is no CPU path")
         self.model = model
         self.ops = ops
+        self.use_graphs = bool(use_graphs)
         self.device = model.device
         self.act_dtype = model.dtype
         cfg = model.config
