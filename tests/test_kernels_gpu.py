@@ -142,10 +142,10 @@ def _paged_setup(T_ctx, nkv, d, ps, dtype, seed, extra_pages=3):
     k = torch.randn(T_ctx, nkv, d, generator=g).to(dtype)
     v = torch.randn(T_ctx, nkv, d, generator=g).to(dtype)
     kc = torch.zeros(num_pages, nkv, ps, d, dtype=dtype)
-    vc = torch.zeros(num_pages, nkv, ps, d, dtype=dtype)
+    vc = torch.zeros(num_pages, nkv, d, ps, dtype=dtype)     # values are kept transposed
     for j in range(T_ctx):
         kc[perm[j // ps], :, j % ps] = k[j]
-        vc[perm[j // ps], :, j % ps] = v[j]
+        vc[perm[j // ps], :, :, j % ps] = v[j]
     return k, v, kc, vc, perm.to(torch.int32)
 
 
@@ -218,7 +218,7 @@ def test_qk_norm_rope_kv(dtype, pairing, nq, nkv, d, rot):
     rope = RotaryEmbedding(d, theta, pairing, rotary_dim=rot)
     table = rope.table(128, DEV)
     kc = torch.zeros(num_pages, nkv, ps, d, dtype=dtype, device=DEV)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(num_pages, nkv, d, ps, dtype=dtype, device=DEV)
     dq = qkv.to(DEV).clone()
     ops.qk_norm_rope_kv(dq, nq, nkv, d, qw.to(DEV), kw.to(DEV), eps, table, 1 if pairing == "interleaved" else 0,
                         positions.to(DEV), slots.to(DEV), kc, vc)
@@ -255,10 +255,11 @@ def test_qk_norm_rope_kv(dtype, pairing, nq, nkv, d, rot):
             continue
         written.add(s)
         _close(kc_h[s // ps, :, s % ps], kr[t], tol, f"k of token {t}")
-        _close(vc_h[s // ps, :, s % ps], v[t], tol if dtype == torch.bfloat16 else 0.0, f"v of token {t}")
+        _close(vc_h[s // ps, :, :, s % ps], v[t], tol if dtype == torch.bfloat16 else 0.0, f"v of token {t}")
     for s in range(num_pages * ps):
         if s not in written:
             assert float(kc_h[s // ps, :, s % ps].abs().max()) == 0.0, f"slot {s} was written"
+            assert float(vc_h[s // ps, :, :, s % ps].abs().max()) == 0.0, f"value slot {s} was written"
 
 
 def test_argmax_first_maximum():
@@ -309,3 +310,113 @@ def test_repetition_penalty():
     ops.repetition_penalty(d, flat.to(DEV), cu.to(DEV), pen.to(DEV))
     for r in range(2):
         assert torch.allclose(d[r].cpu(), plain_repetition_penalty(logits[r], seen[r], float(pen[r])))
+
+
+def _fake_step(entries, ps, nkv, d, dtype, seed, extra_pages=2):
+    """entries: (cached tokens P, new tokens n) per request.  Builds per-request
+    keys/values, a shuffled page pool holding all of them, block tables and the
+    step's flat tables, as the engine's batch builder would."""
+    from types import SimpleNamespace
+    g = torch.Generator().manual_seed(seed)
+    R = len(entries)
+    blocks = [-(-(P + n) // ps) for P, n in entries]
+    num_pages = sum(blocks) + extra_pages
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    kc = torch.zeros(num_pages, nkv, ps, d, dtype=dtype)
+    vc = torch.zeros(num_pages, nkv, d, ps, dtype=dtype)
+    width = max(blocks)
+    bt = torch.zeros(R, width, dtype=torch.int32)
+    ks, vs = [], []
+    for r, (P, n) in enumerate(entries):
+        k = torch.randn(P + n, nkv, d, generator=g).to(dtype)
+        v = torch.randn(P + n, nkv, d, generator=g).to(dtype)
+        ks.append(k)
+        vs.append(v)
+        for b in range(blocks[r]):
+            bt[r, b] = perm.pop()
+        for j in range(P + n):
+            kc[bt[r, j // ps], :, j % ps] = k[j]
+            vc[bt[r, j // ps], :, :, j % ps] = v[j]
+    cu = [0]
+    for P, n in entries:
+        cu.append(cu[-1] + n)
+    T = cu[-1]
+    positions = torch.tensor([P + i for P, n in entries for i in range(n)], dtype=torch.int32)
+    token_req = torch.tensor([r for r, (P, n) in enumerate(entries) for _ in range(n)], dtype=torch.int32)
+    batch = SimpleNamespace(
+        num_reqs=R, num_tokens=T, max_new_tokens=max(n for _, n in entries),
+        max_context=max(P + n for P, n in entries), host_cu_tokens=cu,
+        cu_tokens=torch.tensor(cu, dtype=torch.int32, device=DEV),
+        start_pos=torch.tensor([P for P, _ in entries], dtype=torch.int32, device=DEV),
+        positions=positions.to(DEV), token_req=token_req.to(DEV))
+    kv = SimpleNamespace(k_cache=kc.to(DEV), v_cache=vc.to(DEV), block_tables=bt.to(DEV))
+    return batch, kv, ks, vs, positions, token_req
+
+
+@pytest.mark.parametrize("nq,nkv,d,ps,window", [
+    (4, 2, 16, 16, 0), (8, 2, 32, 8, 24), (6, 3, 48, 8, 0), (32, 8, 128, 16, 0), (5, 5, 80, 32, 0),
+    (12, 2, 64, 16, 40), (3, 1, 256, 64, 0), (40, 2, 96, 8, 0), (7, 7, 112, 16, 5), (4, 1, 192, 8, 0)])
+def test_attention_mfma_prompt_portions_and_mixed(nq, nkv, d, ps, window):
+    ops = _ops()
+    # whole prompts, portions after a cached prefix (ending off page edges), single tokens
+    entries = [(0, 37), (50, 13), (129, 1), (0, 1), (63, 2), (7, 70)]
+    batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=nq + d)
+    T = batch.num_tokens
+    g = torch.Generator().manual_seed(2)
+    q = torch.randn(T, nq, d, generator=g).to(torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    ref = torch.zeros(T, nq, d, dtype=torch.float64)
+    for r in range(len(entries)):
+        sel = (token_req == r).nonzero().flatten()
+        ref[sel] = _attn_ref(q[sel], ks[r], vs[r], positions[sel], window, scale)
+    # a wider row, as the fused projection output has
+    wide = torch.zeros(T, nq * d + 2 * nkv * d, dtype=torch.bfloat16)
+    wide[:, :nq * d] = q.reshape(T, nq * d)
+    out = ops.attention_mfma(wide.to(DEV), nq, nkv, d, kv, batch, window, scale)
+    _close(out.reshape(T, nq, d), ref, 1.5e-2, "mfma attention")
+    gen = ops.attention_generic(wide.to(DEV), nq, nkv, d, kv.k_cache, kv.v_cache, kv.block_tables,
+                                batch.token_req, batch.positions, window, scale)
+    _close(gen.reshape(T, nq, d), ref, 1.5e-2, "generic attention on the same step")
+
+
+@pytest.mark.parametrize("nq,nkv,d,ps,window,splits", [
+    (32, 8, 128, 16, 0, None), (32, 8, 128, 16, 0, 1), (32, 8, 128, 16, 0, 7), (4, 2, 16, 16, 0, 3),
+    (8, 2, 32, 8, 24, 4), (40, 2, 96, 8, 0, 5), (6, 3, 48, 8, 100, None), (16, 1, 64, 32, 0, 64)])
+def test_attention_mfma_decode_split_keys(nq, nkv, d, ps, window, splits):
+    ops = _ops()
+    entries = [(0, 1), (1, 1), (31, 1), (32, 1), (700, 1), (255, 1), (64, 1)]
+    batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=d + ps)
+    T = batch.num_tokens
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(T, nq, d, generator=g).to(torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    ref = torch.stack([_attn_ref(q[r:r + 1], ks[r], vs[r], positions[r:r + 1], window, scale)[0]
+                       for r in range(T)])
+    out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale, splits=splits)
+    _close(out.reshape(T, nq, d), ref, 1.5e-2, "split-key decode attention")
+
+
+def test_attention_mfma_far_key_and_window_edge():
+    """A key far back is made to dominate; with a window that just excludes it
+    the output must not see it, with a window that just includes it, it must."""
+    ops = _ops()
+    nq, nkv, d, ps = 8, 2, 64, 16
+    P = 900
+    far = 517
+    for n in (1, 5):
+        entries = [(P, n)]
+        batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=9)
+        q = torch.randn(n, nq, d).to(torch.bfloat16)
+        for gidx in range(nkv):
+            q[:, gidx * 4:(gidx + 1) * 4] = q[:, gidx * 4:gidx * 4 + 1]
+            kfar = (40 * q[0, gidx * 4].float() / q[0, gidx * 4].float().norm()).to(torch.bfloat16)
+            page = int(kv.block_tables[0, far // ps])
+            kv.k_cache[page, gidx, far % ps] = kfar.to(DEV)
+            ks[0][far, gidx] = kfar
+        q[1:] = q[:1]
+        for window, sees in ((0, True), (P - far + 1, True), (P - far, False)):
+            ref = _attn_ref(q, ks[0], vs[0], positions, window, 1 / math.sqrt(d))
+            out = ops.attention_mfma(q.reshape(n, nq * d).to(DEV), nq, nkv, d, kv, batch, window, 1 / math.sqrt(d))
+            _close(out.reshape(n, nq, d), ref, 1.5e-2, f"n={n} window={window}")
+            hit = torch.allclose(out.reshape(n, nq, d)[0, 0].float().cpu(), vs[0][far, 0].float(), atol=5e-2)
+            assert hit == sees, f"n={n} window={window}: far key {'missed' if sees else 'seen'}"

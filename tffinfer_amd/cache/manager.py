@@ -10,8 +10,10 @@ same token slots in each of them.  A group that keeps all keys gives pages back
 when the request ends; a group with a window also gives back every page the
 window has passed, after each step.
 
-Device layout per group: ``kv[cache index, 0 = K / 1 = V, page, kv head,
-slot in page, head element]``.
+Device layout per group: one tensor ``kv[cache index, 0 = K / 1 = V, page, ...]``;
+a key page is ``[kv head, slot in page, head element]``, a value page is kept
+transposed, ``[kv head, head element, slot in page]``, so that the slots of one
+element lie side by side as a matrix-core operand of P.V wants them.
 
 Reference: LLMKVCache / PageManager / LayerKVContext
 (src/core/runtime/KVCache.h:24-31, :36-184, :189-262, :267-473): pages of 32
@@ -109,7 +111,9 @@ class CacheManager:
     def kv_tensors(self, cache_id: int):
         g = self.groups[self._group_of_cache[cache_id]]
         i = g.index_of(cache_id)
-        return g.kv[i, 0], g.kv[i, 1]
+        k = g.kv[i, 0]
+        pages, nkv, ps, d = k.shape
+        return k, g.kv[i, 1].view(pages, nkv, d, ps)   # values are kept transposed
 
     def num_tokens(self, req) -> int:
         return self.requests[req].num_tokens

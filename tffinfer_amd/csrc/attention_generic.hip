@@ -9,6 +9,7 @@
 //   running max m and sum l over chunks       (paged_flash_attention.cu:746-790)
 //   o = sum_j exp(s_j - m) v_j / l
 // q head h reads kv head h / (nq / nkv)       (paged_flash_attention.cu:891-892).
+// Keys lie [page, kv head, slot, element], values [page, kv head, element, slot].
 // Keys are found by block id arithmetic, not by a table of addresses as in the
 // reference (src/kernel/cuda/get_row.cu:73-109).
 #include "common.h"
@@ -23,7 +24,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const int32_t* __restrict__ token_req, const int32_t* __restrict__ positions, int nq, int nkv,
     int d, int page_size, int window, float scale) {
     __shared__ float qs[AG_MAX_D];
-    __shared__ long long koff[64];
+    __shared__ long long voff[64];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int G = nq / nkv;
     const int g = h / G;
@@ -48,14 +49,15 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
         long long off = 0;
         if (valid) {
             const int page = bt[j / page_size];
-            off = (((long long)page * nkv + g) * page_size + (j % page_size)) * d;
-            const TC* kp = k_cache + off;
+            const long long head_base = ((long long)page * nkv + g) * page_size * d;
+            off = head_base + (j % page_size);   // values: [element][slot]
+            const TC* kp = k_cache + head_base + (long long)(j % page_size) * d;
             float dot = 0.f;
             for (int e = 0; e < d; ++e) dot = fmaf(qs[e], to_f32(kp[e]), dot);
             s = dot * scale;
         }
-        __syncthreads();  // earlier readers of koff are done
-        koff[lane] = off;
+        __syncthreads();  // earlier readers of voff are done
+        voff[lane] = off;
         const float cmax = wave_max(s);
         const float m_new = fmaxf(m, cmax);
         const float p = valid ? expf(s - m_new) : 0.f;
@@ -68,11 +70,11 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
         for (int i = 0; i < AG_MAX_D / 64; ++i) acc[i] *= corr;
         for (int jj = 0; jj < nvalid; ++jj) {
             const float pj = __shfl(p, jj, 64);
-            const TC* vp = v_cache + koff[jj];
+            const TC* vp = v_cache + voff[jj];
 #pragma unroll
             for (int i = 0; i < AG_MAX_D / 64; ++i) {
                 const int e = lane + 64 * i;
-                if (e < d) acc[i] = fmaf(pj, to_f32(vp[e]), acc[i]);
+                if (e < d) acc[i] = fmaf(pj, to_f32(vp[(long long)e * page_size]), acc[i]);
             }
         }
     }

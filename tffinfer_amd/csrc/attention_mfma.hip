@@ -1,0 +1,328 @@
+// bfloat16 attention over the paged cache on the gfx950 matrix cores, for
+// prompt portions and for decoding (with the keys split over several waves and
+// merged by a second kernel).  It replaces the reference's fused kernel
+// (src/kernel/cuda/paged_flash_attention.cu:855-1055: 8 queries x 32 keys per
+// block on SIMT FMA, one shape only) and computes the same thing:
+//   s = (q . k) * scale after the product (:723), causal (mask_op.cu:37-43),
+//   running max / sum over key tiles (:746-790), o = softmax(s) . v,
+//   q head h reads kv head h / G (:891-892).
+//
+// One wave works on up to NQT*16 *columns* of one request and one kv head; a
+// column is a (token, q head of the group) pair, columns are numbered
+// token * G + head, so neighbouring columns share their keys.  Per 32 keys:
+//
+//   S^T[key][col] = K[key][:] . Q[col][:]      MFMA 16x16x32, first operand K:
+//       lane (row = key, g) reads 8 consecutive elements of its key's row, which
+//       is how keys lie in a page ([slot][element]);
+//   the result leaves lane (col, g) with keys g*4..g*4+3 of each 16-key tile:
+//       8 scores of its own column, so max, exp and sum need two shuffles only;
+//   O^T[elem][col] += V^T[elem][key] . P^T[key][col]   MFMA 16x16x32 whose 8
+//       contraction slots per lane group g are defined as keys {g*4..g*4+3} of
+//       the first and of the second tile: exactly what the lane already holds
+//       of P, and two 8-byte runs of a value page, which is kept transposed
+//       ([element][slot]) for this purpose.  No operand goes through LDS.
+#include "common.h"
+#include "tffinfer_kernels.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+template <int DT, int NQT, bool SPLIT>
+__global__ __launch_bounds__(64) void attn_mfma_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int bt_stride,
+    const int32_t* __restrict__ cu_tokens, const int32_t* __restrict__ start_pos,
+    const int32_t* __restrict__ work, int tiles_per_entry, int nq, int nkv, int page_size,
+    int window, float scale, int T_total) {
+    constexpr int D = DT * 16;
+    constexpr int KS = (D + 31) / 32;
+    const int lane = threadIdx.x, qc = lane & 15, kg = lane >> 4;
+    int r, col0;
+    if (work) {
+        r = work[2 * blockIdx.x];
+        col0 = work[2 * blockIdx.x + 1];
+    } else {
+        r = blockIdx.x / tiles_per_entry;
+        col0 = (blockIdx.x % tiles_per_entry) * (16 * NQT);
+    }
+    const int g = blockIdx.y;
+    const int G = nq / nkv;
+    const int tok0 = cu_tokens[r];
+    const int n = cu_tokens[r + 1] - tok0;
+    const int P = start_pos[r];
+    const int ncols = n * G;
+    const int32_t* bt = block_tables + (size_t)r * bt_stride;
+
+    // this lane's column in each tile
+    int c_tok[NQT], c_head[NQT], c_pos[NQT], c_lo[NQT];
+    bool c_ok[NQT];
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+        const int c = col0 + t * 16 + qc;
+        c_ok[t] = c < ncols;
+        const int cc = c_ok[t] ? c : ncols - 1;
+        const int tl = cc / G;
+        c_tok[t] = tok0 + tl;
+        c_head[t] = g * G + (cc - tl * G);
+        c_pos[t] = c_ok[t] ? P + tl : -1;   // a missing column sees no key
+        c_lo[t] = window > 0 ? max(0, P + tl - window + 1) : 0;
+    }
+    // keys any column of this wave can see
+    const int tl_first = col0 / G;
+    const int tl_last = (min(col0 + NQT * 16, ncols) - 1) / G;
+    const int kmin = window > 0 ? max(0, P + tl_first - window + 1) : 0;
+    const int kmax = P + tl_last;
+    const int kb0 = (kmin / 32) * 32;
+    const int nsteps = (kmax - kb0) / 32 + 1;
+    int s_begin = 0, s_end = nsteps;
+    if (SPLIT) {
+        const int per = (nsteps + (int)gridDim.z - 1) / (int)gridDim.z;
+        s_begin = (int)blockIdx.z * per;
+        s_end = min(nsteps, s_begin + per);
+    }
+
+    // Q as second operand: lane (col, g) holds elements ks*32 + g*8 .. +8 of its column
+    bf16x8 qf[NQT][KS];
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+        const bf16_t* qp = q + (size_t)c_tok[t] * q_stride + (size_t)c_head[t] * D;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int e = ks * 32 + kg * 8;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (c_ok[t] && e < D) v = *reinterpret_cast<const uint4*>(qp + e);
+            qf[t][ks] = *reinterpret_cast<bf16x8*>(&v);
+        }
+    }
+
+    floatx4 oacc[NQT][DT];
+    float m_run[NQT], l_run[NQT];
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+        m_run[t] = -INFINITY;
+        l_run[t] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) oacc[t][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    for (int s = s_begin; s < s_end; ++s) {
+        const int kb = kb0 + s * 32;
+        floatx4 sacc[NQT][2];
+#pragma unroll
+        for (int t = 0; t < NQT; ++t) sacc[t][0] = sacc[t][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            const int j = min(kb + kt * 16 + qc, kmax);   // rows past the last key repeat it; masked below
+            const int page = bt[j / page_size];
+            const bf16_t* kp = k_cache + (((size_t)page * nkv + g) * page_size + (j % page_size)) * D;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int e = ks * 32 + kg * 8;
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (e < D) v = *reinterpret_cast<const uint4*>(kp + e);
+                const bf16x8 kf = *reinterpret_cast<bf16x8*>(&v);
+#pragma unroll
+                for (int t = 0; t < NQT; ++t)
+                    sacc[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[t][ks], sacc[t][kt], 0, 0, 0);
+            }
+        }
+        // value runs of this lane group: keys kb + g*4 .. +3 and kb + 16 + g*4 .. +3
+        const bf16_t* vrun[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            const int j0 = min(kb + kt * 16 + kg * 4, (kmax / 4) * 4);
+            const int page = bt[j0 / page_size];
+            vrun[kt] = v_cache + ((size_t)page * nkv + g) * D * page_size + (j0 % page_size);
+        }
+        bf16x8 pf[NQT];
+#pragma unroll
+        for (int t = 0; t < NQT; ++t) {
+            float sv[8];
+            float mt = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int j = kb + kt * 16 + kg * 4 + i;
+                    const bool vis = j >= c_lo[t] && j <= c_pos[t];
+                    const float x = vis ? sacc[t][kt][i] * scale : -INFINITY;
+                    sv[kt * 4 + i] = x;
+                    mt = fmaxf(mt, x);
+                }
+            mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            const float m_new = fmaxf(m_run[t], mt);
+            const float alpha = m_new == -INFINITY ? 1.f : __expf(m_run[t] - m_new);
+            float ps = 0.f;
+            bf16x8 pv;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float p = sv[e] == -INFINITY ? 0.f : __expf(sv[e] - m_new);
+                ps += p;
+                pv[e] = (bf16_t)p;
+            }
+            pf[t] = pv;
+            l_run[t] = l_run[t] * alpha + ps;
+            m_run[t] = m_new;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                oacc[t][dt][0] *= alpha; oacc[t][dt][1] *= alpha;
+                oacc[t][dt][2] *= alpha; oacc[t][dt][3] *= alpha;
+            }
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const size_t eoff = (size_t)(dt * 16 + qc) * page_size;
+            union { uint2 u[2]; bf16x8 v; } vf;
+            vf.u[0] = *reinterpret_cast<const uint2*>(vrun[0] + eoff);
+            vf.u[1] = *reinterpret_cast<const uint2*>(vrun[1] + eoff);
+#pragma unroll
+            for (int t = 0; t < NQT; ++t)
+                oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[t], oacc[t][dt], 0, 0, 0);
+        }
+    }
+
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+        float l = l_run[t];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        if (!c_ok[t]) continue;
+        if (SPLIT) {
+            const size_t row = ((size_t)blockIdx.z * T_total + c_tok[t]) * nq + c_head[t];
+            float* po = part_o + row * D;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                *reinterpret_cast<float4*>(po + dt * 16 + kg * 4) =
+                    make_float4(oacc[t][dt][0], oacc[t][dt][1], oacc[t][dt][2], oacc[t][dt][3]);
+            if (kg == 0) {
+                part_ml[row * 2] = m_run[t];
+                part_ml[row * 2 + 1] = l;
+            }
+        } else {
+            const float inv = 1.0f / l;
+            bf16_t* op = out + ((size_t)c_tok[t] * nq + c_head[t]) * D;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                union { bf16_t h[4]; uint2 u; } pk;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) pk.h[i] = (bf16_t)(oacc[t][dt][i] * inv);
+                *reinterpret_cast<uint2*>(op + dt * 16 + kg * 4) = pk.u;
+            }
+        }
+    }
+}
+
+// merges the partial results of the key splits:
+//   m = max m_s, l = sum l_s e^(m_s - m), o = sum o_s e^(m_s - m) / l
+__global__ __launch_bounds__(64) void attn_split_reduce_kernel(const float* __restrict__ part_o,
+                                                                const float* __restrict__ part_ml,
+                                                                bf16_t* __restrict__ out, int splits,
+                                                                int T_total, int nq, int d) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    float m = -INFINITY;
+    for (int s = 0; s < splits; ++s)
+        m = fmaxf(m, part_ml[(((size_t)s * T_total + t) * nq + h) * 2]);
+    float l = 0.f;
+    for (int s = 0; s < splits; ++s) {
+        const float* ml = part_ml + (((size_t)s * T_total + t) * nq + h) * 2;
+        if (ml[0] != -INFINITY) l += ml[1] * __expf(ml[0] - m);
+    }
+    const float inv = 1.0f / l;
+    for (int e = lane; e < d; e += 64) {
+        float acc = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            const size_t row = ((size_t)s * T_total + t) * nq + h;
+            const float ms = part_ml[row * 2];
+            if (ms != -INFINITY) acc += part_o[row * d + e] * __expf(ms - m);
+        }
+        out[((size_t)t * nq + h) * d + e] = (bf16_t)(acc * inv);
+    }
+}
+
+template <int DT>
+static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o, float* part_ml,
+                       const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* block_tables,
+                       int bt_stride, const int32_t* cu_tokens, const int32_t* start_pos,
+                       const int32_t* work, int num_work, int tiles_per_entry, int cols_per_wave,
+                       int splits, int nq, int nkv, int page_size, int window, float scale,
+                       int T_total, hipStream_t s) {
+    const dim3 grid(num_work, nkv, splits);
+#define TFF_ATTN_ARGS                                                                              \
+    q, q_stride, out, part_o, part_ml, k_cache, v_cache, block_tables, bt_stride, cu_tokens,       \
+        start_pos, work, tiles_per_entry, nq, nkv, page_size, window, scale, T_total
+    if (splits > 1) {
+        if (cols_per_wave == 16)
+            attn_mfma_kernel<DT, 1, true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
+        else
+            attn_mfma_kernel<DT, 2, true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
+    } else {
+        if (cols_per_wave == 16)
+            attn_mfma_kernel<DT, 1, false><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
+        else
+            attn_mfma_kernel<DT, 2, false><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
+    }
+#undef TFF_ATTN_ARGS
+    return tff_check_launch("attention_mfma");
+}
+
+TFF_API int tff_attention_mfma_supported(int d, int page_size) {
+    if (page_size <= 0 || page_size % 8) return 0;
+    switch (d) {
+        case 16: case 32: case 48: case 64: case 80: case 96: case 112: case 128: case 192: case 256:
+            return 1;
+        default:
+            return 0;
+    }
+}
+
+TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* part_o, float* part_ml,
+                               const void* k_cache, const void* v_cache,
+                               const int32_t* block_tables, int bt_stride, const int32_t* cu_tokens,
+                               const int32_t* start_pos, const int32_t* work, int num_work,
+                               int tiles_per_entry, int cols_per_wave, int splits, int T_total,
+                               int nq, int nkv, int d, int page_size, int num_pages, int window,
+                               float scale, tff_stream_t stream) {
+    TFF_REQUIRE(q && out && k_cache && v_cache && block_tables && cu_tokens && start_pos,
+                "attention_mfma: null pointer");
+    TFF_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0,
+                "attention_mfma: %d query heads are not a multiple of %d key heads", nq, nkv);
+    TFF_REQUIRE(tff_attention_mfma_supported(d, page_size),
+                "attention_mfma: head size %d with pages of %d is not supported by the matrix-core "
+                "kernel (head sizes 16..128 in steps of 16, 192, 256; pages a multiple of 8)", d, page_size);
+    TFF_REQUIRE(q_stride >= nq * d && q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0,
+                "attention_mfma: query rows must be 16-byte aligned (stride %d)", q_stride);
+    TFF_REQUIRE(cols_per_wave == 16 || cols_per_wave == 32, "attention_mfma: bad tile width %d", cols_per_wave);
+    TFF_REQUIRE(splits >= 1 && splits <= 65535 && nkv <= 65535, "attention_mfma: bad split count %d", splits);
+    TFF_REQUIRE(splits == 1 || (part_o && part_ml), "attention_mfma: split keys need a workspace");
+    TFF_REQUIRE(work || tiles_per_entry >= 1, "attention_mfma: neither a work table nor a tile count");
+    TFF_REQUIRE(bt_stride > 0 && num_pages > 0 && window >= 0 && T_total >= 0, "attention_mfma: bad geometry");
+    if (num_work <= 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+#define TFF_ATTN_CASE(DTV)                                                                          \
+    case DTV * 16:                                                                                  \
+        return launch_attn<DTV>((const bf16_t*)q, q_stride, (bf16_t*)out, part_o, part_ml,          \
+                                (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,       \
+                                bt_stride, cu_tokens, start_pos, work, num_work, tiles_per_entry,   \
+                                cols_per_wave, splits, nq, nkv, page_size, window, scale, T_total, s);
+    switch (d) {
+        TFF_ATTN_CASE(1) TFF_ATTN_CASE(2) TFF_ATTN_CASE(3) TFF_ATTN_CASE(4) TFF_ATTN_CASE(5)
+        TFF_ATTN_CASE(6) TFF_ATTN_CASE(7) TFF_ATTN_CASE(8) TFF_ATTN_CASE(12) TFF_ATTN_CASE(16)
+        default: break;
+    }
+#undef TFF_ATTN_CASE
+    return tff_fail("attention_mfma: head size %d", d);
+}
+
+TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml, void* out,
+                                       int splits, int T_total, int nq, int d, tff_stream_t stream) {
+    TFF_REQUIRE(part_o && part_ml && out, "attention_split_reduce: null pointer");
+    TFF_REQUIRE(splits >= 1 && T_total >= 0 && nq > 0 && nq <= 65535 && d > 0,
+                "attention_split_reduce: bad sizes");
+    if (T_total == 0) return 0;
+    attn_split_reduce_kernel<<<dim3(T_total, nq), 64, 0, (hipStream_t)stream>>>(
+        part_o, part_ml, (bf16_t*)out, splits, T_total, nq, d);
+    return tff_check_launch("attention_split_reduce");
+}

@@ -170,7 +170,12 @@ __global__ void qk_norm_rope_kv_kernel(T* __restrict__ qkv, int nq, int nkv, int
         dst = base + (((size_t)page * nkv + head) * page_size + off) * d;
     }
     if (kind == 2) {
-        for (int e = lane; e < d; e += 64) dst[e] = from_f32<TC>(to_f32(x[e]));
+        // values are kept transposed, [page, kv head, element, slot]: the slots of one element
+        // lie side by side, which is the order a matrix-core operand of P.V wants
+        const int head = hh - nq - nkv;
+        const int page = slot / page_size, off = slot % page_size;
+        TC* vt = v_cache + ((size_t)page * nkv + head) * d * page_size + off;
+        for (int e = lane; e < d; e += 64) vt[(size_t)e * page_size] = from_f32<TC>(to_f32(x[e]));
         return;
     }
     const float* w = kind == 0 ? qw : kw;

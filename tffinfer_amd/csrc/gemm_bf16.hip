@@ -116,6 +116,129 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
     }
 }
 
+// ------------------------------------------------------------- skinny M ---
+// For a few rows of A (decoding: M = number of live requests) the product is
+// a stream of W from HBM; what counts is bytes in flight, not LDS tiling.
+// A block owns a slab of 16*R rows of W for the whole of K; its waves split K
+// among them in contiguous runs, each wave reading W straight from global
+// memory into MFMA operands (16 rows x 64 contiguous bytes per load) and the
+// few rows of A from cache; partial sums meet in LDS and are added in a fixed
+// order, so no partial result goes through global memory and the result does
+// not depend on the launch.
+#define SK_WAVES 8
+
+template <int MT, int R, typename TC>
+__global__ __launch_bounds__(64 * SK_WAVES) void gemm_bf16_skinny_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, TC* __restrict__ C, int M, int N,
+    int K, int lda) {
+    __shared__ floatx4 part[SK_WAVES - 1][R * MT][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int fr = lane & 15, fg = lane >> 4;
+    const int n0 = blockIdx.x * (16 * R);
+
+    floatx4 acc[R][MT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[r][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // k-steps of 32 are dealt out to the waves in contiguous runs
+    const int nsteps = (K + 31) / 32;
+    const int per = (nsteps + SK_WAVES - 1) / SK_WAVES;
+    const int s_begin = wave * per;
+    const int s_end = min(nsteps, s_begin + per);
+
+    const bf16_t* wrow[R];
+    bool wok[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int n = n0 + r * 16 + fr;
+        wok[r] = n < N;
+        wrow[r] = W + (size_t)(wok[r] ? n : 0) * K;
+    }
+    const bf16_t* arow[MT];
+    bool aok[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + fr;
+        aok[t] = m < M;
+        arow[t] = A + (size_t)(aok[t] ? m : 0) * lda;
+    }
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    constexpr int UNROLL = 4;
+    for (int s0 = s_begin; s0 < s_end; s0 += UNROLL) {
+        uint4 rw[UNROLL][R], ra[UNROLL][MT];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int k = (s0 + u) * 32 + fg * 8;
+            const bool kok = (s0 + u) < s_end && k < K;
+#pragma unroll
+            for (int r = 0; r < R; ++r) rw[u][r] = (kok && wok[r]) ? ld16(wrow[r] + k) : zero;
+#pragma unroll
+            for (int t = 0; t < MT; ++t) ra[u][t] = (kok && aok[t]) ? ld16(arow[t] + k) : zero;
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        *reinterpret_cast<bf16x8*>(&rw[u][r]), *reinterpret_cast<bf16x8*>(&ra[u][t]),
+                        acc[r][t], 0, 0, 0);
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) part[wave - 1][r * MT + t][lane] = acc[r][t];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const bool vec = (N % 4) == 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                floatx4 v = acc[r][t];
+#pragma unroll
+                for (int w = 0; w < SK_WAVES - 1; ++w) {
+                    const floatx4 p = part[w][r * MT + t][lane];
+                    v[0] += p[0]; v[1] += p[1]; v[2] += p[2]; v[3] += p[3];
+                }
+                const int n = n0 + r * 16 + fg * 4;
+                const int m = t * 16 + fr;
+                if (m >= M || n >= N) continue;
+                TC* dst = C + (size_t)m * N + n;
+                if (vec) {
+                    if constexpr (sizeof(TC) == 4) {
+                        *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+                    } else {
+                        union { bf16_t h[4]; uint2 u; } pk;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) pk.h[e] = (bf16_t)v[e];
+                        *reinterpret_cast<uint2*>(dst) = pk.u;
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < N) dst[e] = from_f32<TC>(v[e]);
+                }
+            }
+    }
+}
+
+template <int MT, int R>
+static int launch_skinny(const bf16_t* A, const bf16_t* W, void* C, int M, int N, int K, int lda,
+                         int c_dtype, hipStream_t s) {
+    const dim3 grid((N + 16 * R - 1) / (16 * R));
+    if (c_dtype == TFF_F32)
+        gemm_bf16_skinny_kernel<MT, R, float><<<grid, 64 * SK_WAVES, 0, s>>>(A, W, (float*)C, M, N, K, lda);
+    else
+        gemm_bf16_skinny_kernel<MT, R, bf16_t><<<grid, 64 * SK_WAVES, 0, s>>>(A, W, (bf16_t*)C, M, N, K, lda);
+    return tff_check_launch("gemm_bf16_skinny");
+}
+
 int tff_gemm_bf16(const bf16_t* A, const bf16_t* W, void* C, int M, int N, int K, int lda,
                   int c_dtype, hipStream_t s) {
     TFF_REQUIRE(K % 8 == 0 && lda % 8 == 0,
@@ -123,6 +246,22 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* W, void* C, int M, int N, int K
                 K, lda);
     TFF_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)C % 16) == 0,
                 "gemm: operands must be 16-byte aligned");
+    TFF_REQUIRE(c_dtype == TFF_F32 || c_dtype == TFF_BF16, "gemm: unknown output type %d", c_dtype);
+    if (M <= 64) {
+        // slabs of 32 rows when that still gives every CU several blocks, else of 16
+        const bool wide = N >= 32 * 1024;
+        const int mt = (M + 15) / 16;
+        switch (mt * 2 + (wide ? 1 : 0)) {
+            case 2: return launch_skinny<1, 1>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 3: return launch_skinny<1, 2>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 4: return launch_skinny<2, 1>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 5: return launch_skinny<2, 2>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 6: return launch_skinny<3, 1>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 7: return launch_skinny<3, 2>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 8: return launch_skinny<4, 1>(A, W, C, M, N, K, lda, c_dtype, s);
+            default: return launch_skinny<4, 2>(A, W, C, M, N, K, lda, c_dtype, s);
+        }
+    }
     dim3 grid((N + G_BN - 1) / G_BN, (M + G_BM - 1) / G_BM);
     TFF_REQUIRE(grid.y <= 65535, "gemm: too many rows M=%d", M);
     if (c_dtype == TFF_F32)

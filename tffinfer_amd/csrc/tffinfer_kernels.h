@@ -42,7 +42,7 @@ TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K,
 // then the rotation of pairs by cos_sin[pos, pair] (skipped if null); q is
 // written back in place, k and v go to their page slot slot_mapping[t]
 // (skipped if negative).  pairing 0: pairs (i, i + rot/2); 1: pairs (2i, 2i+1).
-// Cache layout: [pages, nkv, page_size, d].
+// Cache layout: keys [pages, nkv, page_size, d], values transposed [pages, nkv, d, page_size].
 TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d,
                                 const float* q_weight, const float* k_weight, float eps,
                                 const float* cos_sin, int rot_dim, int pairing, int max_pos,

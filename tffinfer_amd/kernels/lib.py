@@ -28,6 +28,10 @@ _SIGNATURES = {
                             _I, _I, _I, _I, _P],
     "tff_attention_generic": [_P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                               _F, _I, _I, _P],
+    "tff_attention_mfma_supported": [_I, _I],
+    "tff_attention_mfma": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I,
+                           _I, _I, _I, _F, _P],
+    "tff_attention_split_reduce": [_P, _P, _P, _I, _I, _I, _I, _P],
     "tff_swiglu": [_P, _P, _I, _I, _I, _P],
     "tff_cast": [_P, _I, _P, _I, c_int64, _P],
     "tff_argmax": [_P, _P, _I, _I, _P],

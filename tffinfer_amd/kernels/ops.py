@@ -44,6 +44,15 @@ def _req(t: torch.Tensor, name: str, dtype=None, ndim=None):
     return t
 
 
+def _check_cache(k_cache, v_cache, nkv, d, what):
+    """Keys [pages, nkv, page_size, d]; values transposed [pages, nkv, d, page_size]."""
+    pages, h, ps, dd = k_cache.shape
+    if h != nkv or dd != d or tuple(v_cache.shape) != (pages, nkv, d, ps) or v_cache.dtype != k_cache.dtype:
+        raise _lib.KernelError(
+            f"{what}: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} are not keys "
+            f"[pages, {nkv}, page_size, {d}] and values [pages, {nkv}, {d}, page_size]")
+
+
 def _ptr(t):
     return None if t is None else t.data_ptr()
 
@@ -168,9 +177,7 @@ def qk_norm_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int,
         raise _lib.KernelError("qk_norm_rope_kv: positions and slot_mapping need one entry per token")
     _req(k_cache, "k cache", ndim=4)
     _req(v_cache, "v cache", ndim=4)
-    if k_cache.shape != v_cache.shape or k_cache.shape[1] != nkv or k_cache.shape[3] != d:
-        raise _lib.KernelError(
-            f"qk_norm_rope_kv: cache {tuple(k_cache.shape)} is not [pages, {nkv}, page_size, {d}]")
+    _check_cache(k_cache, v_cache, nkv, d, "qk_norm_rope_kv")
     L = _lib.load()
     _lib.check(L.tff_qk_norm_rope_kv(
         qkv.data_ptr(), T, nq, nkv, d, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin),
@@ -191,9 +198,7 @@ def attention_generic(q: torch.Tensor, nq: int, nkv: int, d: int, k_cache: torch
         raise _lib.KernelError(f"attention q: rows of {q.shape[1]} hold fewer than nq*d = {nq * d}")
     _req(k_cache, "k cache", q.dtype, 4)
     _req(v_cache, "v cache", q.dtype, 4)
-    if k_cache.shape != v_cache.shape or k_cache.shape[1] != nkv or k_cache.shape[3] != d:
-        raise _lib.KernelError(
-            f"attention: cache {tuple(k_cache.shape)} is not [pages, {nkv}, page_size, {d}]")
+    _check_cache(k_cache, v_cache, nkv, d, "attention")
     _req(block_tables, "block tables", torch.int32, 2)
     _req(token_req, "token_req", torch.int32, 1)
     _req(positions, "positions", torch.int32, 1)
@@ -212,11 +217,93 @@ def attention_generic(q: torch.Tensor, nq: int, nkv: int, d: int, k_cache: torch
     return out
 
 
+def mfma_attention_supported(dtype: torch.dtype, d: int, page_size: int) -> bool:
+    return dtype == torch.bfloat16 and bool(_lib.load().tff_attention_mfma_supported(int(d), int(page_size)))
+
+
+def _attention_work(batch, G: int, cols: int, device) -> torch.Tensor:
+    """(entry, first column) of every wave's tile for the step's entries; a
+    column is a (token, q head of the group) pair numbered token * G + head."""
+    cache = getattr(batch, "_attn_work", None)
+    if cache is None:
+        cache = batch._attn_work = {}
+    key = (G, cols)
+    if key not in cache:
+        cu = batch.host_cu_tokens
+        flat = []
+        for r in range(len(cu) - 1):
+            for c0 in range(0, (cu[r + 1] - cu[r]) * G, cols):
+                flat.extend((r, c0))
+        cache[key] = torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(device)
+    return cache[key]
+
+
+def pick_splits(waves: int, max_context: int) -> int:
+    """Into how many runs the keys of a decoding request are split so that
+    the launch has enough waves to pull on all of HBM: about 2048 waves, at
+    least 64 keys per run."""
+    return max(1, min(-(-2048 // max(1, waves)), -(-max_context // 64), 256))
+
+
+def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,
+                   scale: float | None = None, splits: int | None = None) -> torch.Tensor:
+    """bfloat16 attention of the step's tokens on the matrix cores; decode-only
+    steps split each request's keys over several waves and merge them."""
+    _req(q, "attention q", torch.bfloat16, 2)
+    T = q.shape[0]
+    if q.shape[1] < nq * d:
+        raise _lib.KernelError(f"attention q: rows of {q.shape[1]} hold fewer than nq*d = {nq * d}")
+    k_cache, v_cache = kv.k_cache, kv.v_cache
+    _req(k_cache, "k cache", q.dtype, 4)
+    _req(v_cache, "v cache", q.dtype, 4)
+    _check_cache(k_cache, v_cache, nkv, d, "attention")
+    bt = _req(kv.block_tables, "block tables", torch.int32, 2)
+    _req(batch.cu_tokens, "cu_tokens", torch.int32, 1)
+    _req(batch.start_pos, "start_pos", torch.int32, 1)
+    R = batch.num_reqs
+    if batch.cu_tokens.numel() != R + 1 or batch.start_pos.numel() != R or bt.shape[0] != R:
+        raise _lib.KernelError("attention: the step's tables do not describe the same number of requests")
+    if batch.num_tokens != T:
+        raise _lib.KernelError(f"attention: {T} query rows for a step of {batch.num_tokens} tokens")
+    G = nq // nkv
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    out = torch.empty(T, nq * d, dtype=q.dtype, device=q.device)
+    L = _lib.load()
+    part_o = part_ml = None
+    if batch.max_new_tokens == 1:
+        tiles = -(-G // 16)
+        work, num_work, cols = None, R * tiles, 16
+        if splits is None:
+            splits = getattr(batch, "attn_splits", None) or pick_splits(num_work * nkv, batch.max_context)
+        if splits > 1:
+            part_o = torch.empty(splits, T, nq, d, dtype=torch.float32, device=q.device)
+            part_ml = torch.empty(splits, T, nq, 2, dtype=torch.float32, device=q.device)
+    else:
+        tiles, splits = 1, 1
+        cols = 32 if batch.max_new_tokens * G > 16 else 16
+        work = _attention_work(batch, G, cols, q.device)
+        num_work = work.shape[0]
+    dest = out
+    _lib.check(L.tff_attention_mfma(
+        q.data_ptr(), q.stride(0), dest.data_ptr(), _ptr(part_o), _ptr(part_ml), k_cache.data_ptr(),
+        v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(),
+        batch.start_pos.data_ptr(), _ptr(work), num_work, tiles, cols, splits, T, nq, nkv, d,
+        k_cache.shape[2], k_cache.shape[0], int(window), float(scale), _stream()))
+    if splits > 1:
+        _lib.check(L.tff_attention_split_reduce(part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(),
+                                                splits, T, nq, d, _stream()))
+    return out
+
+
 def paged_attention(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,
                     scale: float | None = None) -> torch.Tensor:
     """Attention of a step's tokens over the cache view ``kv`` (k_cache,
-    v_cache, block_tables) with the step's ``batch`` (token_req, positions).
-    Picks the kernel for the element type and the shape of the step."""
+    v_cache, block_tables) with the step's ``batch``.  bfloat16 with a head
+    size the matrix-core kernel takes runs there; everything else (float32,
+    other head sizes) on the general kernel."""
+    if mfma_attention_supported(q.dtype, d, kv.k_cache.shape[2]):
+        return attention_mfma(q, nq, nkv, d, kv, batch, window, scale)
     return attention_generic(q, nq, nkv, d, kv.k_cache, kv.v_cache, kv.block_tables,
                              batch.token_req, batch.positions, window, scale)
 
@@ -299,7 +386,9 @@ OP_TABLE = {
     "rmsnorm": rmsnorm,
     "linear": linear,
     "qk_norm_rope_kv": qk_norm_rope_kv,
-    "attention": attention_generic,
+    "attention": paged_attention,
+    "attention_generic": attention_generic,
+    "attention_mfma": attention_mfma,
     "swiglu": swiglu,
     "cast": cast,
     "argmax": argmax,
