@@ -54,3 +54,27 @@ def test_trace_run_program(model_dirs, tmp_path, dtype):
     out = rl.run_steps_subprocess(model_dir, dtype, steps, str(tmp_path / "out"),
                                   rl.max_live_tokens(steps, 64))
     rl.check_against_oracle(model_dir, reqs, steps, out, TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("mode", ["tail", "mixed"])
+def test_replay_with_decode_graphs(model_dirs, name, dtype, mode):
+    """Decode-only steps run as replays of a captured HIP graph: every replay,
+    with the engine's own eager steps between them, must match the plain
+    implementation (a graph that bakes in a size or a table goes wrong on the
+    second replay, not on the first)."""
+    from tffinfer_amd.engine.runner import ModelRunner
+    from tffinfer_amd.models import load_model
+    model_dir = model_dirs[name]
+    reqs = requests_for(name, model_dir)
+    steps = {"tail": rl.trace_tail, "mixed": rl.trace_mixed}[mode](reqs)
+    ps = PAGE_SIZE[name]
+    num_pages = rl.max_live_tokens(steps, unit=ps) // ps
+    model = load_model(model_dir, DTYPES[dtype], "cuda:0")
+    runner = ModelRunner(model, page_size=ps, num_pages=num_pages, max_seqs=4, use_graphs=True)
+    results = rl.run_steps_in_process(runner, steps)
+    assert runner._graphs, "no decode step went through a graph"
+    decode_only = sum(1 for s in steps if s["entries"] and all(len(e["tokens"]) == 1 for e in s["entries"]))
+    assert decode_only >= 3
+    rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])

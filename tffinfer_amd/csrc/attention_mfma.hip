@@ -109,9 +109,9 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
 
     for (int s = s_begin; s < s_end; ++s) {
         const int kb = kb0 + s * 32;
-        floatx4 sacc[NQT][2];
-#pragma unroll
-        for (int t = 0; t < NQT; ++t) sacc[t][0] = sacc[t][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+        // every load of the step is issued before the first product, so the wave keeps the
+        // whole 32-key slice of K and of V in flight at once
+        bf16x8 kf[2][KS];
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt) {
             const int j = min(kb + kt * 16 + qc, kmax);   // rows past the last key repeat it; masked below
@@ -122,20 +122,37 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
                 const int e = ks * 32 + kg * 8;
                 uint4 v = make_uint4(0, 0, 0, 0);
                 if (e < D) v = *reinterpret_cast<const uint4*>(kp + e);
-                const bf16x8 kf = *reinterpret_cast<bf16x8*>(&v);
-#pragma unroll
-                for (int t = 0; t < NQT; ++t)
-                    sacc[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[t][ks], sacc[t][kt], 0, 0, 0);
+                kf[kt][ks] = *reinterpret_cast<bf16x8*>(&v);
             }
         }
         // value runs of this lane group: keys kb + g*4 .. +3 and kb + 16 + g*4 .. +3
-        const bf16_t* vrun[2];
+        union VF { uint2 u[2]; bf16x8 v; };
+        VF vf[DT];
+        {
+            const bf16_t* vrun[2];
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-            const int j0 = min(kb + kt * 16 + kg * 4, (kmax / 4) * 4);
-            const int page = bt[j0 / page_size];
-            vrun[kt] = v_cache + ((size_t)page * nkv + g) * D * page_size + (j0 % page_size);
+            for (int kt = 0; kt < 2; ++kt) {
+                const int j0 = min(kb + kt * 16 + kg * 4, (kmax / 4) * 4);
+                const int page = bt[j0 / page_size];
+                vrun[kt] = v_cache + ((size_t)page * nkv + g) * D * page_size + (j0 % page_size);
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const size_t eoff = (size_t)(dt * 16 + qc) * page_size;
+                vf[dt].u[0] = *reinterpret_cast<const uint2*>(vrun[0] + eoff);
+                vf[dt].u[1] = *reinterpret_cast<const uint2*>(vrun[1] + eoff);
+            }
         }
+        floatx4 sacc[NQT][2];
+#pragma unroll
+        for (int t = 0; t < NQT; ++t) sacc[t][0] = sacc[t][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int t = 0; t < NQT; ++t)
+                    sacc[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kt][ks], qf[t][ks], sacc[t][kt], 0, 0, 0);
         bf16x8 pf[NQT];
 #pragma unroll
         for (int t = 0; t < NQT; ++t) {
@@ -173,15 +190,10 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
             }
         }
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const size_t eoff = (size_t)(dt * 16 + qc) * page_size;
-            union { uint2 u[2]; bf16x8 v; } vf;
-            vf.u[0] = *reinterpret_cast<const uint2*>(vrun[0] + eoff);
-            vf.u[1] = *reinterpret_cast<const uint2*>(vrun[1] + eoff);
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int t = 0; t < NQT; ++t)
-                oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[t], oacc[t][dt], 0, 0, 0);
-        }
+                oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf[t], oacc[t][dt], 0, 0, 0);
     }
 
 #pragma unroll
@@ -217,27 +229,29 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
 
 // merges the partial results of the key splits:
 //   m = max m_s, l = sum l_s e^(m_s - m), o = sum o_s e^(m_s - m) / l
-__global__ __launch_bounds__(64) void attn_split_reduce_kernel(const float* __restrict__ part_o,
-                                                                const float* __restrict__ part_ml,
-                                                                bf16_t* __restrict__ out, int splits,
-                                                                int T_total, int nq, int d) {
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    float m = -INFINITY;
-    for (int s = 0; s < splits; ++s)
-        m = fmaxf(m, part_ml[(((size_t)s * T_total + t) * nq + h) * 2]);
-    float l = 0.f;
-    for (int s = 0; s < splits; ++s) {
-        const float* ml = part_ml + (((size_t)s * T_total + t) * nq + h) * 2;
-        if (ml[0] != -INFINITY) l += ml[1] * __expf(ml[0] - m);
+__global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __restrict__ part_o,
+                                                                 const float* __restrict__ part_ml,
+                                                                 bf16_t* __restrict__ out, int splits,
+                                                                 int T_total, int nq, int d) {
+    __shared__ float w[256];
+    __shared__ float red[17];
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    float ms = -INFINITY, ls = 0.f;
+    if (tid < splits) {
+        const float* ml = part_ml + (((size_t)tid * T_total + t) * nq + h) * 2;
+        ms = ml[0];
+        ls = ml[1];
     }
+    const float m = block_max(ms, red);
+    const float ws = ms == -INFINITY ? 0.f : __expf(ms - m);
+    w[tid] = ws;
+    const float l = block_sum(ls * ws, red);   // its barriers also publish w
     const float inv = 1.0f / l;
-    for (int e = lane; e < d; e += 64) {
+    for (int e = tid; e < d; e += blockDim.x) {
         float acc = 0.f;
-        for (int s = 0; s < splits; ++s) {
-            const size_t row = ((size_t)s * T_total + t) * nq + h;
-            const float ms = part_ml[row * 2];
-            if (ms != -INFINITY) acc += part_o[row * d + e] * __expf(ms - m);
-        }
+#pragma unroll 8
+        for (int s = 0; s < splits; ++s)
+            acc = fmaf(part_o[(((size_t)s * T_total + t) * nq + h) * d + e], w[s], acc);
         out[((size_t)t * nq + h) * d + e] = (bf16_t)(acc * inv);
     }
 }
@@ -322,7 +336,8 @@ TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml
     TFF_REQUIRE(splits >= 1 && T_total >= 0 && nq > 0 && nq <= 65535 && d > 0,
                 "attention_split_reduce: bad sizes");
     if (T_total == 0) return 0;
-    attn_split_reduce_kernel<<<dim3(T_total, nq), 64, 0, (hipStream_t)stream>>>(
+    TFF_REQUIRE(splits <= 256, "attention_split_reduce: at most 256 splits, got %d", splits);
+    attn_split_reduce_kernel<<<dim3(T_total, nq), 256, 0, (hipStream_t)stream>>>(
         part_o, part_ml, (bf16_t*)out, splits, T_total, nq, d);
     return tff_check_launch("attention_split_reduce");
 }

@@ -127,7 +127,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
 // not depend on the launch.
 #define SK_WAVES 8
 
-template <int MT, int R, typename TC>
+// UNROLL k-steps of loads are issued before the first is used: a wave keeps
+// UNROLL * (R + MT) KB in flight, which is what hides the latency of HBM.
+template <int MT, int R, int UNROLL, typename TC>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, TC* __restrict__ C, int M, int N,
     int K, int lda) {
@@ -165,7 +167,6 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_bf16_skinny_kernel(
         arow[t] = A + (size_t)(aok[t] ? m : 0) * lda;
     }
     const uint4 zero = make_uint4(0, 0, 0, 0);
-    constexpr int UNROLL = 4;
     for (int s0 = s_begin; s0 < s_end; s0 += UNROLL) {
         uint4 rw[UNROLL][R], ra[UNROLL][MT];
 #pragma unroll
@@ -228,14 +229,14 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_bf16_skinny_kernel(
     }
 }
 
-template <int MT, int R>
+template <int MT, int R, int UNROLL>
 static int launch_skinny(const bf16_t* A, const bf16_t* W, void* C, int M, int N, int K, int lda,
                          int c_dtype, hipStream_t s) {
     const dim3 grid((N + 16 * R - 1) / (16 * R));
     if (c_dtype == TFF_F32)
-        gemm_bf16_skinny_kernel<MT, R, float><<<grid, 64 * SK_WAVES, 0, s>>>(A, W, (float*)C, M, N, K, lda);
+        gemm_bf16_skinny_kernel<MT, R, UNROLL, float><<<grid, 64 * SK_WAVES, 0, s>>>(A, W, (float*)C, M, N, K, lda);
     else
-        gemm_bf16_skinny_kernel<MT, R, bf16_t><<<grid, 64 * SK_WAVES, 0, s>>>(A, W, (bf16_t*)C, M, N, K, lda);
+        gemm_bf16_skinny_kernel<MT, R, UNROLL, bf16_t><<<grid, 64 * SK_WAVES, 0, s>>>(A, W, (bf16_t*)C, M, N, K, lda);
     return tff_check_launch("gemm_bf16_skinny");
 }
 
@@ -252,14 +253,14 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* W, void* C, int M, int N, int K
         const bool wide = N >= 32 * 1024;
         const int mt = (M + 15) / 16;
         switch (mt * 2 + (wide ? 1 : 0)) {
-            case 2: return launch_skinny<1, 1>(A, W, C, M, N, K, lda, c_dtype, s);
-            case 3: return launch_skinny<1, 2>(A, W, C, M, N, K, lda, c_dtype, s);
-            case 4: return launch_skinny<2, 1>(A, W, C, M, N, K, lda, c_dtype, s);
-            case 5: return launch_skinny<2, 2>(A, W, C, M, N, K, lda, c_dtype, s);
-            case 6: return launch_skinny<3, 1>(A, W, C, M, N, K, lda, c_dtype, s);
-            case 7: return launch_skinny<3, 2>(A, W, C, M, N, K, lda, c_dtype, s);
-            case 8: return launch_skinny<4, 1>(A, W, C, M, N, K, lda, c_dtype, s);
-            default: return launch_skinny<4, 2>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 2: return launch_skinny<1, 1, 16>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 3: return launch_skinny<1, 2, 8>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 4: return launch_skinny<2, 1, 8>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 5: return launch_skinny<2, 2, 6>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 6: return launch_skinny<3, 1, 6>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 7: return launch_skinny<3, 2, 4>(A, W, C, M, N, K, lda, c_dtype, s);
+            case 8: return launch_skinny<4, 1, 6>(A, W, C, M, N, K, lda, c_dtype, s);
+            default: return launch_skinny<4, 2, 4>(A, W, C, M, N, K, lda, c_dtype, s);
         }
     }
     dim3 grid((N + G_BN - 1) / G_BN, (M + G_BM - 1) / G_BM);

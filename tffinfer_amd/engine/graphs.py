@@ -1,0 +1,166 @@
+"""Decode steps as HIP graphs.
+
+A step in which every request brings exactly one token launches some four
+hundred small kernels; at small batches the time to launch them from Python
+exceeds the time they run.  Such steps are therefore captured once per batch
+size bucket into a HIP graph (through torch's CUDAGraph, which records the
+launches made on its capture stream, ours included) and replayed: the step's
+tables are written into fixed device buffers, the graph runs, the logits
+appear in a fixed tensor.  Rows beyond the live requests are padding: token 0
+at position 0 that writes no key and whose logits nobody reads.
+
+Nothing in a captured step clears memory with a memset node, and the kernels
+take every size from the tables, so one graph serves any mix of context
+lengths.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from .batch import GroupTables, StepBatch
+
+
+def _pad4(n: int) -> int:
+    return (n + 3) & ~3
+
+
+class DecodeGraph:
+    def __init__(self, runner, bucket: int):
+        self.runner = runner
+        self.B = B = int(bucket)
+        cache = runner.cache
+        ps = cache.page_size
+        self.widths = [-(-runner.max_model_len // ps) for _ in cache.groups]
+        # sections of the packed table buffer, as in build_step_batch
+        sizes = [B, B, B, B + 1, B, B, B, B, B]
+        for w in self.widths:
+            sizes += [B * w, B]
+        self.offs, total = [], 0
+        for n in sizes:
+            self.offs.append(total)
+            total += _pad4(n)
+        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.hv = self.host.numpy()
+        self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
+        o = self.offs
+
+        def sl(i, n):
+            return self.dev[o[i]:o[i] + n]
+
+        b = StepBatch()
+        b.num_tokens = b.num_reqs = b.num_logit_rows = B
+        b.max_new_tokens = 1
+        b.max_context = runner.max_model_len
+        b.token_ids, b.positions, b.token_req = sl(0, B), sl(1, B), sl(2, B)
+        b.cu_tokens, b.start_pos, b.context_lens = sl(3, B + 1), sl(4, B), sl(5, B)
+        b.state_slots, b.logit_rows = sl(6, B), sl(7, B)
+        no_slot = sl(8, B)
+        for gi, w in enumerate(self.widths):
+            bt = self.dev[o[9 + 2 * gi]:o[9 + 2 * gi] + B * w].view(B, w)
+            b.groups.append(GroupTables(bt, sl(10 + 2 * gi, B), no_slot))
+        b.host_cu_tokens = list(range(B + 1))
+        b.host_start_pos = [0] * B
+        b.host_state_slots = [0] * B
+        b.reqs = [None] * B
+        self.batch = b
+        # fixed parts of the tables
+        hv = self.hv
+        hv[o[2]:o[2] + B] = np.arange(B)            # token_req
+        hv[o[3]:o[3] + B + 1] = np.arange(B + 1)    # cu_tokens
+        hv[o[7]:o[7] + B] = np.arange(B)            # logit rows: every row
+        hv[o[8]:o[8] + B] = -1                      # no-slot mapping
+        self._row_state = [None] * B                # (request, table lengths) last written per row
+        self._pad_rows(0)
+        self.graph = None
+        self.logits = None
+        self._copied = torch.cuda.Event()
+
+    def _pad_rows(self, first: int) -> None:
+        o, hv, B = self.offs, self.hv, self.B
+        if first >= B:
+            return
+        hv[o[0] + first:o[0] + B] = 0               # token
+        hv[o[1] + first:o[1] + B] = 0               # position
+        hv[o[4] + first:o[4] + B] = 0               # start_pos
+        hv[o[5] + first:o[5] + B] = 1               # context length
+        hv[o[6] + first:o[6] + B] = 0               # state slot
+        for gi, w in enumerate(self.widths):
+            hv[o[10 + 2 * gi] + first:o[10 + 2 * gi] + B] = -1   # writes no key
+            for r in range(first, B):
+                if self._row_state[r] is not None:
+                    hv[o[9 + 2 * gi] + r * w:o[9 + 2 * gi] + (r + 1) * w] = 0
+        for r in range(first, B):
+            self._row_state[r] = None
+
+    def fill(self, entries) -> None:
+        """Writes the step's tables for ``entries`` (one token each, pages reserved)."""
+        cache, o, hv = self.runner.cache, self.offs, self.hv
+        ps = cache.page_size
+        R = len(entries)
+        self._copied.synchronize()      # the last copy out of the host buffer is done
+        for r, e in enumerate(entries):
+            P = cache.num_tokens(e.req)
+            hv[o[0] + r] = e.tokens[0]
+            hv[o[1] + r] = P
+            hv[o[4] + r] = P
+            hv[o[5] + r] = P + 1
+            hv[o[6] + r] = cache.slot(e.req)
+            prev = self._row_state[r]
+            lens = []
+            for gi, w in enumerate(self.widths):
+                table = cache.block_table(gi, e.req)
+                base = o[9 + 2 * gi] + r * w
+                n = len(table)
+                same = prev is not None and prev[0] == e.req and cache.groups[gi].spec.window == 0
+                if same:
+                    # a table that keeps all keys only grows: write what is new
+                    if n > prev[1][gi]:
+                        hv[base + prev[1][gi]:base + n] = table[prev[1][gi]:]
+                else:
+                    hv[base:base + n] = [p if p >= 0 else 0 for p in table]
+                    if prev is not None and prev[1][gi] > n:
+                        hv[base + n:base + prev[1][gi]] = 0
+                lens.append(n)
+                hv[o[10 + 2 * gi] + r] = table[P // ps] * ps + P % ps
+            self._row_state[r] = (e.req, lens)
+        self._pad_rows(R)
+
+    def _forward(self):
+        from .runner import StepContext
+        rn = self.runner
+        ctx = StepContext(rn.ops, rn.act_dtype, self.batch, rn.max_model_len, rn._calls, rn.cache)
+        return rn.model.forward(ctx)
+
+    def capture(self) -> None:
+        rn = self.runner
+        # the decode attention sizes its key splits for the longest context the engine allows
+        # (batch.max_context), so the launch is the same whatever the requests hold
+        side = torch.cuda.Stream(device=rn.device)
+        side.wait_stream(torch.cuda.current_stream(rn.device))
+        with torch.cuda.stream(side):
+            self.dev.copy_(self.host, non_blocking=True)
+            for _ in range(2):          # warm up: allocations, rotation tables
+                self._forward()
+            side.synchronize()
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph, stream=side):
+                self.logits = self._forward()
+        torch.cuda.current_stream(rn.device).wait_stream(side)
+        torch.cuda.synchronize(rn.device)
+
+    def run(self, entries) -> torch.Tensor:
+        self.fill(entries)
+        self.dev.copy_(self.host, non_blocking=True)
+        self._copied.record()
+        self.graph.replay()
+        return self.logits
+
+
+def graph_buckets(max_seqs: int) -> list[int]:
+    out, b = [], 1
+    while b < max_seqs:
+        out.append(b)
+        b *= 2
+    out.append(max_seqs)
+    return out

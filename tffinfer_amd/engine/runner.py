@@ -15,6 +15,7 @@ from ..cache.block_pool import OutOfPages
 from ..cache.manager import CacheManager
 from ..kernels import ops as _ops
 from .batch import KVView, StepBatch, StepEntry, build_step_batch
+from .graphs import DecodeGraph, graph_buckets
 
 
 class StepError(ValueError):
@@ -79,6 +80,9 @@ class ModelRunner:
             if group is not None:
                 k, v = self.cache.kv_tensors(cache_id)
             self._calls.append((cache_id, writes, group, k, v, self.cache.state_tensors.get(cache_id)))
+        # decode-only steps replay a HIP graph if every part of the model can be captured
+        self._graphs = {}
+        self._graph_buckets = graph_buckets(max_seqs) if (self.use_graphs and model.graph_safe()) else []
 
     # ---- requests --------------------------------------------------------
     def add_request(self, req) -> int:
@@ -134,6 +138,9 @@ class ModelRunner:
             return torch.empty(0, self.vocab_size, dtype=torch.float32, device=self.device)
         self._validate(entries)
         self.reserve(entries)
+        if self._graph_buckets and len(entries) <= self._graph_buckets[-1] \
+                and all(len(e.tokens) == 1 for e in entries):
+            return self._step_graph(entries)
         with torch.cuda.device(self.device):
             batch = build_step_batch(entries, self.cache, self.device)
             ctx = StepContext(self.ops, self.act_dtype, batch, self.max_model_len, self._calls, self.cache)
@@ -141,3 +148,25 @@ class ModelRunner:
         for e in entries:
             self.cache.commit(e.req, len(e.tokens))
         return logits
+
+    def _step_graph(self, entries) -> torch.Tensor:
+        """A decode-only step through the HIP graph of its batch size bucket.
+        The logits live in a tensor the next such step overwrites."""
+        R = len(entries)
+        bucket = next(b for b in self._graph_buckets if b >= R)
+        with torch.cuda.device(self.device):
+            g = self._graphs.get(bucket)
+            if g is None:
+                g = self._graphs[bucket] = DecodeGraph(self, bucket)
+                g.capture()
+            logits = g.run(entries)
+            rows = [r for r, e in enumerate(entries) if e.want]
+            if len(rows) == R:
+                out = logits[:R]
+            elif rows:
+                out = logits[torch.tensor(rows, device=self.device)]
+            else:
+                out = logits[:0]
+        for e in entries:
+            self.cache.commit(e.req, 1)
+        return out

@@ -240,9 +240,9 @@ def _attention_work(batch, G: int, cols: int, device) -> torch.Tensor:
 
 def pick_splits(waves: int, max_context: int) -> int:
     """Into how many runs the keys of a decoding request are split so that
-    the launch has enough waves to pull on all of HBM: about 2048 waves, at
-    least 64 keys per run."""
-    return max(1, min(-(-2048 // max(1, waves)), -(-max_context // 64), 256))
+    the launch has enough waves to pull on all of HBM: about 1024 waves, at
+    least 128 keys per run."""
+    return max(1, min(-(-1024 // max(1, waves)), -(-max_context // 128), 256))
 
 
 def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,

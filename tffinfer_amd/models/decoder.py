@@ -106,6 +106,14 @@ class DecoderModel:
                     ws[local] = t if spec.init == "norm" else t.to(torch.bfloat16)
                 part.load_weights(ws, dtype, self.device)
 
+    def graph_safe(self) -> bool:
+        """True if every part launches only kernels that read the step's sizes
+        from device tables, so a decode step can be captured in a HIP graph."""
+        parts = [p for _, p in self._weighted_parts()]
+        for block in self.blocks:
+            parts.extend(p for _, p in _leaves("", block, {}))
+        return all(getattr(p, "graph_safe", False) for p in parts)
+
     # ---- cache needs -----------------------------------------------------
     def call_requirements(self):
         """For every entry of the run order: (cache id, writes, KVCacheSpec or

@@ -26,6 +26,8 @@ class GQAttention(Mixer):
     load; the reference keeps three products (QWen3Creator.cpp:66-75).
     """
 
+    graph_safe = True
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position, qk_norm_eps: float | None = 1e-6, window: int = 0,
                  scale: float | None = None):

@@ -50,6 +50,11 @@ class StateSpec:
 
 
 class Part:
+    #: True if ``forward`` launches only kernels that take the step's sizes from
+    #: device tables (no host loop over the step's entries), so that a decode step
+    #: with this part can be captured in a HIP graph and replayed.
+    graph_safe = False
+
     def weight_specs(self) -> dict[str, WeightSpec]:
         return {}
 

@@ -15,6 +15,8 @@ class PreNormBlock(Block):
     block's first norm (or the model's final norm) adds.
     """
 
+    graph_safe = True
+
     def __init__(self, mixer, feed_forward, make_norm):
         self.norm1 = make_norm()
         self.mixer = mixer

@@ -10,6 +10,8 @@ class Embedding(Part):
     """x[t, :] = E[token[t], :], no scaling, into the float32 residual stream.
     Reference: src/kernel/cpu/embedding.cpp:34-49 (a CPU lookup there)."""
 
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
@@ -29,6 +31,8 @@ class OutputHead(Part):
     """logits = y . Wout^T in float32, no bias, no scale
     (src/core/model/qwen3/QWen3Creator.cpp:161-165, :324-329).  With tied
     embeddings the head has no tensor of its own and uses the embedding's."""
+
+    graph_safe = True
 
     def __init__(self, vocab_size: int, hidden_size: int, tied_to: Embedding | None):
         self.vocab_size = int(vocab_size)

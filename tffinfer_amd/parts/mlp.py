@@ -16,6 +16,8 @@ class SwiGLU(FeedForward):
     streams both; the activation reads the two halves of its rows.
     """
 
+    graph_safe = True
+
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)

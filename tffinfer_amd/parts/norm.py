@@ -13,6 +13,8 @@ class RMSNorm(Norm):
     products in float32.  Reference: src/kernel/cuda/norm.cu:31-48 (the weight
     product fused as in src/core/runtime/GraphOptimizer.cpp:197-229)."""
 
+    graph_safe = True
+
     def __init__(self, size: int, eps: float):
         self.size = int(size)
         self.eps = float(eps)
