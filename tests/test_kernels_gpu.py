@@ -15,6 +15,12 @@ def _ops():
     return ops
 
 
+def _w(w):
+    """A weight as ops.linear takes it: row-major float32, fragment order bfloat16."""
+    w = w.to(DEV)
+    return _ops().pack_weight(w) if w.dtype == torch.bfloat16 else w
+
+
 def _close(got, ref, tol, what=""):
     got, ref = got.double().cpu(), ref.double().cpu()
     err = float((got - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
@@ -84,15 +90,15 @@ def test_linear(M, N, K, dtype):
     x = torch.randn(M, K, generator=g).to(dtype)
     w = (torch.randn(N, K, generator=g) * 0.1).to(dtype)
     ref = x.double() @ w.double().T
-    out = ops.linear(x.to(DEV), w.to(DEV), out_dtype=torch.float32)
+    out = ops.linear(x.to(DEV), _w(w), out_dtype=torch.float32)
     _close(out, ref, 2e-6 if dtype == torch.float32 else 2e-5, f"linear {M}x{N}x{K} f32 out")
     if dtype == torch.bfloat16:
-        out_b = ops.linear(x.to(DEV), w.to(DEV))
+        out_b = ops.linear(x.to(DEV), _w(w))
         assert out_b.dtype == torch.bfloat16
         _close(out_b, ref, 6e-3, "linear bf16 out")
     # strided rows (a slice of a wider matrix)
     wide = torch.randn(M, K + 16, generator=g).to(dtype).to(DEV)
-    out_s = ops.linear(wide[:, :K], w.to(DEV), out_dtype=torch.float32)
+    out_s = ops.linear(wide[:, :K], _w(w), out_dtype=torch.float32)
     _close(out_s, wide[:, :K].double().cpu() @ w.double().T, 2e-6 if dtype == torch.float32 else 2e-5, "strided")
 
 
@@ -113,7 +119,29 @@ def test_linear_refuses_bad_inner_size():
     x = torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV)
     w = torch.zeros(8, 12, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(KernelError, match="multiple of 8"):
-        ops.linear(x, w)
+        ops.pack_weight(w)
+    with pytest.raises(KernelError, match="PackedWeight"):
+        ops.linear(torch.zeros(4, 16, dtype=torch.bfloat16, device=DEV),
+                   torch.zeros(8, 16, dtype=torch.bfloat16, device=DEV))
+
+
+@pytest.mark.parametrize("N,K", [(16, 32), (5, 8), (320, 96), (200, 200), (33, 1000)])
+def test_pack_weight_round_trip_and_embedding(N, K):
+    """Fragment order: element (n, k) at ((n/16) * KB + k/32) * 512 + ((k%32)/8 * 16 + n%16) * 8 + k%8."""
+    ops = _ops()
+    w = torch.randn(N, K).to(torch.bfloat16)
+    pw = ops.pack_weight(w.to(DEV))
+    assert pw.shape == (N, K)
+    assert torch.equal(pw.unpack().cpu(), w)
+    flat = pw.data.cpu()
+    KB = -(-K // 32)
+    for n, k in ((0, 0), (N - 1, K - 1), (N // 2, K // 3), (min(N - 1, 17), min(K - 1, 41))):
+        off = ((n // 16) * KB + k // 32) * 512 + (((k % 32) // 8) * 16 + n % 16) * 8 + k % 8
+        assert flat[off] == w[n, k]
+    assert float(flat.float().abs().sum()) == float(w.float().abs().sum())   # the padding is zero
+    ids = torch.tensor([0, N - 1, N // 2], dtype=torch.int32)
+    out = ops.embed(pw, ids.to(DEV))
+    assert torch.equal(out.cpu(), w.float()[ids.long()])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -3,115 +3,157 @@
 // SIMT products (src/kernel/cuda/quant/quant_q_8_0_mat_mul.cu:338-447,
 // src/kernel/cuda/mat_mul.cu:149-518) with a design for 64-wide waves.
 //
-// Both operands are stored with k contiguous ([M, K] and [N, K]), which is the
-// layout an MFMA lane wants: lane l feeds 8 consecutive k of row (l % 16) at
-// k-chunk (l / 16).  The W tile is the MFMA's first operand, so a lane ends up
-// with 4 consecutive output columns of one row and stores them as one vector.
+// Weights are kept in *fragment order*: W [N, K] is cut into tiles of 16 rows
+// by 32 k, and each tile is stored as the 1 KB an MFMA operand is, lane after
+// lane: element (n, k) lies at
+//     ((n / 16) * (Kp / 32) + k / 32) * 512 + (((k % 32) / 8) * 16 + n % 16) * 8 + k % 8
+// with N and K padded to multiples of 16 and 32 by zeros.  A wave fetches an
+// operand with one fully contiguous 1 KB load (measured: a quarter more of
+// the HBM bandwidth than 16 rows x 64 bytes of a row-major matrix), and a tile
+// staged in LDS in the same order is read back without bank conflicts.
+// Activations A [M, K] stay row-major.  The W tile is the MFMA's first operand,
+// so a lane ends up with 4 consecutive output columns of one row.
 #include "common.h"
 #include "tffinfer_kernels.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
-#define G_BM 128
-#define G_BN 128
-#define G_BK 64
-#define G_LD (G_BK + 8)  // LDS row stride in elements; 144 bytes keeps 16-byte reads aligned and spreads banks
-
 __device__ __forceinline__ uint4 ld16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ bf16x8 as_frag(const uint4& v) { return *reinterpret_cast<const bf16x8*>(&v); }
 
 template <typename TC>
+__device__ __forceinline__ void store4(TC* dst, const floatx4& v, int n, int N, bool vec) {
+    if (vec) {  // n % 4 == 0 and N % 4 == 0: the four columns exist
+        if constexpr (sizeof(TC) == 4) {
+            *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+            union { bf16_t h[4]; uint2 u; } pk;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pk.h[e] = (bf16_t)v[e];
+            *reinterpret_cast<uint2*>(dst) = pk.u;
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (n + e < N) dst[e] = from_f32<TC>(v[e]);
+    }
+}
+
+// ------------------------------------------------------------------ tiled ---
+// Block tile (WTM*32) x (WTN*32) x 64 with 4 waves in 2 x 2, each wave
+// WTM x WTN MFMA tiles.  Both operands go global -> registers -> LDS in
+// fragment order (linear 16-byte stores), double buffered; a wave reads a
+// fragment back as one linear 1 KB.  The padding of W to 32 k holds zeros, so
+// k past the end of A only has to be readable: what it multiplies is zero.
+template <int WTM, int WTN, typename TC>
 __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __restrict__ A,
-                                                               const bf16_t* __restrict__ W,
+                                                               const bf16_t* __restrict__ Wp,
                                                                TC* __restrict__ C, int M, int N,
-                                                               int K, int lda) {
-    __shared__ __attribute__((aligned(16))) bf16_t As[2][G_BM * G_LD];
-    __shared__ __attribute__((aligned(16))) bf16_t Ws[2][G_BN * G_LD];
+                                                               int K, int lda, int KB) {
+    constexpr int BM = WTM * 32, BN = WTN * 32;
+    constexpr int AF = BM / 16 * 2, WF = BN / 16 * 2;   // fragments per operand tile (2 k-steps)
+    constexpr int AL = AF / 4, WL = WF / 4;             // 16-byte loads per thread and operand
+    __shared__ __attribute__((aligned(16))) bf16_t As[2][AF * 512];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[2][WF * 512];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * G_BM, n0 = blockIdx.x * G_BN;
     const int fr = lane & 15, fg = lane >> 4;
+    // blocks that run at the same time differ in m first: they share their W tiles out of L2
+    const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+    const int NB = (N + 15) / 16;
 
-    floatx4 acc[4][4];  // [n subtile][m subtile]
+    floatx4 acc[WTN][WTM];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < WTN; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < WTM; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    uint4 ra[4], rw[4];
-    const uint4 zero = make_uint4(0, 0, 0, 0);
-    auto load_global = [&](int k0) {
+    // a thread's share of a tile: fragments f = wave + 4 j (f = row group * 2 + k-step), this
+    // lane's 16 bytes of each
+    const bf16_t* a_src[AL];
+    int a_koff[AL];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int c = tid + 256 * j;       // 1024 chunks of 8 elements per operand tile
-            const int row = c >> 3, kc = (c & 7) * 8;
-            const int k = k0 + kc;
-            const int am = m0 + row, wr = n0 + row;
-            ra[j] = (am < M && k < K) ? ld16(A + (size_t)am * lda + k) : zero;
-            rw[j] = (wr < N && k < K) ? ld16(W + (size_t)wr * K + k) : zero;
-        }
-    };
-    auto store_lds = [&](int buf) {
+    for (int j = 0; j < AL; ++j) {
+        const int f = wave + 4 * j;
+        const int row = min(m0 + (f >> 1) * 16 + fr, M - 1);   // rows past the end repeat the last
+        a_koff[j] = (f & 1) * 32 + fg * 8;
+        a_src[j] = A + (size_t)row * lda;
+    }
+    const bf16_t* w_src[WL];
+    int w_ks[WL];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int c = tid + 256 * j;
-            const int row = c >> 3, kc = (c & 7) * 8;
-            *reinterpret_cast<uint4*>(&As[buf][row * G_LD + kc]) = ra[j];
-            *reinterpret_cast<uint4*>(&Ws[buf][row * G_LD + kc]) = rw[j];
-        }
-    };
+    for (int j = 0; j < WL; ++j) {
+        const int f = wave + 4 * j;
+        const int nb = min(n0 / 16 + (f >> 1), NB - 1);
+        w_ks[j] = f & 1;
+        w_src[j] = Wp + (size_t)nb * KB * 512 + lane * 8;
+    }
+    uint4 ra[AL], rw[WL];
+    const int nk = (K + 63) / 64;
 
-    const int nk = (K + G_BK - 1) / G_BK;
-    load_global(0);
-    store_lds(0);
+#define TFF_LOAD_TILE(kt)                                                                          \
+    {                                                                                              \
+        const int k0_ = (kt) * 64;                                                                 \
+        if (k0_ + 64 <= K) {                                                                       \
+            _Pragma("unroll") for (int j = 0; j < AL; ++j) ra[j] = ld16(a_src[j] + k0_ + a_koff[j]); \
+            _Pragma("unroll") for (int j = 0; j < WL; ++j)                                         \
+                rw[j] = ld16(w_src[j] + (size_t)(2 * (kt) + w_ks[j]) * 512);                       \
+        } else { /* the last, partial tile: clamp what does not exist */                           \
+            _Pragma("unroll") for (int j = 0; j < AL; ++j)                                         \
+                ra[j] = ld16(a_src[j] + min(k0_ + a_koff[j], K - 8));                              \
+            _Pragma("unroll") for (int j = 0; j < WL; ++j) {                                       \
+                const int ks_ = 2 * (kt) + w_ks[j];                                                \
+                const uint4 v_ = ld16(w_src[j] + (size_t)min(ks_, KB - 1) * 512);                  \
+                rw[j] = ks_ < KB ? v_ : make_uint4(0, 0, 0, 0);                                    \
+            }                                                                                      \
+        }                                                                                          \
+    }
+#define TFF_STORE_LDS(buf)                                                                         \
+    {                                                                                              \
+        _Pragma("unroll") for (int j = 0; j < AL; ++j)                                             \
+            *reinterpret_cast<uint4*>(&As[buf][(wave + 4 * j) * 512 + lane * 8]) = ra[j];          \
+        _Pragma("unroll") for (int j = 0; j < WL; ++j)                                             \
+            *reinterpret_cast<uint4*>(&Ws[buf][(wave + 4 * j) * 512 + lane * 8]) = rw[j];          \
+    }
+
+    TFF_LOAD_TILE(0)
+    TFF_STORE_LDS(0)
     __syncthreads();
     for (int kt = 0; kt < nk; ++kt) {
         const int buf = kt & 1;
-        if (kt + 1 < nk) load_global((kt + 1) * G_BK);
+        if (kt + 1 < nk) TFF_LOAD_TILE(kt + 1)
 #pragma unroll
-        for (int ks = 0; ks < G_BK; ks += 32) {
-            bf16x8 fw[4], fa[4];
+        for (int ks = 0; ks < 2; ++ks) {
+            bf16x8 fw[WTN], fa[WTM];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                fw[i] = *reinterpret_cast<const bf16x8*>(&Ws[buf][(wn * 64 + i * 16 + fr) * G_LD + ks + fg * 8]);
-                fa[i] = *reinterpret_cast<const bf16x8*>(&As[buf][(wm * 64 + i * 16 + fr) * G_LD + ks + fg * 8]);
-            }
+            for (int i = 0; i < WTN; ++i)
+                fw[i] = *reinterpret_cast<const bf16x8*>(&Ws[buf][((wn * WTN + i) * 2 + ks) * 512 + lane * 8]);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int j = 0; j < WTM; ++j)
+                fa[j] = *reinterpret_cast<const bf16x8*>(&As[buf][((wm * WTM + j) * 2 + ks) * 512 + lane * 8]);
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+            for (int i = 0; i < WTN; ++i)
+#pragma unroll
+                for (int j = 0; j < WTM; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[i], fa[j], acc[i][j], 0, 0, 0);
         }
-        if (kt + 1 < nk) store_lds(buf ^ 1);
+        if (kt + 1 < nk) TFF_STORE_LDS(buf ^ 1)
         __syncthreads();
     }
+#undef TFF_LOAD_TILE
+#undef TFF_STORE_LDS
 
-    // lane holds C[m][n .. n+3], n = n0 + wn*64 + i*16 + fg*4, m = m0 + wm*64 + j*16 + fr
+    // lane holds C[m][n .. n+3], n = n0 + (wn*WTN + i)*16 + fg*4, m = m0 + (wm*WTM + j)*16 + fr
     const bool vec = (N % 4) == 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int n = n0 + wn * 64 + i * 16 + fg * 4;
+    for (int i = 0; i < WTN; ++i) {
+        const int n = n0 + (wn * WTN + i) * 16 + fg * 4;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int m = m0 + wm * 64 + j * 16 + fr;
-            if (m >= M || n >= N) continue;
-            TC* dst = C + (size_t)m * N + n;
-            if (vec) {  // n % 4 == 0 and N % 4 == 0: the four columns exist
-                if constexpr (sizeof(TC) == 4) {
-                    *reinterpret_cast<float4*>(dst) =
-                        make_float4(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
-                } else {
-                    union { bf16_t h[4]; uint2 u; } pk;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) pk.h[e] = (bf16_t)acc[i][j][e];
-                    *reinterpret_cast<uint2*>(dst) = pk.u;
-                }
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (n + e < N) dst[e] = from_f32<TC>(acc[i][j][e]);
-            }
+        for (int j = 0; j < WTM; ++j) {
+            const int m = m0 + (wm * WTM + j) * 16 + fr;
+            if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, acc[i][j], n, N, vec);
         }
     }
 }
@@ -120,23 +162,21 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
 // For a few rows of A (decoding: M = number of live requests) the product is
 // a stream of W from HBM; what counts is bytes in flight, not LDS tiling.
 // A block owns a slab of 16*R rows of W for the whole of K; its waves split K
-// among them in contiguous runs, each wave reading W straight from global
-// memory into MFMA operands (16 rows x 64 contiguous bytes per load) and the
-// few rows of A from cache; partial sums meet in LDS and are added in a fixed
-// order, so no partial result goes through global memory and the result does
-// not depend on the launch.
-#define SK_WAVES 8
-
-// UNROLL k-steps of loads are issued before the first is used: a wave keeps
-// UNROLL * (R + MT) KB in flight, which is what hides the latency of HBM.
-template <int MT, int R, int UNROLL, typename TC>
+// among them in contiguous runs, each wave reading its W fragments straight
+// from global memory into MFMA operands and the few rows of A from cache;
+// partial sums meet in LDS and are added in a fixed order, so no partial
+// result goes through global memory and the result does not depend on the
+// launch.  UNROLL k-steps of loads are issued before the first is used: a wave
+// keeps UNROLL * (R + MT) KB in flight, which is what hides the latency of HBM.
+template <int MT, int R, int UNROLL, int SK_WAVES, typename TC>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_bf16_skinny_kernel(
-    const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, TC* __restrict__ C, int M, int N,
-    int K, int lda) {
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
+    int K, int lda, int KB) {
     __shared__ floatx4 part[SK_WAVES - 1][R * MT][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int fr = lane & 15, fg = lane >> 4;
-    const int n0 = blockIdx.x * (16 * R);
+    const int NB = (N + 15) / 16;
+    const int nb0 = blockIdx.x * R;
 
     floatx4 acc[R][MT];
 #pragma unroll
@@ -145,38 +185,29 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_bf16_skinny_kernel(
         for (int t = 0; t < MT; ++t) acc[r][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     // k-steps of 32 are dealt out to the waves in contiguous runs
-    const int nsteps = (K + 31) / 32;
-    const int per = (nsteps + SK_WAVES - 1) / SK_WAVES;
+    const int per = (KB + SK_WAVES - 1) / SK_WAVES;
     const int s_begin = wave * per;
-    const int s_end = min(nsteps, s_begin + per);
+    const int s_end = min(KB, s_begin + per);
 
-    const bf16_t* wrow[R];
-    bool wok[R];
+    // Row groups past the end of W and rows past the end of A repeat the last: their results
+    // are never stored, and no load of the main loop carries a predicate.
+    const bf16_t* wfrag[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int n = n0 + r * 16 + fr;
-        wok[r] = n < N;
-        wrow[r] = W + (size_t)(wok[r] ? n : 0) * K;
-    }
+    for (int r = 0; r < R; ++r) wfrag[r] = Wp + (size_t)min(nb0 + r, NB - 1) * KB * 512 + lane * 8;
     const bf16_t* arow[MT];
-    bool aok[MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        const int m = t * 16 + fr;
-        aok[t] = m < M;
-        arow[t] = A + (size_t)(aok[t] ? m : 0) * lda;
-    }
-    const uint4 zero = make_uint4(0, 0, 0, 0);
-    for (int s0 = s_begin; s0 < s_end; s0 += UNROLL) {
+    for (int t = 0; t < MT; ++t) arow[t] = A + (size_t)min(t * 16 + fr, M - 1) * lda;
+
+    const int full_end = min(s_end, K / 32);   // steps below K / 32 have all their 32 k in A
+    int s0 = s_begin;
+    for (; s0 + UNROLL <= full_end; s0 += UNROLL) {
         uint4 rw[UNROLL][R], ra[UNROLL][MT];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            const int k = (s0 + u) * 32 + fg * 8;
-            const bool kok = (s0 + u) < s_end && k < K;
 #pragma unroll
-            for (int r = 0; r < R; ++r) rw[u][r] = (kok && wok[r]) ? ld16(wrow[r] + k) : zero;
+            for (int r = 0; r < R; ++r) rw[u][r] = ld16(wfrag[r] + (size_t)(s0 + u) * 512);
 #pragma unroll
-            for (int t = 0; t < MT; ++t) ra[u][t] = (kok && aok[t]) ? ld16(arow[t] + k) : zero;
+            for (int t = 0; t < MT; ++t) ra[u][t] = ld16(arow[t] + (s0 + u) * 32 + fg * 8);
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
@@ -184,9 +215,26 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_bf16_skinny_kernel(
             for (int r = 0; r < R; ++r)
 #pragma unroll
                 for (int t = 0; t < MT; ++t)
-                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        *reinterpret_cast<bf16x8*>(&rw[u][r]), *reinterpret_cast<bf16x8*>(&ra[u][t]),
-                        acc[r][t], 0, 0, 0);
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(rw[u][r]), as_frag(ra[u][t]),
+                                                                        acc[r][t], 0, 0, 0);
+    }
+    // what is left, a step at a time; in the last step of K some k may not exist in A
+    for (; s0 < s_end; ++s0) {
+        const int k = s0 * 32 + fg * 8;
+        const bool kok = k < K;
+        uint4 rw[R], ra[MT];
+#pragma unroll
+        for (int r = 0; r < R; ++r) rw[r] = ld16(wfrag[r] + (size_t)s0 * 512);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const uint4 v = ld16(arow[t] + (kok ? k : 0));
+            ra[t] = kok ? v : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(rw[r]), as_frag(ra[t]), acc[r][t], 0, 0, 0);
     }
     if (wave > 0) {
 #pragma unroll
@@ -207,83 +255,136 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_bf16_skinny_kernel(
                     const floatx4 p = part[w][r * MT + t][lane];
                     v[0] += p[0]; v[1] += p[1]; v[2] += p[2]; v[3] += p[3];
                 }
-                const int n = n0 + r * 16 + fg * 4;
+                const int n = (nb0 + r) * 16 + fg * 4;
                 const int m = t * 16 + fr;
-                if (m >= M || n >= N) continue;
-                TC* dst = C + (size_t)m * N + n;
-                if (vec) {
-                    if constexpr (sizeof(TC) == 4) {
-                        *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
-                    } else {
-                        union { bf16_t h[4]; uint2 u; } pk;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) pk.h[e] = (bf16_t)v[e];
-                        *reinterpret_cast<uint2*>(dst) = pk.u;
-                    }
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (n + e < N) dst[e] = from_f32<TC>(v[e]);
-                }
+                if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, v, n, N, vec);
             }
     }
 }
 
-template <int MT, int R, int UNROLL>
-static int launch_skinny(const bf16_t* A, const bf16_t* W, void* C, int M, int N, int K, int lda,
+template <int MT, int R, int UNROLL, int SK_WAVES>
+static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
                          int c_dtype, hipStream_t s) {
-    const dim3 grid((N + 16 * R - 1) / (16 * R));
+    const int NB = (N + 15) / 16, KB = (K + 31) / 32;
+    const dim3 grid((NB + R - 1) / R);
     if (c_dtype == TFF_F32)
-        gemm_bf16_skinny_kernel<MT, R, UNROLL, float><<<grid, 64 * SK_WAVES, 0, s>>>(A, W, (float*)C, M, N, K, lda);
+        gemm_bf16_skinny_kernel<MT, R, UNROLL, SK_WAVES, float><<<grid, 64 * SK_WAVES, 0, s>>>(
+            A, Wp, (float*)C, M, N, K, lda, KB);
     else
-        gemm_bf16_skinny_kernel<MT, R, UNROLL, bf16_t><<<grid, 64 * SK_WAVES, 0, s>>>(A, W, (bf16_t*)C, M, N, K, lda);
+        gemm_bf16_skinny_kernel<MT, R, UNROLL, SK_WAVES, bf16_t><<<grid, 64 * SK_WAVES, 0, s>>>(
+            A, Wp, (bf16_t*)C, M, N, K, lda, KB);
     return tff_check_launch("gemm_bf16_skinny");
 }
 
-int tff_gemm_bf16(const bf16_t* A, const bf16_t* W, void* C, int M, int N, int K, int lda,
+template <int WTM, int WTN>
+static int launch_tiled(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
+                        int c_dtype, hipStream_t s) {
+    const int KB = (K + 31) / 32;
+    const dim3 grid((M + WTM * 32 - 1) / (WTM * 32), (N + WTN * 32 - 1) / (WTN * 32));
+    TFF_REQUIRE(grid.y <= 65535, "gemm: too many columns N=%d", N);
+    if (c_dtype == TFF_F32)
+        gemm_bf16_tiled_kernel<WTM, WTN, float><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB);
+    else
+        gemm_bf16_tiled_kernel<WTM, WTN, bf16_t><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB);
+    return tff_check_launch("gemm_bf16_tiled");
+}
+
+int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
                   int c_dtype, hipStream_t s) {
     TFF_REQUIRE(K % 8 == 0 && lda % 8 == 0,
                 "gemm: the bfloat16 product needs the inner size (K=%d, row stride %d) to be a multiple of 8",
                 K, lda);
-    TFF_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)C % 16) == 0,
+    TFF_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)Wp % 16) == 0 && ((uintptr_t)C % 16) == 0,
                 "gemm: operands must be 16-byte aligned");
     TFF_REQUIRE(c_dtype == TFF_F32 || c_dtype == TFF_BF16, "gemm: unknown output type %d", c_dtype);
-    if (M <= 64) {
-        // slabs of 32 rows when that still gives every CU several blocks, else of 16
-        const bool wide = N >= 32 * 1024;
-        const int mt = (M + 15) / 16;
-        switch (mt * 2 + (wide ? 1 : 0)) {
-            case 2: return launch_skinny<1, 1, 16>(A, W, C, M, N, K, lda, c_dtype, s);
-            case 3: return launch_skinny<1, 2, 8>(A, W, C, M, N, K, lda, c_dtype, s);
-            case 4: return launch_skinny<2, 1, 8>(A, W, C, M, N, K, lda, c_dtype, s);
-            case 5: return launch_skinny<2, 2, 6>(A, W, C, M, N, K, lda, c_dtype, s);
-            case 6: return launch_skinny<3, 1, 6>(A, W, C, M, N, K, lda, c_dtype, s);
-            case 7: return launch_skinny<3, 2, 4>(A, W, C, M, N, K, lda, c_dtype, s);
-            case 8: return launch_skinny<4, 1, 6>(A, W, C, M, N, K, lda, c_dtype, s);
-            default: return launch_skinny<4, 2, 4>(A, W, C, M, N, K, lda, c_dtype, s);
-        }
+    if (M <= 16) {
+        // more waves per block where there are few blocks (small N) or long rows (large K)
+        if (N >= 32 * 1024) return launch_skinny<1, 1, 16, 8>(A, Wp, C, M, N, K, lda, c_dtype, s);
+        if (K >= 8192 || N <= 8192) return launch_skinny<1, 1, 8, 16>(A, Wp, C, M, N, K, lda, c_dtype, s);
+        return launch_skinny<1, 1, 16, 8>(A, Wp, C, M, N, K, lda, c_dtype, s);
     }
-    dim3 grid((N + G_BN - 1) / G_BN, (M + G_BM - 1) / G_BM);
-    TFF_REQUIRE(grid.y <= 65535, "gemm: too many rows M=%d", M);
-    if (c_dtype == TFF_F32)
-        gemm_bf16_tiled_kernel<float><<<grid, 256, 0, s>>>(A, W, (float*)C, M, N, K, lda);
-    else if (c_dtype == TFF_BF16)
-        gemm_bf16_tiled_kernel<bf16_t><<<grid, 256, 0, s>>>(A, W, (bf16_t*)C, M, N, K, lda);
-    else
-        return tff_fail("gemm: unknown output type %d", c_dtype);
-    return tff_check_launch("gemm_bf16");
+    if (M <= 32) return launch_skinny<2, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, s);
+    if (M <= 64) {
+        if (N >= 16 * 1024) return launch_skinny<4, 4, 4, 4>(A, Wp, C, M, N, K, lda, c_dtype, s);
+        return launch_skinny<4, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, s);
+    }
+    return launch_tiled<4, 4>(A, Wp, C, M, N, K, lda, c_dtype, s);
 }
 
 int tff_gemm_f32(const float* A, const float* W, void* C, int M, int N, int K, int lda,
                  int c_dtype, hipStream_t s);
 
 TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda,
-                     int ab_dtype, int c_dtype, tff_stream_t stream) {
+                     int ab_dtype, int c_dtype, int w_packed, tff_stream_t stream) {
     TFF_REQUIRE(A && W && C, "gemm: null pointer");
     TFF_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K, "gemm: bad sizes M=%d N=%d K=%d lda=%d", M, N, K, lda);
     if (M == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    if (ab_dtype == TFF_F32) return tff_gemm_f32((const float*)A, (const float*)W, C, M, N, K, lda, c_dtype, s);
-    if (ab_dtype == TFF_BF16) return tff_gemm_bf16((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, c_dtype, s);
+    if (ab_dtype == TFF_F32) {
+        TFF_REQUIRE(!w_packed, "gemm: the float32 product takes a row-major weight");
+        return tff_gemm_f32((const float*)A, (const float*)W, C, M, N, K, lda, c_dtype, s);
+    }
+    if (ab_dtype == TFF_BF16) {
+        TFF_REQUIRE(w_packed, "gemm: the bfloat16 product takes a weight in fragment order");
+        return tff_gemm_bf16((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, c_dtype, s);
+    }
     return tff_fail("gemm: unknown operand type %d", ab_dtype);
+}
+
+// ------------------------------------------------------------- packing ---
+// Row-major [N, K] -> fragment order, with zero padding to 16 rows and 32 k.
+__global__ void pack_weight_kernel(const bf16_t* __restrict__ src, bf16_t* __restrict__ dst, int N,
+                                   int K, int KB, size_t total_chunks) {
+    // one thread per 16-byte chunk of the packed matrix
+    const size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= total_chunks) return;
+    const int l = (int)(c & 63);
+    const size_t frag = c >> 6;
+    const int kb = (int)(frag % KB);
+    const int nb = (int)(frag / KB);
+    const int n = nb * 16 + (l & 15);
+    const int k = kb * 32 + (l >> 4) * 8;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (n < N && k < K) v = *reinterpret_cast<const uint4*>(src + (size_t)n * K + k);   // K % 8 == 0
+    *reinterpret_cast<uint4*>(dst + c * 8) = v;
+}
+
+TFF_API int tff_pack_weight(const void* src, void* dst, int N, int K, tff_stream_t stream) {
+    TFF_REQUIRE(src && dst, "pack_weight: null pointer");
+    TFF_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "pack_weight: inner size %d must be a multiple of 8", K);
+    const int NB = (N + 15) / 16, KB = (K + 31) / 32;
+    const size_t chunks = (size_t)NB * KB * 64;
+    const size_t blocks = (chunks + 255) / 256;
+    TFF_REQUIRE(blocks < 2147483647ULL, "pack_weight: matrix too large");
+    pack_weight_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const bf16_t*)src, (bf16_t*)dst, N, K,
+                                                                           KB, chunks);
+    return tff_check_launch("pack_weight");
+}
+
+// Gather of rows out of a matrix in fragment order (the embedding of a model whose
+// output head shares the table): out[t, :] = float(E[ids[t], :]).
+__global__ void embed_packed_kernel(const bf16_t* __restrict__ table, const int32_t* __restrict__ ids,
+                                    float* __restrict__ out, int H, int V, int KB) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    const bool bad = id < 0 || id >= V;
+    if (bad) id = 0;
+    const bf16_t* base = table + (size_t)(id / 16) * KB * 512 + (id % 16) * 8;
+    float* o = out + (size_t)t * H;
+    for (int c = threadIdx.x; c < H / 8; c += blockDim.x) {   // chunk c holds k = 8c .. 8c+7
+        const bf16_t* p = base + (size_t)(c / 4) * 512 + (c % 4) * 128;
+        union { uint4 u; bf16_t h[8]; } v;
+        v.u = *reinterpret_cast<const uint4*>(p);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[c * 8 + e] = bad ? __builtin_nanf("") : (float)v.h[e];
+    }
+}
+
+TFF_API int tff_embed_packed(const void* table, const int32_t* ids, float* out, int T, int H, int V,
+                             tff_stream_t stream) {
+    TFF_REQUIRE(table && ids && out, "embed: null pointer");
+    TFF_REQUIRE(T >= 0 && H > 0 && V > 0 && H % 8 == 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
+    if (T == 0) return 0;
+    embed_packed_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const bf16_t*)table, ids, out, H, V, (H + 31) / 32);
+    return tff_check_launch("embed_packed");
 }

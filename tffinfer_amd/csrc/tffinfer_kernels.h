@@ -31,11 +31,23 @@ TFF_API int tff_add_rmsnorm(float* resid, const float* delta, const float* weigh
 TFF_API int tff_rmsnorm(const void* x, const float* weight, float eps, void* out,
                         int n, int H, int dtype, tff_stream_t stream);
 
-// C[M, N] = A[M, K] . W[N, K]^T.  A has row stride lda (elements), W and C are
-// dense.  A and W are of ab_dtype; C is of c_dtype.  float32 runs on plain FMA
-// in a fixed summation order, bfloat16 on MFMA with float32 accumulation.
-TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K,
-                     int lda, int ab_dtype, int c_dtype, tff_stream_t stream);
+// C[M, N] = A[M, K] . W[N, K]^T.  A has row stride lda (elements), C is dense.
+// A and W are of ab_dtype; C is of c_dtype.  float32 runs on plain FMA in a
+// fixed summation order with a row-major W (w_packed = 0); bfloat16 runs on
+// MFMA with float32 accumulation and takes W in fragment order (w_packed = 1,
+// see tff_pack_weight).
+TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda,
+                     int ab_dtype, int c_dtype, int w_packed, tff_stream_t stream);
+
+// bfloat16 row-major [N, K] (K a multiple of 8) -> fragment order: tiles of
+// 16 rows x 32 k, each stored as the 1 KB operand of a 16x16x32 MFMA, element
+// (n, k) at ((n/16) * ceil(K/32) + k/32) * 512 + (((k%32)/8) * 16 + n%16) * 8 + k%8,
+// zero padded.  dst holds ceil(N/16) * ceil(K/32) * 512 elements.
+TFF_API int tff_pack_weight(const void* src, void* dst, int N, int K, tff_stream_t stream);
+
+// tff_embed for a table in fragment order.
+TFF_API int tff_embed_packed(const void* table, const int32_t* ids, float* out, int T, int H,
+                             int V, tff_stream_t stream);
 
 // Per (token, head) of a fused projection output qkv [T, (nq + 2 nkv) d]:
 // q and k heads get an RMS norm over d (q_weight / k_weight, skipped if null),
@@ -62,6 +74,25 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out,
                                   int T, int nq, int nkv, int d, int page_size, int num_pages,
                                   int window, float scale, int dtype, int cache_dtype,
                                   tff_stream_t stream);
+
+// bfloat16 attention on the matrix cores.  A wave works on `cols_per_wave` (16
+// or 32) columns of one request and kv head; a column is a (token, q head of
+// the group) pair numbered token * G + head.  work != null: pairs (request,
+// first column) per wave; work == null: every request brings one token and
+// gets tiles_per_entry waves.  splits > 1 cuts each request's keys into runs
+// whose partial results (part_o [splits, T, nq, d], part_ml [splits, T, nq, 2],
+// float32) tff_attention_split_reduce merges.  Head sizes 16..128 in steps of
+// 16, 192 and 256; pages a multiple of 8; values transposed in their pages.
+TFF_API int tff_attention_mfma_supported(int d, int page_size);
+TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* part_o, float* part_ml,
+                               const void* k_cache, const void* v_cache,
+                               const int32_t* block_tables, int bt_stride, const int32_t* cu_tokens,
+                               const int32_t* start_pos, const int32_t* work, int num_work,
+                               int tiles_per_entry, int cols_per_wave, int splits, int T_total,
+                               int nq, int nkv, int d, int page_size, int num_pages, int window,
+                               float scale, tff_stream_t stream);
+TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml, void* out,
+                                       int splits, int T_total, int nq, int d, tff_stream_t stream);
 
 // out[t, i] = silu(gu[t, i]) * gu[t, I + i]
 TFF_API int tff_swiglu(const void* gu, void* out, int T, int I, int dtype, tff_stream_t stream);

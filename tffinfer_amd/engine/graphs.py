@@ -15,6 +15,9 @@ lengths.
 """
 from __future__ import annotations
 
+import gc
+import weakref
+
 import numpy as np
 import torch
 
@@ -27,7 +30,7 @@ def _pad4(n: int) -> int:
 
 class DecodeGraph:
     def __init__(self, runner, bucket: int):
-        self.runner = runner
+        self._runner = weakref.ref(runner)   # the runner owns its graphs; no reference cycle
         self.B = B = int(bucket)
         cache = runner.cache
         ps = cache.page_size
@@ -75,6 +78,10 @@ class DecodeGraph:
         self.graph = None
         self.logits = None
         self._copied = torch.cuda.Event()
+
+    @property
+    def runner(self):
+        return self._runner()
 
     def _pad_rows(self, first: int) -> None:
         o, hv, B = self.offs, self.hv, self.B
@@ -138,14 +145,23 @@ class DecodeGraph:
         # (batch.max_context), so the launch is the same whatever the requests hold
         side = torch.cuda.Stream(device=rn.device)
         side.wait_stream(torch.cuda.current_stream(rn.device))
-        with torch.cuda.stream(side):
-            self.dev.copy_(self.host, non_blocking=True)
-            for _ in range(2):          # warm up: allocations, rotation tables
-                self._forward()
-            side.synchronize()
-            self.graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(self.graph, stream=side):
-                self.logits = self._forward()
+        # No collection of garbage may run while the stream records: the finaliser of an old
+        # graph or tensor would make a HIP call that is illegal during capture and abort.
+        gc.collect()
+        gc_was_on = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.stream(side):
+                self.dev.copy_(self.host, non_blocking=True)
+                for _ in range(2):          # warm up: allocations, rotation tables
+                    self._forward()
+                side.synchronize()
+                self.graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(self.graph, stream=side):
+                    self.logits = self._forward()
+        finally:
+            if gc_was_on:
+                gc.enable()
         torch.cuda.current_stream(rn.device).wait_stream(side)
         torch.cuda.synchronize(rn.device)
 

@@ -57,9 +57,58 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """Rows of ``table`` [V, H] for int32 ``ids`` [T] as float32 [T, H]."""
-    _req(table, "embed table", ndim=2)
+class PackedWeight:
+    """A bfloat16 matrix [N, K] in the fragment order of the matrix-core
+    products: tiles of 16 rows by 32 k stored as the 1 KB operand a wave loads,
+    rows and k padded with zeros to multiples of 16 and 32."""
+    __slots__ = ("data", "N", "K")
+
+    def __init__(self, data: torch.Tensor, N: int, K: int):
+        self.data, self.N, self.K = data, int(N), int(K)
+
+    @property
+    def shape(self):
+        return (self.N, self.K)
+
+    @property
+    def dtype(self):
+        return self.data.dtype
+
+    @property
+    def device(self):
+        return self.data.device
+
+    def data_ptr(self) -> int:
+        return self.data.data_ptr()
+
+    def unpack(self) -> torch.Tensor:
+        """Back to row-major [N, K] (for tests and inspection)."""
+        NB, KB = -(-self.N // 16), -(-self.K // 32)
+        t = self.data.view(NB, KB, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(NB * 16, KB * 32)
+        return t[:self.N, :self.K].contiguous()
+
+
+def pack_weight(w: torch.Tensor) -> PackedWeight:
+    """Row-major bfloat16 [N, K] on the GPU -> fragment order."""
+    _req(w, "pack_weight", torch.bfloat16, 2)
+    N, K = w.shape
+    if K % 8:
+        raise _lib.KernelError(f"pack_weight: inner size {K} must be a multiple of 8")
+    NB, KB = -(-N // 16), -(-K // 32)
+    out = torch.empty(NB * KB * 512, dtype=torch.bfloat16, device=w.device)
+    L = _lib.load()
+    _lib.check(L.tff_pack_weight(w.data_ptr(), out.data_ptr(), N, K, _stream()))
+    return PackedWeight(out, N, K)
+
+
+def embed(table, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Rows of ``table`` [V, H] (a row-major tensor or a PackedWeight) for
+    int32 ``ids`` [T] as float32 [T, H]."""
+    packed = isinstance(table, PackedWeight)
+    if packed:
+        _req(table.data, "embed table", torch.bfloat16, 1)
+    else:
+        _req(table, "embed table", ndim=2)
     _req(ids, "embed ids", torch.int32, 1)
     V, H = table.shape
     T = ids.numel()
@@ -70,8 +119,11 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = Non
         if tuple(out.shape) != (T, H):
             raise _lib.KernelError(f"embed out: shape {tuple(out.shape)} is not {(T, H)}")
     L = _lib.load()
-    _lib.check(L.tff_embed(table.data_ptr(), ids.data_ptr(), out.data_ptr(), T, H, V,
-                           dtype_code(table.dtype), _stream()))
+    if packed:
+        _lib.check(L.tff_embed_packed(table.data_ptr(), ids.data_ptr(), out.data_ptr(), T, H, V, _stream()))
+    else:
+        _lib.check(L.tff_embed(table.data_ptr(), ids.data_ptr(), out.data_ptr(), T, H, V,
+                               dtype_code(table.dtype), _stream()))
     return out
 
 
@@ -121,12 +173,19 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return out
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None = None,
+def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
            out: torch.Tensor | None = None) -> torch.Tensor:
-    """``x . weight^T`` for x [M, K] (rows may be strided) and weight [N, K]."""
+    """``x . weight^T`` for x [M, K] (rows may be strided) and weight [N, K]:
+    a row-major float32 tensor, or a PackedWeight for bfloat16."""
     if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
         raise _lib.KernelError("linear x: expected a GPU matrix with unit inner stride")
-    _req(weight, "linear weight", x.dtype, 2)
+    packed = isinstance(weight, PackedWeight)
+    if packed:
+        _req(weight.data, "linear weight", x.dtype, 1)
+    else:
+        _req(weight, "linear weight", x.dtype, 2)
+        if weight.dtype == torch.bfloat16:
+            raise _lib.KernelError("linear: a bfloat16 weight must be a PackedWeight (pack_weight)")
     M, K = x.shape
     N, K2 = weight.shape
     if K != K2:
@@ -143,7 +202,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None 
             raise _lib.KernelError(f"linear out: shape {tuple(out.shape)} is not {(M, N)}")
     L = _lib.load()
     _lib.check(L.tff_gemm(x.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K, lda,
-                          dtype_code(x.dtype), dtype_code(out_dtype), _stream()))
+                          dtype_code(x.dtype), dtype_code(out_dtype), 1 if packed else 0, _stream()))
     return out
 
 
@@ -385,6 +444,7 @@ OP_TABLE = {
     "add_rmsnorm": add_rmsnorm,
     "rmsnorm": rmsnorm,
     "linear": linear,
+    "pack_weight": pack_weight,
     "qk_norm_rope_kv": qk_norm_rope_kv,
     "attention": paged_attention,
     "attention_generic": attention_generic,

@@ -160,7 +160,13 @@ register_position_encoding = POSITION_ENCODINGS.register
 register_block = BLOCKS.register
 
 
-def to_device(t: torch.Tensor, dtype: torch.dtype, device) -> torch.Tensor:
-    """Host tensor to the device in ``dtype`` (the conversion runs on the host,
-    round-to-nearest-even for float32 -> bfloat16)."""
-    return t.to(dtype).contiguous().to(device)
+def to_device(t: torch.Tensor, dtype: torch.dtype, device):
+    """A matrix to the device in ``dtype`` (float32 -> bfloat16 rounds to
+    nearest even).  A bfloat16 matrix on a GPU is put into the fragment order
+    the matrix-core products read (``ops.PackedWeight``); float32 stays
+    row-major."""
+    out = t.to(dtype).contiguous().to(device)
+    if dtype == torch.bfloat16 and out.is_cuda and out.dim() == 2:
+        from ..kernels import ops
+        return ops.pack_weight(out)
+    return out
