@@ -448,3 +448,22 @@ def test_attention_mfma_far_key_and_window_edge():
             _close(out.reshape(n, nq, d), ref, 1.5e-2, f"n={n} window={window}")
             hit = torch.allclose(out.reshape(n, nq, d)[0, 0].float().cpu(), vs[0][far, 0].float(), atol=5e-2)
             assert hit == sees, f"n={n} window={window}: far key {'missed' if sees else 'seen'}"
+
+
+@pytest.mark.parametrize("M", [1, 8, 20, 50, 200])
+@pytest.mark.parametrize("I,K", [(200, 96), (64, 64), (1000, 256), (12288, 512)])
+def test_linear_with_gated_epilogue(M, I, K):
+    """Gate and up interleaved in one weight: the product yields silu(x Wg^T) * (x Wu^T)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(I + M)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    wg = (torch.randn(I, K, generator=g) * 0.2).to(torch.bfloat16)
+    wu = (torch.randn(I, K, generator=g) * 0.2).to(torch.bfloat16)
+    pw = ops.pack_gate_up(wg.to(DEV), wu.to(DEV))
+    assert pw.glu_out == I and pw.N == 2 * (-(-I // 16) * 16)
+    out = ops.linear(x.to(DEV), pw)
+    assert out.shape == (M, I) and out.dtype == torch.bfloat16
+    gt, up = x.double() @ wg.double().T, x.double() @ wu.double().T
+    _close(out, gt / (1 + torch.exp(-gt)) * up, 8e-3, "gated product")
+    out32 = ops.linear(x.to(DEV), pw, out_dtype=torch.float32)
+    _close(out32, gt / (1 + torch.exp(-gt)) * up, 3e-5, "gated product, float32 out")

@@ -29,7 +29,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 template <int DT, int NQT, bool SPLIT>
-__global__ __launch_bounds__(64) void attn_mfma_kernel(
+__global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int bt_stride,
@@ -107,52 +107,74 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
         for (int dt = 0; dt < DT; ++dt) oacc[t][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 
+    union VF { uint2 u[2]; bf16x8 v; };
+    bf16x8 kf[2][2][KS];   // [buffer][key tile][k-step]
+    VF vf[2][DT];
+
+#define TFF_ATTN_LOAD(buf, step)                                                                    \
+    {                                                                                               \
+        const int kb_ = kb0 + (step) * 32;                                                          \
+        _Pragma("unroll") for (int kt = 0; kt < 2; ++kt) {                                          \
+            /* rows past the last key repeat it; they are masked */                                 \
+            const int j_ = min(kb_ + kt * 16 + qc, kmax);                                           \
+            const int page_ = bt[j_ / page_size];                                                   \
+            const bf16_t* kp_ = k_cache + (((size_t)page_ * nkv + g) * page_size + (j_ % page_size)) * D; \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                     \
+                const int e_ = ks * 32 + kg * 8;                                                    \
+                uint4 v_ = make_uint4(0, 0, 0, 0);                                                  \
+                if (e_ < D) v_ = *reinterpret_cast<const uint4*>(kp_ + e_);                         \
+                kf[buf][kt][ks] = *reinterpret_cast<bf16x8*>(&v_);                                  \
+            }                                                                                       \
+        }                                                                                           \
+        /* value runs of this lane group: keys kb + g*4 .. +3 and kb + 16 + g*4 .. +3 */            \
+        const bf16_t* vrun_[2];                                                                     \
+        _Pragma("unroll") for (int kt = 0; kt < 2; ++kt) {                                          \
+            const int j0_ = min(kb_ + kt * 16 + kg * 4, (kmax / 4) * 4);                            \
+            const int page_ = bt[j0_ / page_size];                                                  \
+            vrun_[kt] = v_cache + ((size_t)page_ * nkv + g) * D * page_size + (j0_ % page_size);    \
+        }                                                                                           \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                         \
+            const size_t eoff_ = (size_t)(dt * 16 + qc) * page_size;                                \
+            vf[buf][dt].u[0] = *reinterpret_cast<const uint2*>(vrun_[0] + eoff_);                   \
+            vf[buf][dt].u[1] = *reinterpret_cast<const uint2*>(vrun_[1] + eoff_);                   \
+        }                                                                                           \
+    }
+
+    // One column tile per wave (decoding, short portions): the loads of step s + 1 are issued
+    // before the arithmetic of step s.  Two tiles per wave need the registers for accumulators
+    // and rely on other waves of the SIMD to cover the latency instead.
+    constexpr bool PIPE = NQT == 1;
+    if (PIPE && s_begin < s_end) TFF_ATTN_LOAD(0, s_begin)
     for (int s = s_begin; s < s_end; ++s) {
         const int kb = kb0 + s * 32;
-        // every load of the step is issued before the first product, so the wave keeps the
-        // whole 32-key slice of K and of V in flight at once
-        bf16x8 kf[2][KS];
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-            const int j = min(kb + kt * 16 + qc, kmax);   // rows past the last key repeat it; masked below
-            const int page = bt[j / page_size];
-            const bf16_t* kp = k_cache + (((size_t)page * nkv + g) * page_size + (j % page_size)) * D;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const int e = ks * 32 + kg * 8;
-                uint4 v = make_uint4(0, 0, 0, 0);
-                if (e < D) v = *reinterpret_cast<const uint4*>(kp + e);
-                kf[kt][ks] = *reinterpret_cast<bf16x8*>(&v);
+        const int cur = PIPE ? ((s - s_begin) & 1) : 0;
+        if constexpr (PIPE) {
+            if (s + 1 < s_end) {
+                if (cur == 0) TFF_ATTN_LOAD(1, s + 1) else TFF_ATTN_LOAD(0, s + 1)
             }
-        }
-        // value runs of this lane group: keys kb + g*4 .. +3 and kb + 16 + g*4 .. +3
-        union VF { uint2 u[2]; bf16x8 v; };
-        VF vf[DT];
-        {
-            const bf16_t* vrun[2];
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt) {
-                const int j0 = min(kb + kt * 16 + kg * 4, (kmax / 4) * 4);
-                const int page = bt[j0 / page_size];
-                vrun[kt] = v_cache + ((size_t)page * nkv + g) * D * page_size + (j0 % page_size);
-            }
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                const size_t eoff = (size_t)(dt * 16 + qc) * page_size;
-                vf[dt].u[0] = *reinterpret_cast<const uint2*>(vrun[0] + eoff);
-                vf[dt].u[1] = *reinterpret_cast<const uint2*>(vrun[1] + eoff);
-            }
+        } else {
+            TFF_ATTN_LOAD(0, s)
         }
         floatx4 sacc[NQT][2];
 #pragma unroll
         for (int t = 0; t < NQT; ++t) sacc[t][0] = sacc[t][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+        if (cur == 0) {
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
+            for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
+                for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-                for (int t = 0; t < NQT; ++t)
-                    sacc[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kt][ks], qf[t][ks], sacc[t][kt], 0, 0, 0);
+                    for (int t = 0; t < NQT; ++t)
+                        sacc[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][kt][ks], qf[t][ks], sacc[t][kt], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                    for (int t = 0; t < NQT; ++t)
+                        sacc[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][kt][ks], qf[t][ks], sacc[t][kt], 0, 0, 0);
+        }
         bf16x8 pf[NQT];
 #pragma unroll
         for (int t = 0; t < NQT; ++t) {
@@ -189,12 +211,21 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
                 oacc[t][dt][2] *= alpha; oacc[t][dt][3] *= alpha;
             }
         }
+        if (cur == 0) {
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+            for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int t = 0; t < NQT; ++t)
-                oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf[t], oacc[t][dt], 0, 0, 0);
+                for (int t = 0; t < NQT; ++t)
+                    oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[0][dt].v, pf[t], oacc[t][dt], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int t = 0; t < NQT; ++t)
+                    oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[1][dt].v, pf[t], oacc[t][dt], 0, 0, 0);
+        }
     }
+#undef TFF_ATTN_LOAD
 
 #pragma unroll
     for (int t = 0; t < NQT; ++t) {

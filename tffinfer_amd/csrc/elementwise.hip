@@ -23,7 +23,7 @@ int tff_check_launch(const char* what) {
     return 0;
 }
 TFF_API const char* tff_last_error() { return g_error; }
-TFF_API int tff_abi_version() { return 4; }
+TFF_API int tff_abi_version() { return 5; }
 
 // ----------------------------------------------------------------- embed ---
 // x[t, :] = E[token[t], :]   (reference: src/kernel/cpu/embedding.cpp:34-49,
@@ -87,6 +87,71 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __res
     }
 }
 
+// The same for rows whose width is a multiple of 4: 16-byte accesses, and rows of up to 4096
+// elements pass through memory once (the sum is kept in registers for the second sweep).
+template <typename TO>
+__device__ __forceinline__ void store_out4(TO* o, float4 v);
+template <>
+__device__ __forceinline__ void store_out4<float>(float* o, float4 v) { *reinterpret_cast<float4*>(o) = v; }
+template <>
+__device__ __forceinline__ void store_out4<bf16_t>(bf16_t* o, float4 v) {
+    union { bf16_t h[4]; uint2 u; } pk;
+    pk.h[0] = (bf16_t)v.x; pk.h[1] = (bf16_t)v.y; pk.h[2] = (bf16_t)v.z; pk.h[3] = (bf16_t)v.w;
+    *reinterpret_cast<uint2*>(o) = pk.u;
+}
+
+template <typename TO>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid,
+                                                               const float* __restrict__ delta,
+                                                               const float* __restrict__ w, float eps,
+                                                               TO* __restrict__ out,
+                                                               const int32_t* __restrict__ rows, int H) {
+    __shared__ float red[17];
+    const int i = blockIdx.x, tid = threadIdx.x;
+    const int r = rows ? rows[i] : i;
+    const int H4 = H >> 2;
+    float4* x4 = reinterpret_cast<float4*>(resid + (size_t)r * H);
+    const float4* d4 = delta ? reinterpret_cast<const float4*>(delta + (size_t)r * H) : nullptr;
+    const float4* w4 = reinterpret_cast<const float4*>(w);
+    const bool store = rows == nullptr && d4 != nullptr;
+    float4 cache[4];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int j = tid + it * 256;
+        if (j < H4) {
+            float4 v = x4[j];
+            if (d4) { const float4 dv = d4[j]; v.x += dv.x; v.y += dv.y; v.z += dv.z; v.w += dv.w; }
+            if (store) x4[j] = v;
+            cache[it] = v;
+            ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+        }
+    }
+    for (int j = tid + 1024; j < H4; j += 256) {
+        float4 v = x4[j];
+        if (d4) { const float4 dv = d4[j]; v.x += dv.x; v.y += dv.y; v.z += dv.z; v.w += dv.w; }
+        if (store) x4[j] = v;
+        ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+    }
+    ss = block_sum(ss, red);
+    const float rr = rsqrtf(ss / (float)H + eps);
+    TO* o = out + (size_t)i * H;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int j = tid + it * 256;
+        if (j < H4) {
+            const float4 v = cache[it], wv = w4[j];
+            store_out4<TO>(o + 4 * j, make_float4(v.x * rr * wv.x, v.y * rr * wv.y, v.z * rr * wv.z, v.w * rr * wv.w));
+        }
+    }
+    for (int j = tid + 1024; j < H4; j += 256) {
+        float4 v = x4[j];
+        if (d4 && !store) { const float4 dv = d4[j]; v.x += dv.x; v.y += dv.y; v.z += dv.z; v.w += dv.w; }
+        const float4 wv = w4[j];
+        store_out4<TO>(o + 4 * j, make_float4(v.x * rr * wv.x, v.y * rr * wv.y, v.z * rr * wv.z, v.w * rr * wv.w));
+    }
+}
+
 TFF_API int tff_add_rmsnorm(float* resid, const float* delta, const float* weight, float eps,
                             void* out, const int32_t* rows, int n, int H, int out_dtype,
                             tff_stream_t stream) {
@@ -94,13 +159,21 @@ TFF_API int tff_add_rmsnorm(float* resid, const float* delta, const float* weigh
     TFF_REQUIRE(n >= 0 && H > 0, "add_rmsnorm: bad sizes n=%d H=%d", n, H);
     if (n == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    TFF_REQUIRE(out_dtype == TFF_F32 || out_dtype == TFF_BF16, "add_rmsnorm: unknown dtype %d", out_dtype);
+    const bool vec = H % 4 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)weight % 16) == 0 &&
+                     ((uintptr_t)out % 16) == 0 && (!delta || ((uintptr_t)delta % 16) == 0);
+    if (vec) {
+        if (out_dtype == TFF_F32)
+            add_rmsnorm_vec_kernel<float><<<n, 256, 0, s>>>(resid, delta, weight, eps, (float*)out, rows, H);
+        else
+            add_rmsnorm_vec_kernel<bf16_t><<<n, 256, 0, s>>>(resid, delta, weight, eps, (bf16_t*)out, rows, H);
+        return tff_check_launch("add_rmsnorm");
+    }
     const int threads = H >= 2048 ? 1024 : 256;
     if (out_dtype == TFF_F32)
         add_rmsnorm_kernel<float><<<n, threads, 0, s>>>(resid, delta, weight, eps, (float*)out, rows, H);
-    else if (out_dtype == TFF_BF16)
-        add_rmsnorm_kernel<bf16_t><<<n, threads, 0, s>>>(resid, delta, weight, eps, (bf16_t*)out, rows, H);
     else
-        return tff_fail("add_rmsnorm: unknown dtype %d", out_dtype);
+        add_rmsnorm_kernel<bf16_t><<<n, threads, 0, s>>>(resid, delta, weight, eps, (bf16_t*)out, rows, H);
     return tff_check_launch("add_rmsnorm");
 }
 
@@ -213,6 +286,66 @@ __global__ void qk_norm_rope_kv_kernel(T* __restrict__ qkv, int nq, int nkv, int
     }
 }
 
+// The same when the whole head is rotated (or nothing is): a lane holds both elements of its
+// pairs, so norm and rotation stay in registers; four heads share a block.
+template <typename T, typename TC>
+__global__ __launch_bounds__(256) void qk_norm_rope_kv_reg_kernel(
+    T* __restrict__ qkv, int nq, int nkv, int d, const float* __restrict__ qw,
+    const float* __restrict__ kw, float eps, const float* __restrict__ cos_sin, int pairing,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ slot_mapping,
+    TC* __restrict__ k_cache, TC* __restrict__ v_cache, int page_size) {
+    const int t = blockIdx.x;
+    const int hh = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (hh >= nq + 2 * nkv) return;
+    const int width = (nq + 2 * nkv) * d;
+    T* x = qkv + (size_t)t * width + (size_t)hh * d;
+    const int kind = hh < nq ? 0 : (hh < nq + nkv ? 1 : 2);  // q, k, v
+    const int slot = slot_mapping[t];
+    if (kind != 0 && slot < 0) return;
+    const int page = slot / page_size, off = slot % page_size;
+    if (kind == 2) {
+        const int head = hh - nq - nkv;
+        TC* vt = v_cache + ((size_t)page * nkv + head) * d * page_size + off;
+        for (int e = lane; e < d; e += 64) vt[(size_t)e * page_size] = from_f32<TC>(to_f32(x[e]));
+        return;
+    }
+    const int half = d >> 1;
+    float xa[4], xb[4];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int p = lane + 64 * i;
+        if (p < half) {
+            const int a = pairing == 0 ? p : 2 * p, b = pairing == 0 ? p + half : 2 * p + 1;
+            xa[i] = to_f32(x[a]);
+            xb[i] = to_f32(x[b]);
+            ss = fmaf(xa[i], xa[i], fmaf(xb[i], xb[i], ss));
+        }
+    }
+    ss = wave_sum(ss);
+    const float* w = kind == 0 ? qw : kw;
+    const float rr = w ? rsqrtf(ss / (float)d + eps) : 1.f;
+    const float* cs = cos_sin ? cos_sin + (size_t)positions[t] * d : nullptr;   // [pos][pair][cos, sin]
+    TC* kdst = kind == 1 ? k_cache + (((size_t)page * nkv + (hh - nq)) * page_size + off) * d : nullptr;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int p = lane + 64 * i;
+        if (p < half) {
+            const int a = pairing == 0 ? p : 2 * p, b = pairing == 0 ? p + half : 2 * p + 1;
+            float va = xa[i], vb = xb[i];
+            if (w) { va = va * rr * w[a]; vb = vb * rr * w[b]; }
+            if (cs) {
+                const float c = cs[2 * p], sn = cs[2 * p + 1];
+                const float ra = va * c - vb * sn, rb = va * sn + vb * c;
+                va = ra; vb = rb;
+            }
+            if (kind == 0) { x[a] = from_f32<T>(va); x[b] = from_f32<T>(vb); }
+            else { kdst[a] = from_f32<TC>(va); kdst[b] = from_f32<TC>(vb); }
+        }
+    }
+}
+
 TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d, const float* q_weight,
                                 const float* k_weight, float eps, const float* cos_sin,
                                 int rot_dim, int pairing, int max_pos, const int32_t* positions,
@@ -239,6 +372,19 @@ TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d, const 
                 cache_dtype, dtype);
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    TFF_REQUIRE(dtype == TFF_F32 || dtype == TFF_BF16, "qk_norm_rope_kv: unknown dtype %d", dtype);
+    if (!cos_sin || rot_dim == d) {
+        dim3 grid4(T, (nq + 2 * nkv + 3) / 4);
+        if (dtype == TFF_F32)
+            qk_norm_rope_kv_reg_kernel<float, float><<<grid4, 256, 0, s>>>(
+                (float*)qkv, nq, nkv, d, q_weight, k_weight, eps, cos_sin, pairing, positions, slot_mapping,
+                (float*)k_cache, (float*)v_cache, page_size);
+        else
+            qk_norm_rope_kv_reg_kernel<bf16_t, bf16_t><<<grid4, 256, 0, s>>>(
+                (bf16_t*)qkv, nq, nkv, d, q_weight, k_weight, eps, cos_sin, pairing, positions, slot_mapping,
+                (bf16_t*)k_cache, (bf16_t*)v_cache, page_size);
+        return tff_check_launch("qk_norm_rope_kv");
+    }
     dim3 grid(T, nq + 2 * nkv);
     if (dtype == TFF_F32)
         qk_norm_rope_kv_kernel<float, float><<<grid, 64, 0, s>>>(

@@ -46,11 +46,20 @@ __device__ __forceinline__ void store4(TC* dst, const floatx4& v, int n, int N, 
 // fragment order (linear 16-byte stores), double buffered; a wave reads a
 // fragment back as one linear 1 KB.  The padding of W to 32 k holds zeros, so
 // k past the end of A only has to be readable: what it multiplies is zero.
-template <int WTM, int WTN, typename TC>
+// GLU: the 16-row groups of W alternate between a gate and an up projection
+// (group 2p gate, group 2p+1 up); the epilogue writes silu(gate) * up, N / 2 columns.
+__device__ __forceinline__ floatx4 silu_mul(const floatx4& g, const floatx4& u) {
+    floatx4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = g[e] / (1.0f + __expf(-g[e])) * u[e];
+    return o;
+}
+
+template <int WTM, int WTN, bool GLU, typename TC>
 __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __restrict__ A,
                                                                const bf16_t* __restrict__ Wp,
                                                                TC* __restrict__ C, int M, int N,
-                                                               int K, int lda, int KB) {
+                                                               int K, int lda, int KB, int n_out) {
     constexpr int BM = WTM * 32, BN = WTN * 32;
     constexpr int AF = BM / 16 * 2, WF = BN / 16 * 2;   // fragments per operand tile (2 k-steps)
     constexpr int AL = AF / 4, WL = WF / 4;             // 16-byte loads per thread and operand
@@ -146,16 +155,167 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
 #undef TFF_STORE_LDS
 
     // lane holds C[m][n .. n+3], n = n0 + (wn*WTN + i)*16 + fg*4, m = m0 + (wm*WTM + j)*16 + fr
-    const bool vec = (N % 4) == 0;
+    if constexpr (GLU) {
+        static_assert(WTN % 2 == 0, "gate and up groups come in pairs");
+        const int No = n_out;
+        const bool vec = (No % 4) == 0;
 #pragma unroll
-    for (int i = 0; i < WTN; ++i) {
-        const int n = n0 + (wn * WTN + i) * 16 + fg * 4;
+        for (int i = 0; i < WTN; i += 2) {
+            const int n = (n0 + (wn * WTN + i) * 16) / 2 + fg * 4;
 #pragma unroll
-        for (int j = 0; j < WTM; ++j) {
-            const int m = m0 + (wm * WTM + j) * 16 + fr;
-            if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, acc[i][j], n, N, vec);
+            for (int j = 0; j < WTM; ++j) {
+                const int m = m0 + (wm * WTM + j) * 16 + fr;
+                if (m < M && n < No)
+                    store4<TC>(C + (size_t)m * No + n, silu_mul(acc[i][j], acc[i + 1][j]), n, No, vec);
+            }
+        }
+    } else {
+        const bool vec = (N % 4) == 0;
+#pragma unroll
+        for (int i = 0; i < WTN; ++i) {
+            const int n = n0 + (wn * WTN + i) * 16 + fg * 4;
+#pragma unroll
+            for (int j = 0; j < WTM; ++j) {
+                const int m = m0 + (wm * WTM + j) * 16 + fr;
+                if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, acc[i][j], n, N, vec);
+            }
         }
     }
+}
+
+// ------------------------------------------------------- tiled, async copy ---
+// The same tiling with the copies global -> LDS done by the load unit itself
+// (global_load_lds_dwordx4: every lane's 16 bytes land at LDS base + lane * 16,
+// which is exactly fragment order), so no register and no LDS store instruction
+// is spent on staging, and STAGES - 1 tiles are in flight while one is worked on.
+// A wave waits for its own copies of the tile it is about to read
+// (s_waitcnt vmcnt), the barrier that follows makes the other waves' visible.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* glb_ptr_t;
+
+constexpr int vmcnt_imm(int v) { return (v & 15) | (7 << 4) | (15 << 8) | ((v >> 4) << 14); }
+
+template <int WTM, int WTN, int STAGES, bool GLU, typename TC>
+__global__ __launch_bounds__(256) void gemm_bf16_async_kernel(const bf16_t* __restrict__ A,
+                                                               const bf16_t* __restrict__ Wp,
+                                                               TC* __restrict__ C, int M, int N,
+                                                               int K, int lda, int KB, int n_out) {
+    constexpr int BM = WTM * 32, BN = WTN * 32;
+    constexpr int AF = BM / 16 * 2, WF = BN / 16 * 2;   // fragments per operand tile (2 k-steps)
+    constexpr int FR = AF + WF;                          // fragments per stage, 1 KB each
+    constexpr int LPW = FR / 4;                          // copies a wave issues per tile
+    static_assert(FR % 4 == 0, "fragments are dealt to 4 waves");
+    static_assert((STAGES - 2) * LPW < 64, "vmcnt has 6 bits");
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[STAGES * FR * 512];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int fr = lane & 15, fg = lane >> 4;
+    const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+    const int NB = (N + 15) / 16;
+    const int nk = (K + 63) / 64;
+
+    floatx4 acc[WTN][WTM];
+#pragma unroll
+    for (int i = 0; i < WTN; ++i)
+#pragma unroll
+        for (int j = 0; j < WTM; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // this wave's copies: fragments f = wave + 4 j of a stage; f < AF is of A, else of W
+    const bf16_t* src[LPW];
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) {
+        const int f = wave + 4 * j;
+        if (f < AF) {
+            const int row = min(m0 + (f >> 1) * 16 + fr, M - 1);   // rows past the end repeat the last
+            src[j] = A + (size_t)row * lda;
+        } else {
+            const int nb = min(n0 / 16 + ((f - AF) >> 1), NB - 1);
+            src[j] = Wp + (size_t)nb * KB * 512 + lane * 8;
+        }
+    }
+    // Tiles past the end are copied too (as the last tile, into stages nobody reads any more):
+    // then the number of copies in flight is the same in every iteration and one constant wait
+    // covers them all.
+#define TFF_ISSUE_TILE(tile)                                                                       \
+    {                                                                                              \
+        const int kt_ = min((tile), nk - 1);                                                       \
+        const int st_ = (tile) % STAGES;                                                           \
+        _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                          \
+            const int f = wave + 4 * j;                                                            \
+            const bf16_t* g_;                                                                      \
+            if (f < AF) g_ = src[j] + min(kt_ * 64 + (f & 1) * 32 + fg * 8, K - 8);                \
+            else g_ = src[j] + (size_t)min(2 * kt_ + ((f - AF) & 1), KB - 1) * 512;                \
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)g_, (lds_ptr_t)(smem + (st_ * FR + f) * 512), 16, 0, 0); \
+        }                                                                                          \
+    }
+
+#pragma unroll
+    for (int t = 0; t < STAGES - 1; ++t) TFF_ISSUE_TILE(t)
+    for (int kt = 0; kt < nk; ++kt) {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * LPW));   // this wave's part of tile kt is in
+        __syncthreads();                                             // ... and everybody else's
+        TFF_ISSUE_TILE(kt + STAGES - 1)                              // into the stage read last iteration
+        const bf16_t* st = smem + (kt % STAGES) * FR * 512;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            if (2 * kt + ks < KB) {   // k-steps past the end of K are not in W
+                bf16x8 fw[WTN], fa[WTM];
+#pragma unroll
+                for (int i = 0; i < WTN; ++i)
+                    fw[i] = *reinterpret_cast<const bf16x8*>(st + (AF + (wn * WTN + i) * 2 + ks) * 512 + lane * 8);
+#pragma unroll
+                for (int j = 0; j < WTM; ++j)
+                    fa[j] = *reinterpret_cast<const bf16x8*>(st + ((wm * WTM + j) * 2 + ks) * 512 + lane * 8);
+#pragma unroll
+                for (int i = 0; i < WTN; ++i)
+#pragma unroll
+                    for (int j = 0; j < WTM; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[i], fa[j], acc[i][j], 0, 0, 0);
+            }
+        }
+    }
+#undef TFF_ISSUE_TILE
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));   // the copies past the end must not outlive the block
+
+    if constexpr (GLU) {
+        static_assert(WTN % 2 == 0, "gate and up groups come in pairs");
+        const bool vec = (n_out % 4) == 0;
+#pragma unroll
+        for (int i = 0; i < WTN; i += 2) {
+            const int n = (n0 + (wn * WTN + i) * 16) / 2 + fg * 4;
+#pragma unroll
+            for (int j = 0; j < WTM; ++j) {
+                const int m = m0 + (wm * WTM + j) * 16 + fr;
+                if (m < M && n < n_out)
+                    store4<TC>(C + (size_t)m * n_out + n, silu_mul(acc[i][j], acc[i + 1][j]), n, n_out, vec);
+            }
+        }
+    } else {
+        const bool vec = (N % 4) == 0;
+#pragma unroll
+        for (int i = 0; i < WTN; ++i) {
+            const int n = n0 + (wn * WTN + i) * 16 + fg * 4;
+#pragma unroll
+            for (int j = 0; j < WTM; ++j) {
+                const int m = m0 + (wm * WTM + j) * 16 + fr;
+                if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, acc[i][j], n, N, vec);
+            }
+        }
+    }
+}
+
+template <int WTM, int WTN, int STAGES, bool GLU = false>
+static int launch_async(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
+                        int c_dtype, int n_out, hipStream_t s) {
+    const int KB = (K + 31) / 32;
+    const dim3 grid((M + WTM * 32 - 1) / (WTM * 32), (N + WTN * 32 - 1) / (WTN * 32));
+    TFF_REQUIRE(grid.y <= 65535, "gemm: too many columns N=%d", N);
+    if (c_dtype == TFF_F32)
+        gemm_bf16_async_kernel<WTM, WTN, STAGES, GLU, float><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
+    else
+        gemm_bf16_async_kernel<WTM, WTN, STAGES, GLU, bf16_t><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
+    return tff_check_launch("gemm_bf16_async");
 }
 
 // ------------------------------------------------------------- skinny M ---
@@ -168,15 +328,24 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
 // result goes through global memory and the result does not depend on the
 // launch.  UNROLL k-steps of loads are issued before the first is used: a wave
 // keeps UNROLL * (R + MT) KB in flight, which is what hides the latency of HBM.
-template <int MT, int R, int UNROLL, int SK_WAVES, typename TC>
-__global__ __launch_bounds__(64 * SK_WAVES) void gemm_bf16_skinny_kernel(
+// The block's waves form NSETS sets of KSPLIT waves: a set works on R row groups
+// of W, its waves split K.  Sets walk K at the same pace, so the rows of A one
+// set has fetched are in cache for the others: with many rows of A (MT > 1)
+// that, not W, is most of a wave's traffic.  With GLU, sets 2p and 2p+1 hold a
+// gate group and the up group that follows it in W; the epilogue writes
+// silu(gate) * up.
+template <int MT, int R, int UNROLL, int KSPLIT, int NSETS, bool GLU, typename TC>
+__global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
-    int K, int lda, int KB) {
-    __shared__ floatx4 part[SK_WAVES - 1][R * MT][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int K, int lda, int KB, int n_out) {
+    constexpr int SK_WAVES = KSPLIT * NSETS;
+    static_assert(!GLU || (R == 1 && NSETS % 2 == 0), "a gate and its up group are one row group each");
+    __shared__ floatx4 part[SK_WAVES][R * MT][64];
+    const int lane = threadIdx.x & 63, wave_id = threadIdx.x >> 6;
+    const int set = wave_id / KSPLIT, wave = wave_id % KSPLIT;
     const int fr = lane & 15, fg = lane >> 4;
     const int NB = (N + 15) / 16;
-    const int nb0 = blockIdx.x * R;
+    const int nb0 = (blockIdx.x * NSETS + set) * R;
 
     floatx4 acc[R][MT];
 #pragma unroll
@@ -185,7 +354,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_bf16_skinny_kernel(
         for (int t = 0; t < MT; ++t) acc[r][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     // k-steps of 32 are dealt out to the waves in contiguous runs
-    const int per = (KB + SK_WAVES - 1) / SK_WAVES;
+    const int per = (KB + KSPLIT - 1) / KSPLIT;
     const int s_begin = wave * per;
     const int s_end = min(KB, s_begin + per);
 
@@ -236,97 +405,130 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_bf16_skinny_kernel(
             for (int t = 0; t < MT; ++t)
                 acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(rw[r]), as_frag(ra[t]), acc[r][t], 0, 0, 0);
     }
-    if (wave > 0) {
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+    for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int t = 0; t < MT; ++t) part[wave - 1][r * MT + t][lane] = acc[r][t];
-    }
+        for (int t = 0; t < MT; ++t) part[wave_id][r * MT + t][lane] = acc[r][t];
     __syncthreads();
-    if (wave == 0) {
-        const bool vec = (N % 4) == 0;
+    if (wave == 0) {   // the first wave of every set adds up the set's partial sums, in a fixed order
+        if constexpr (GLU) {
+            if ((set & 1) == 0) {
+                const bool vec = (n_out % 4) == 0;
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+                for (int t = 0; t < MT; ++t) {
+                    floatx4 g = part[set * KSPLIT][t][lane], u = part[(set + 1) * KSPLIT][t][lane];
 #pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                floatx4 v = acc[r][t];
+                    for (int w = 1; w < KSPLIT; ++w) {
+                        const floatx4 pg = part[set * KSPLIT + w][t][lane], pu = part[(set + 1) * KSPLIT + w][t][lane];
 #pragma unroll
-                for (int w = 0; w < SK_WAVES - 1; ++w) {
-                    const floatx4 p = part[w][r * MT + t][lane];
-                    v[0] += p[0]; v[1] += p[1]; v[2] += p[2]; v[3] += p[3];
+                        for (int e = 0; e < 4; ++e) { g[e] += pg[e]; u[e] += pu[e]; }
+                    }
+                    const int n = (nb0 >> 1) * 16 + fg * 4;
+                    const int m = t * 16 + fr;
+                    if (m < M && n < n_out) store4<TC>(C + (size_t)m * n_out + n, silu_mul(g, u), n, n_out, vec);
                 }
-                const int n = (nb0 + r) * 16 + fg * 4;
-                const int m = t * 16 + fr;
-                if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, v, n, N, vec);
             }
+        } else {
+            const bool vec = (N % 4) == 0;
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    floatx4 v = part[set * KSPLIT][r * MT + t][lane];
+#pragma unroll
+                    for (int w = 1; w < KSPLIT; ++w) {
+                        const floatx4 p = part[set * KSPLIT + w][r * MT + t][lane];
+                        v[0] += p[0]; v[1] += p[1]; v[2] += p[2]; v[3] += p[3];
+                    }
+                    const int n = (nb0 + r) * 16 + fg * 4;
+                    const int m = t * 16 + fr;
+                    if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, v, n, N, vec);
+                }
+        }
     }
 }
 
-template <int MT, int R, int UNROLL, int SK_WAVES>
+template <int MT, int R, int UNROLL, int KSPLIT, int NSETS = 1, bool GLU = false>
 static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
-                         int c_dtype, hipStream_t s) {
+                         int c_dtype, int n_out, hipStream_t s) {
     const int NB = (N + 15) / 16, KB = (K + 31) / 32;
-    const dim3 grid((NB + R - 1) / R);
+    const int per_block = NSETS * R;
+    const dim3 grid((NB + per_block - 1) / per_block);
     if (c_dtype == TFF_F32)
-        gemm_bf16_skinny_kernel<MT, R, UNROLL, SK_WAVES, float><<<grid, 64 * SK_WAVES, 0, s>>>(
-            A, Wp, (float*)C, M, N, K, lda, KB);
+        gemm_bf16_skinny_kernel<MT, R, UNROLL, KSPLIT, NSETS, GLU, float>
+            <<<grid, 64 * KSPLIT * NSETS, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
     else
-        gemm_bf16_skinny_kernel<MT, R, UNROLL, SK_WAVES, bf16_t><<<grid, 64 * SK_WAVES, 0, s>>>(
-            A, Wp, (bf16_t*)C, M, N, K, lda, KB);
+        gemm_bf16_skinny_kernel<MT, R, UNROLL, KSPLIT, NSETS, GLU, bf16_t>
+            <<<grid, 64 * KSPLIT * NSETS, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
     return tff_check_launch("gemm_bf16_skinny");
 }
 
-template <int WTM, int WTN>
+template <int WTM, int WTN, bool GLU = false>
 static int launch_tiled(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
-                        int c_dtype, hipStream_t s) {
+                        int c_dtype, int n_out, hipStream_t s) {
     const int KB = (K + 31) / 32;
     const dim3 grid((M + WTM * 32 - 1) / (WTM * 32), (N + WTN * 32 - 1) / (WTN * 32));
     TFF_REQUIRE(grid.y <= 65535, "gemm: too many columns N=%d", N);
     if (c_dtype == TFF_F32)
-        gemm_bf16_tiled_kernel<WTM, WTN, float><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB);
+        gemm_bf16_tiled_kernel<WTM, WTN, GLU, float><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
     else
-        gemm_bf16_tiled_kernel<WTM, WTN, bf16_t><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB);
+        gemm_bf16_tiled_kernel<WTM, WTN, GLU, bf16_t><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
     return tff_check_launch("gemm_bf16_tiled");
 }
 
+// glu_out > 0: W holds gate and up groups in turn (N = 2 * ceil16(glu_out) rows) and C is
+// [M, glu_out] = silu(gate) * up.
 int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
-                  int c_dtype, hipStream_t s) {
+                  int c_dtype, int glu_out, hipStream_t s) {
     TFF_REQUIRE(K % 8 == 0 && lda % 8 == 0,
                 "gemm: the bfloat16 product needs the inner size (K=%d, row stride %d) to be a multiple of 8",
                 K, lda);
     TFF_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)Wp % 16) == 0 && ((uintptr_t)C % 16) == 0,
                 "gemm: operands must be 16-byte aligned");
     TFF_REQUIRE(c_dtype == TFF_F32 || c_dtype == TFF_BF16, "gemm: unknown output type %d", c_dtype);
+    // The choices below were measured at the sizes of an 8B model on an MI355X.
+    if (glu_out > 0) {
+        TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
+                    "gemm: a gated weight of %d rows does not fit %d output columns", N, glu_out);
+        if (M <= 16) return launch_skinny<1, 1, 32, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
+        if (M <= 64) return launch_async<2, 4, 4, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
+        if (M >= 1024 && N >= 8192) return launch_async<8, 8, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
+        return launch_async<4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
+    }
     if (M <= 16) {
-        // more waves per block where there are few blocks (small N) or long rows (large K)
-        if (N >= 32 * 1024) return launch_skinny<1, 1, 16, 8>(A, Wp, C, M, N, K, lda, c_dtype, s);
-        if (K >= 8192 || N <= 8192) return launch_skinny<1, 1, 8, 16>(A, Wp, C, M, N, K, lda, c_dtype, s);
-        return launch_skinny<1, 1, 16, 8>(A, Wp, C, M, N, K, lda, c_dtype, s);
+        // more waves per block where there are few blocks (small N) or long rows (large K),
+        // fewer and deeper ones in between
+        if (N >= 32 * 1024) return launch_skinny<1, 1, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+        if (K >= 8192 || N <= 4096) return launch_skinny<1, 1, 4, 16>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+        return launch_skinny<1, 1, 8, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
     }
-    if (M <= 32) return launch_skinny<2, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, s);
     if (M <= 64) {
-        if (N >= 16 * 1024) return launch_skinny<4, 4, 4, 4>(A, Wp, C, M, N, K, lda, c_dtype, s);
-        return launch_skinny<4, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, s);
+        // many columns: enough blocks for the tiled kernel with a deep pipeline; few columns: the
+        // streaming kernel, whose blocks split K among their waves
+        if (N >= 16 * 1024) return launch_async<2, 4, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+        if (M <= 32) return launch_skinny<2, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+        return launch_skinny<4, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
     }
-    return launch_tiled<4, 4>(A, Wp, C, M, N, K, lda, c_dtype, s);
+    if (M >= 1024 && N >= 16 * 1024) return launch_async<8, 8, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+    return launch_async<4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
 }
 
 int tff_gemm_f32(const float* A, const float* W, void* C, int M, int N, int K, int lda,
                  int c_dtype, hipStream_t s);
 
 TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda,
-                     int ab_dtype, int c_dtype, int w_packed, tff_stream_t stream) {
+                     int ab_dtype, int c_dtype, int w_packed, int glu_out, tff_stream_t stream) {
     TFF_REQUIRE(A && W && C, "gemm: null pointer");
     TFF_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K, "gemm: bad sizes M=%d N=%d K=%d lda=%d", M, N, K, lda);
     if (M == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (ab_dtype == TFF_F32) {
-        TFF_REQUIRE(!w_packed, "gemm: the float32 product takes a row-major weight");
+        TFF_REQUIRE(!w_packed && glu_out == 0, "gemm: the float32 product takes a plain row-major weight");
         return tff_gemm_f32((const float*)A, (const float*)W, C, M, N, K, lda, c_dtype, s);
     }
     if (ab_dtype == TFF_BF16) {
         TFF_REQUIRE(w_packed, "gemm: the bfloat16 product takes a weight in fragment order");
-        return tff_gemm_bf16((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, c_dtype, s);
+        return tff_gemm_bf16((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, c_dtype, glu_out, s);
     }
     return tff_fail("gemm: unknown operand type %d", ab_dtype);
 }

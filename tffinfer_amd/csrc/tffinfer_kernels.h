@@ -35,9 +35,11 @@ TFF_API int tff_rmsnorm(const void* x, const float* weight, float eps, void* out
 // A and W are of ab_dtype; C is of c_dtype.  float32 runs on plain FMA in a
 // fixed summation order with a row-major W (w_packed = 0); bfloat16 runs on
 // MFMA with float32 accumulation and takes W in fragment order (w_packed = 1,
-// see tff_pack_weight).
+// see tff_pack_weight).  glu_out > 0 (bfloat16 only): the 16-row groups of W
+// alternate between a gate and an up projection, N = 2 * ceil16(glu_out), and
+// C is [M, glu_out] = silu(gate) * up.
 TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda,
-                     int ab_dtype, int c_dtype, int w_packed, tff_stream_t stream);
+                     int ab_dtype, int c_dtype, int w_packed, int glu_out, tff_stream_t stream);
 
 // bfloat16 row-major [N, K] (K a multiple of 8) -> fragment order: tiles of
 // 16 rows x 32 k, each stored as the 1 KB operand of a 16x16x32 MFMA, element

@@ -61,14 +61,21 @@ class PackedWeight:
     """A bfloat16 matrix [N, K] in the fragment order of the matrix-core
     products: tiles of 16 rows by 32 k stored as the 1 KB operand a wave loads,
     rows and k padded with zeros to multiples of 16 and 32."""
-    __slots__ = ("data", "N", "K")
+    __slots__ = ("data", "N", "K", "glu_out")
 
-    def __init__(self, data: torch.Tensor, N: int, K: int):
+    def __init__(self, data: torch.Tensor, N: int, K: int, glu_out: int = 0):
         self.data, self.N, self.K = data, int(N), int(K)
+        #: > 0: the 16-row groups alternate between a gate and an up projection and the
+        #: product yields silu(gate) * up with this many columns
+        self.glu_out = int(glu_out)
 
     @property
     def shape(self):
         return (self.N, self.K)
+
+    @property
+    def out_features(self) -> int:
+        return self.glu_out or self.N
 
     @property
     def dtype(self):
@@ -99,6 +106,26 @@ def pack_weight(w: torch.Tensor) -> PackedWeight:
     L = _lib.load()
     _lib.check(L.tff_pack_weight(w.data_ptr(), out.data_ptr(), N, K, _stream()))
     return PackedWeight(out, N, K)
+
+
+def pack_gate_up(gate: torch.Tensor, up: torch.Tensor) -> PackedWeight:
+    """Gate and up projections [I, K] (bfloat16, on the GPU) as one weight whose
+    16-row groups alternate gate, up, gate, up, ..., in fragment order.  A
+    product with it yields silu(x gate^T) * (x up^T) directly: the activation
+    runs in the product's epilogue, on the float32 accumulators."""
+    _req(gate, "gate", torch.bfloat16, 2)
+    _req(up, "up", torch.bfloat16, 2)
+    if gate.shape != up.shape:
+        raise _lib.KernelError(f"pack_gate_up: gate {tuple(gate.shape)} and up {tuple(up.shape)} differ")
+    I, K = gate.shape
+    groups = -(-I // 16)
+    padded = torch.zeros(2, groups * 16, K, dtype=torch.bfloat16, device=gate.device)
+    padded[0, :I] = gate
+    padded[1, :I] = up
+    both = padded.view(2, groups, 16, K).permute(1, 0, 2, 3).reshape(groups * 32, K).contiguous()
+    pw = pack_weight(both)
+    pw.glu_out = I
+    return pw
 
 
 def embed(table, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
@@ -194,15 +221,18 @@ def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
     if lda < K:
         raise _lib.KernelError("linear x: rows overlap")
     out_dtype = out_dtype or x.dtype
+    glu_out = weight.glu_out if packed else 0
+    n_out = glu_out or N
     if out is None:
-        out = torch.empty(M, N, dtype=out_dtype, device=x.device)
+        out = torch.empty(M, n_out, dtype=out_dtype, device=x.device)
     else:
         _req(out, "linear out", out_dtype, 2)
-        if tuple(out.shape) != (M, N):
-            raise _lib.KernelError(f"linear out: shape {tuple(out.shape)} is not {(M, N)}")
+        if tuple(out.shape) != (M, n_out):
+            raise _lib.KernelError(f"linear out: shape {tuple(out.shape)} is not {(M, n_out)}")
     L = _lib.load()
     _lib.check(L.tff_gemm(x.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K, lda,
-                          dtype_code(x.dtype), dtype_code(out_dtype), 1 if packed else 0, _stream()))
+                          dtype_code(x.dtype), dtype_code(out_dtype), 1 if packed else 0, glu_out,
+                          _stream()))
     return out
 
 

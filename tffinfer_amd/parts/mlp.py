@@ -12,8 +12,7 @@ class SwiGLU(FeedForward):
 
     Reference: src/core/model/base/ModelCreatorBase.cpp:51-94 (up, gate, the
     unary op with x1 = gate, x2 = up, down), src/kernel/cuda/unary.cu:10-27.
-    Gate and up are stacked into one [2I, H] matrix at load so that one product
-    streams both; the activation reads the two halves of its rows.
+    Gate and up are put into one matrix at load so that one product streams both.
     """
 
     graph_safe = True
@@ -33,11 +32,19 @@ class SwiGLU(FeedForward):
         }
 
     def load_weights(self, weights, dtype, device):
-        gu = torch.cat([weights["gate_proj.weight"], weights["up_proj.weight"]], 0)
-        self.w_gate_up = to_device(gu, dtype, device)
+        gate, up = weights["gate_proj.weight"], weights["up_proj.weight"]
+        if dtype == torch.bfloat16 and torch.device(device).type == "cuda":
+            # bfloat16: gate and up rows interleaved in groups of 16 in one weight, so that one
+            # product streams both and applies silu(gate) * up to its float32 accumulators
+            from ..kernels import ops
+            self.w_gate_up = ops.pack_gate_up(gate.to(dtype).contiguous().to(device),
+                                              up.to(dtype).contiguous().to(device))
+        else:
+            # float32: gate and up stacked to [2I, H]; the activation is a kernel of its own
+            self.w_gate_up = to_device(torch.cat([gate, up], 0), dtype, device)
         self.w_down = to_device(weights["down_proj.weight"], dtype, device)
 
     def forward(self, ctx, x):
         gu = ctx.ops.linear(x, self.w_gate_up)
-        m = ctx.ops.swiglu(gu)
+        m = gu if getattr(self.w_gate_up, "glu_out", 0) else ctx.ops.swiglu(gu)
         return ctx.ops.linear(m, self.w_down, out_dtype=torch.float32)
