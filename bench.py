@@ -39,6 +39,8 @@ def parse_args():
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
+                    help="measure one phase only (for profiling); the JSON line then lacks the other")
     ap.add_argument("--seed", type=int, default=0)
     return ap.parse_args()
 
@@ -144,8 +146,16 @@ def main():
                         max_model_len=cfg["max_position_embeddings"], use_graphs=not args.no_graphs)
     engine = LLMEngine(model, opt)
 
-    t_prefill = measure_prefill(engine, gen, args.prefill_tokens, vocab)
-    t_decode = measure_decode(engine, gen, args.batch, args.context, args.steps, args.warmup, vocab)
+    t_prefill = t_decode = None
+    if args.only != "decode":
+        t_prefill = measure_prefill(engine, gen, args.prefill_tokens, vocab)
+    if args.only != "prefill":
+        t_decode = measure_decode(engine, gen, args.batch, args.context, args.steps, args.warmup, vocab)
+    if args.only:
+        part = ({"prefill_ms": round(1000 * t_prefill, 3)} if t_prefill else
+                {"decode_ms_per_step": round(1000 * t_decode / args.steps, 4)})
+        print(json.dumps({"only": args.only, **part, "batch": args.batch, "context": args.context}))
+        return
     points = {}
     if not args.no_points:
         for b, key in ((1, "decode_b1"), (64, "decode_b64")):

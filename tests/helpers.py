@@ -20,8 +20,16 @@ TINY_B = dict(
     vocab_size=320, max_position_embeddings=256, rms_norm_eps=1e-5, rope_theta=1000000.0,
     tie_word_embeddings=False, use_sliding_window=True, sliding_window=24, max_window_layers=1,
 )
-TINY_CONFIGS = {"A": (TINY_A, 11), "B": (TINY_B, 23)}
-PAGE_SIZE = {"A": 16, "B": 8}
+# A third one with the head size of the large models, an odd group size and sizes that are
+# multiples of 8 only.
+TINY_C = dict(
+    architectures=["Qwen3ForCausalLM"], hidden_size=168, num_hidden_layers=2,
+    num_attention_heads=5, num_key_value_heads=1, head_dim=128, intermediate_size=136,
+    vocab_size=1000, max_position_embeddings=512, rms_norm_eps=3e-6, rope_theta=500000.0,
+    tie_word_embeddings=False,
+)
+TINY_CONFIGS = {"A": (TINY_A, 11), "B": (TINY_B, 23), "C": (TINY_C, 31)}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 32}
 
 
 def make_model_dir(path: str, cfg: dict, seed: int, dtype: str = "bfloat16") -> str:

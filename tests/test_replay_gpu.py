@@ -10,7 +10,7 @@ from helpers import PAGE_SIZE, TOL, random_tokens, read_config
 pytestmark = pytest.mark.gpu
 
 DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
-LENGTHS = {"A": [1, 9, 40, 100], "B": [3, 17, 31, 64, 100, 150]}
+LENGTHS = {"A": [1, 9, 40, 100], "B": [3, 17, 31, 64, 100, 150], "C": [2, 33, 70, 129, 200]}
 
 
 def requests_for(name, model_dir):
@@ -26,7 +26,7 @@ def make_runner(model_dir, dtype, page_size, num_pages, max_seqs=8):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 @pytest.mark.parametrize("mode", ["whole", "tail", "chunks", "mixed"])
 def test_replay_modes(model_dirs, name, dtype, mode):
     model_dir = model_dirs[name]
@@ -78,3 +78,72 @@ def test_replay_with_decode_graphs(model_dirs, name, dtype, mode):
     decode_only = sum(1 for s in steps if s["entries"] and all(len(e["tokens"]) == 1 for e in s["entries"]))
     assert decode_only >= 3
     rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,n", [("A", 128), ("B", 256)])
+@pytest.mark.parametrize("graphs", [False, True])
+def test_long_decoding(model_dirs, name, dtype, n, graphs):
+    """A few prompt tokens, then one token a step up to the model's longest
+    position: every position against the plain implementation (B's window
+    passes its pages many times over)."""
+    from tffinfer_amd.engine.runner import ModelRunner
+    from tffinfer_amd.models import load_model
+    model_dir = model_dirs[name]
+    V = read_config(model_dir)["vocab_size"]
+    reqs = {"long": random_tokens(n, V, 4242)}
+    steps = rl.trace_tail(reqs, tail=n - 5)
+    ps = PAGE_SIZE[name]
+    runner = ModelRunner(load_model(model_dir, DTYPES[dtype], "cuda:0"), page_size=ps,
+                         num_pages=-(-n // ps), max_seqs=2, use_graphs=graphs)
+    results = rl.run_steps_in_process(runner, steps)
+    rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
+    if name == "B":   # the window groups gave pages back on the way
+        assert any(g.spec.window > 0 for g in runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_first_tokens(model_dirs, name, dtype):
+    """Sequences of one, two and three tokens: whole, and token by token."""
+    model_dir = model_dirs[name]
+    V = read_config(model_dir)["vocab_size"]
+    reqs = {f"s{n}": random_tokens(n, V, 90 + n) for n in (1, 2, 3)}
+    for steps in (rl.trace_whole(reqs), rl.trace_tail(reqs, tail=3)):
+        runner = make_runner(model_dir, dtype, PAGE_SIZE[name], 4)
+        results = rl.run_steps_in_process(runner, steps)
+        rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
+
+
+MID = dict(
+    architectures=["Qwen3ForCausalLM"], hidden_size=1024, num_hidden_layers=3,
+    num_attention_heads=16, num_key_value_heads=4, head_dim=64, intermediate_size=8200,
+    vocab_size=9000, max_position_embeddings=2048, rms_norm_eps=1e-6, rope_theta=1000000.0,
+    tie_word_embeddings=True,
+)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_midsize_model_long_prompt(tmp_path_factory, dtype):
+    """Sizes at which the large-tile products, the gated epilogue and the
+    two-tile attention kernel run: a prompt of 1,100 tokens whole, in portions
+    of 512, and followed by decoding, against the plain implementation."""
+    from helpers import make_model_dir
+    model_dir = make_model_dir(str(tmp_path_factory.mktemp("mid") / "m"), MID, 5)
+    toks = random_tokens(1100, MID["vocab_size"], 77)
+    reqs = {"p": toks}
+    look = [0, 1, 63, 64, 500, 1023, 1024, 1087]
+    whole = [{"step": 0, "entries": [{"id": "p", "tokens": toks[:1088], "want": look}], "end": []}]
+    whole += [{"step": 1 + i, "entries": [{"id": "p", "tokens": [toks[1088 + i]], "want": [0]}],
+               "end": ["p"] if i == 11 else []} for i in range(12)]
+    parts, done = [], 0
+    for n in (512, 512, 64, 12):
+        want = [w - done for w in look if done <= w < done + n]
+        parts.append({"step": len(parts), "entries": [{"id": "p", "tokens": toks[done:done + n], "want": want}],
+                      "end": ["p"] if done + n == 1100 else []})
+        done += n
+    for steps in (whole, parts):
+        runner = make_runner(model_dir, dtype, 16, 72, max_seqs=2)
+        results = rl.run_steps_in_process(runner, steps)
+        worst = rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
+        print(f"mid {dtype}: worst rel. error {worst:.3e}")

@@ -195,21 +195,22 @@ typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 
 constexpr int vmcnt_imm(int v) { return (v & 15) | (7 << 4) | (15 << 8) | ((v >> 4) << 14); }
 
-template <int WTM, int WTN, int STAGES, bool GLU, typename TC>
-__global__ __launch_bounds__(256) void gemm_bf16_async_kernel(const bf16_t* __restrict__ A,
-                                                               const bf16_t* __restrict__ Wp,
-                                                               TC* __restrict__ C, int M, int N,
-                                                               int K, int lda, int KB, int n_out) {
-    constexpr int BM = WTM * 32, BN = WTN * 32;
+template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU, typename TC>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
+    int K, int lda, int KB, int n_out) {
+    // WGM x WGN waves, each WTM x WTN MFMA tiles of 16 x 16
+    constexpr int NW = WGM * WGN;
+    constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
     constexpr int AF = BM / 16 * 2, WF = BN / 16 * 2;   // fragments per operand tile (2 k-steps)
     constexpr int FR = AF + WF;                          // fragments per stage, 1 KB each
-    constexpr int LPW = FR / 4;                          // copies a wave issues per tile
-    static_assert(FR % 4 == 0, "fragments are dealt to 4 waves");
+    constexpr int LPW = FR / NW;                         // copies a wave issues per tile
+    static_assert(FR % NW == 0, "fragments are dealt to the waves evenly");
     static_assert((STAGES - 2) * LPW < 64, "vmcnt has 6 bits");
     __shared__ __attribute__((aligned(1024))) bf16_t smem[STAGES * FR * 512];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WGN, wn = wave % WGN;
     const int fr = lane & 15, fg = lane >> 4;
     const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
     const int NB = (N + 15) / 16;
@@ -221,11 +222,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_async_kernel(const bf16_t* __re
 #pragma unroll
         for (int j = 0; j < WTM; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // this wave's copies: fragments f = wave + 4 j of a stage; f < AF is of A, else of W
+    // this wave's copies: fragments f = wave + NW j of a stage; f < AF is of A, else of W
     const bf16_t* src[LPW];
 #pragma unroll
     for (int j = 0; j < LPW; ++j) {
-        const int f = wave + 4 * j;
+        const int f = wave + NW * j;
         if (f < AF) {
             const int row = min(m0 + (f >> 1) * 16 + fr, M - 1);   // rows past the end repeat the last
             src[j] = A + (size_t)row * lda;
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_async_kernel(const bf16_t* __re
         const int kt_ = min((tile), nk - 1);                                                       \
         const int st_ = (tile) % STAGES;                                                           \
         _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                          \
-            const int f = wave + 4 * j;                                                            \
+            const int f = wave + NW * j;                                                            \
             const bf16_t* g_;                                                                      \
             if (f < AF) g_ = src[j] + min(kt_ * 64 + (f & 1) * 32 + fg * 8, K - 8);                \
             else g_ = src[j] + (size_t)min(2 * kt_ + ((f - AF) & 1), KB - 1) * 512;                \
@@ -305,17 +306,27 @@ __global__ __launch_bounds__(256) void gemm_bf16_async_kernel(const bf16_t* __re
     }
 }
 
+template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU = false>
+static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
+                          int c_dtype, int n_out, hipStream_t s) {
+    const int KB = (K + 31) / 32;
+    constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
+    const dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN);
+    TFF_REQUIRE(grid.y <= 65535, "gemm: too many columns N=%d", N);
+    if (c_dtype == TFF_F32)
+        gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, float>
+            <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
+    else
+        gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, bf16_t>
+            <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
+    return tff_check_launch("gemm_bf16_async");
+}
+
+// four waves in 2 x 2
 template <int WTM, int WTN, int STAGES, bool GLU = false>
 static int launch_async(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
                         int c_dtype, int n_out, hipStream_t s) {
-    const int KB = (K + 31) / 32;
-    const dim3 grid((M + WTM * 32 - 1) / (WTM * 32), (N + WTN * 32 - 1) / (WTN * 32));
-    TFF_REQUIRE(grid.y <= 65535, "gemm: too many columns N=%d", N);
-    if (c_dtype == TFF_F32)
-        gemm_bf16_async_kernel<WTM, WTN, STAGES, GLU, float><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
-    else
-        gemm_bf16_async_kernel<WTM, WTN, STAGES, GLU, bf16_t><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
-    return tff_check_launch("gemm_bf16_async");
+    return launch_async_g<2, 2, WTM, WTN, STAGES, GLU>(A, Wp, C, M, N, K, lda, c_dtype, n_out, s);
 }
 
 // ------------------------------------------------------------- skinny M ---
@@ -487,13 +498,15 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
                 "gemm: operands must be 16-byte aligned");
     TFF_REQUIRE(c_dtype == TFF_F32 || c_dtype == TFF_BF16, "gemm: unknown output type %d", c_dtype);
     // The choices below were measured at the sizes of an 8B model on an MI355X.
+    const long big_tiles = (long)((M + 255) / 256) * ((N + 255) / 256);
     if (glu_out > 0) {
         TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
                     "gemm: a gated weight of %d rows does not fit %d output columns", N, glu_out);
         if (M <= 16) return launch_skinny<1, 1, 32, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
-        if (M <= 64) return launch_async<2, 4, 4, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
-        if (M >= 1024 && N >= 8192) return launch_async<8, 8, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
-        return launch_async<4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
+        if (M < 128) return launch_async<2, 4, 4, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
+        if (M >= 512 && big_tiles >= 160)
+            return launch_async_g<4, 4, 4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
+        return launch_async_g<2, 4, 4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
     }
     if (M <= 16) {
         // more waves per block where there are few blocks (small N) or long rows (large K),
@@ -509,8 +522,10 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
         if (M <= 32) return launch_skinny<2, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
         return launch_skinny<4, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
     }
-    if (M >= 1024 && N >= 16 * 1024) return launch_async<8, 8, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
-    return launch_async<4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+    // 256 x 256 tiles on 16 waves where they still give most CUs a block, else 128 x 256 on 8
+    if (M < 128) return launch_async<2, 4, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+    if (M >= 512 && big_tiles >= 160) return launch_async_g<4, 4, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+    return launch_async_g<2, 4, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
 }
 
 int tff_gemm_f32(const float* A, const float* W, void* C, int M, int N, int K, int lda,
