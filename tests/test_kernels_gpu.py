@@ -407,6 +407,32 @@ def test_attention_mfma_prompt_portions_and_mixed(nq, nkv, d, ps, window):
     _close(gen.reshape(T, nq, d), ref, 1.5e-2, "generic attention on the same step")
 
 
+@pytest.mark.parametrize("nq,nkv,d,ps,window", [
+    (32, 8, 128, 16, 0), (8, 2, 32, 8, 300), (6, 3, 48, 8, 0), (5, 1, 128, 32, 0), (40, 2, 96, 8, 77),
+    (4, 2, 16, 16, 0), (3, 1, 256, 64, 0)])
+def test_attention_mfma_long_portions(nq, nkv, d, ps, window):
+    """Portions long enough for the kernel whose blocks share keys through LDS:
+    several blocks per request, a cached prefix, windows that start mid-page."""
+    ops = _ops()
+    entries = [(0, 700), (333, 200), (5, 1), (1000, 130)]
+    batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=nq * 7 + d)
+    T = batch.num_tokens
+    g = torch.Generator().manual_seed(4)
+    q = torch.randn(T, nq, d, generator=g).to(torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale)
+    # the general kernel is the yardstick here (it is checked against float64 above)
+    gen = ops.attention_generic(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv.k_cache, kv.v_cache, kv.block_tables,
+                                batch.token_req, batch.positions, window, scale)
+    _close(out, gen.double(), 1.5e-2, "block attention against the general kernel")
+    sel = torch.tensor([0, 1, 31, 32, 127, 128, 699, 700, 899, 900, 901, T - 1])
+    for r in range(len(entries)):
+        mine = sel[(token_req[sel] == r)]
+        if len(mine):
+            ref = _attn_ref(q[mine], ks[r], vs[r], positions[mine], window, scale)
+            _close(out.reshape(T, nq, d)[mine], ref, 1.5e-2, f"block attention, request {r}")
+
+
 @pytest.mark.parametrize("nq,nkv,d,ps,window,splits", [
     (32, 8, 128, 16, 0, None), (32, 8, 128, 16, 0, 1), (32, 8, 128, 16, 0, 7), (4, 2, 16, 16, 0, 3),
     (8, 2, 32, 8, 24, 4), (40, 2, 96, 8, 0, 5), (6, 3, 48, 8, 100, None), (16, 1, 64, 32, 0, 64)])

@@ -27,6 +27,19 @@
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* glb_ptr_t;
+// s_waitcnt immediate: vmcnt = 0, the other counters untouched
+constexpr int vmcnt_imm0() { return (7 << 4) | (15 << 8); }
+
+// Page and slot of a key; a shift and a mask when the page size is a power of two
+// (page_shift >= 0), a division otherwise (the GPU has no integer divider).
+__device__ __forceinline__ int page_index(int j, int page_size, int page_shift) {
+    return page_shift >= 0 ? (j >> page_shift) : j / page_size;
+}
+__device__ __forceinline__ int page_slot(int j, int page_size, int page_shift) {
+    return page_shift >= 0 ? (j & (page_size - 1)) : j % page_size;
+}
 
 template <int DT, int NQT, bool SPLIT>
 __global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
@@ -35,7 +48,7 @@ __global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int bt_stride,
     const int32_t* __restrict__ cu_tokens, const int32_t* __restrict__ start_pos,
     const int32_t* __restrict__ work, int tiles_per_entry, int nq, int nkv, int page_size,
-    int window, float scale, int T_total) {
+    int page_shift, int window, float scale, int T_total) {
     constexpr int D = DT * 16;
     constexpr int KS = (D + 31) / 32;
     const int lane = threadIdx.x, qc = lane & 15, kg = lane >> 4;
@@ -117,8 +130,8 @@ __global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
         _Pragma("unroll") for (int kt = 0; kt < 2; ++kt) {                                          \
             /* rows past the last key repeat it; they are masked */                                 \
             const int j_ = min(kb_ + kt * 16 + qc, kmax);                                           \
-            const int page_ = bt[j_ / page_size];                                                   \
-            const bf16_t* kp_ = k_cache + (((size_t)page_ * nkv + g) * page_size + (j_ % page_size)) * D; \
+            const int page_ = bt[page_index(j_, page_size, page_shift)];                            \
+            const bf16_t* kp_ = k_cache + (((size_t)page_ * nkv + g) * page_size + page_slot(j_, page_size, page_shift)) * D; \
             _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                     \
                 const int e_ = ks * 32 + kg * 8;                                                    \
                 uint4 v_ = make_uint4(0, 0, 0, 0);                                                  \
@@ -130,8 +143,8 @@ __global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
         const bf16_t* vrun_[2];                                                                     \
         _Pragma("unroll") for (int kt = 0; kt < 2; ++kt) {                                          \
             const int j0_ = min(kb_ + kt * 16 + kg * 4, (kmax / 4) * 4);                            \
-            const int page_ = bt[j0_ / page_size];                                                  \
-            vrun_[kt] = v_cache + ((size_t)page_ * nkv + g) * D * page_size + (j0_ % page_size);    \
+            const int page_ = bt[page_index(j0_, page_size, page_shift)];                           \
+            vrun_[kt] = v_cache + ((size_t)page_ * nkv + g) * D * page_size + page_slot(j0_, page_size, page_shift); \
         }                                                                                           \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                         \
             const size_t eoff_ = (size_t)(dt * 16 + qc) * page_size;                                \
@@ -287,6 +300,238 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __r
     }
 }
 
+// ------------------------------------------------- prompt portions, by block ---
+// For portions of many tokens a block of four waves shares its keys and values:
+// every 32-key slice is copied once from the pages into LDS (by the load unit,
+// global_load_lds_dwordx4, in MFMA operand order, two slices in flight) and read
+// from there by all four waves, each of which works on NQT column tiles.
+//
+// Within a slice the 16 rows of key tile t are the keys (r / 4) * 8 + t * 4 + r % 4:
+// lane (col, g) then holds the scores of the 8 consecutive keys g*8 .. g*8+7,
+// which makes the P.V operand of values one 16-byte run of a value page.
+#define ATTN_BT_LDS 2048
+#define ATTN_STAGES 4
+constexpr int attn_vmcnt_imm(int v) { return (v & 15) | (7 << 4) | (15 << 8) | ((v >> 4) << 14); }
+
+template <int DT, int NQT>
+__global__ __launch_bounds__(256, 2) void attn_mfma_block_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ block_tables, int bt_stride, const int32_t* __restrict__ cu_tokens,
+    const int32_t* __restrict__ start_pos, const int32_t* __restrict__ work, int nq, int nkv,
+    int page_size, int page_shift, int window, float scale) {
+    constexpr int D = DT * 16;
+    constexpr int KS = (D + 31) / 32;
+    constexpr int KFR = 2 * KS, VFR = DT, FR = KFR + VFR;   // 1 KB fragments per slice
+    constexpr int LPW = (FR + 3) / 4;                        // copies a wave issues per slice
+    constexpr int BCOLS = 4 * NQT * 16;                      // columns of a block
+    constexpr int STAGES = ATTN_STAGES;                      // slices in LDS: one in use, the rest in flight
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[STAGES * FR * 512];
+    __shared__ int32_t pages[ATTN_BT_LDS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int qc = lane & 15, kg = lane >> 4;
+    // the last blocks of a request see the most keys: they start first
+    const int bx = gridDim.x - 1 - blockIdx.x;
+    const int r = work[2 * bx];
+    const int bcol0 = work[2 * bx + 1];
+    const int g = blockIdx.y;
+    const int G = nq / nkv;
+    const int tok0 = cu_tokens[r];
+    const int n = cu_tokens[r + 1] - tok0;
+    const int P = start_pos[r];
+    const int ncols = n * G;
+    const int32_t* bt = block_tables + (size_t)r * bt_stride;
+    const int col0 = bcol0 + wave * (NQT * 16);   // this wave's first column
+
+    int c_tok[NQT], c_head[NQT], c_pos[NQT], c_lo[NQT];
+    bool c_ok[NQT];
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+        const int c = col0 + t * 16 + qc;
+        c_ok[t] = c < ncols;
+        const int cc = c_ok[t] ? c : ncols - 1;
+        const int tl = cc / G;
+        c_tok[t] = tok0 + tl;
+        c_head[t] = g * G + (cc - tl * G);
+        c_pos[t] = c_ok[t] ? P + tl : -1;
+        c_lo[t] = window > 0 ? max(0, P + tl - window + 1) : 0;
+    }
+    // keys any column of the block can see (the same for all four waves)
+    const int tl_first = bcol0 / G;
+    const int tl_last = (min(bcol0 + BCOLS, ncols) - 1) / G;
+    const int kmin = window > 0 ? max(0, P + tl_first - window + 1) : 0;
+    const int kmax = P + tl_last;
+    const int kb0 = (kmin / 32) * 32;
+    const int nsteps = (kmax - kb0) / 32 + 1;
+    // the block's part of the block table, once
+    const int pg0 = page_index(kb0, page_size, page_shift);
+    const int npg = page_index(kmax, page_size, page_shift) - pg0 + 1;
+    const bool bt_in_lds = npg <= ATTN_BT_LDS;
+    if (bt_in_lds)
+        for (int i = tid; i < npg; i += 256) pages[i] = bt[pg0 + i];
+
+    bf16x8 qf[NQT][KS];
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+        const bf16_t* qp = q + (size_t)c_tok[t] * q_stride + (size_t)c_head[t] * D;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int e = ks * 32 + kg * 8;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (c_ok[t] && e < D) v = *reinterpret_cast<const uint4*>(qp + e);   // zero past D: K may hold anything there
+            qf[t][ks] = *reinterpret_cast<bf16x8*>(&v);
+        }
+    }
+    floatx4 oacc[NQT][DT];
+    float m_run[NQT], l_run[NQT];
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+        m_run[t] = -INFINITY;
+        l_run[t] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) oacc[t][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    __syncthreads();   // pages[] is written
+
+#define ATTN_PAGE(j) (bt_in_lds ? pages[page_index((j), page_size, page_shift) - pg0] \
+                                : bt[page_index((j), page_size, page_shift)])
+    // fragment f of a slice: f < KFR is key tile f / KS, k-step f % KS; else value tile f - KFR
+    // Every wave issues LPW copies per slice, also past the last slice (clamped to it) and past
+    // the last fragment (a second copy of it): the count in flight is then the same for every
+    // wave and iteration, and one constant wait covers the slice about to be read.
+#define ATTN_ISSUE(step)                                                                            \
+    {                                                                                               \
+        const int kb_ = kb0 + min((step), nsteps - 1) * 32;                                         \
+        const int st_ = (step) % STAGES;                                                            \
+        _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                           \
+            const int f = min(wave + 4 * j, FR - 1);                                                \
+            {                                                                                       \
+                const bf16_t* g_;                                                                   \
+                if (f < KFR) {                                                                      \
+                    const int kt = f / KS, ks = f - kt * KS;                                        \
+                    const int key = min(kb_ + (qc >> 2) * 8 + kt * 4 + (qc & 3), kmax);             \
+                    g_ = k_cache + (((size_t)ATTN_PAGE(key) * nkv + g) * page_size +                 \
+                                    page_slot(key, page_size, page_shift)) * D +                      \
+                         min(ks * 32 + kg * 8, D - 8);                                              \
+                } else {                                                                            \
+                    const int j0 = min(kb_ + kg * 8, (kmax / 8) * 8);                               \
+                    g_ = v_cache + (((size_t)ATTN_PAGE(j0) * nkv + g) * D + (f - KFR) * 16 + qc) * page_size + \
+                         page_slot(j0, page_size, page_shift);                                      \
+                }                                                                                   \
+                __builtin_amdgcn_global_load_lds((glb_ptr_t)g_, (lds_ptr_t)(smem + (st_ * FR + f) * 512), 16, 0, 0); \
+            }                                                                                       \
+        }                                                                                           \
+    }
+
+    // The softmax works on raw scores with the scale folded into the exponent:
+    //   p = 2^((s - m) * scale * log2 e),
+    // masks only the slices that touch a column's causal or window edge, and rescales the
+    // accumulators only when some column's maximum moved: away from the diagonal the vector
+    // unit then has a fused multiply-add, an exponential and an addition per score to do.
+    const float sl2 = scale * 1.44269504088896f;
+    int t_min_pos[NQT], t_max_lo[NQT];
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+        int mn = c_pos[t], mx = c_lo[t];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            mn = min(mn, __shfl_xor(mn, o, 64));
+            mx = max(mx, __shfl_xor(mx, o, 64));
+        }
+        t_min_pos[t] = mn;
+        t_max_lo[t] = mx;
+    }
+
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) ATTN_ISSUE(s)
+    for (int s = 0; s < nsteps; ++s) {
+        __builtin_amdgcn_s_waitcnt(attn_vmcnt_imm((STAGES - 2) * LPW));   // this wave's copies of slice s are in
+        __syncthreads();                            // ... and the other waves'; slice s - 1 is read
+        ATTN_ISSUE(s + STAGES - 1)                  // into the stage of slice s - 1
+        const int kb = kb0 + s * 32;
+        const bf16_t* st = smem + (s % STAGES) * FR * 512;
+        floatx4 sacc[NQT][2];
+#pragma unroll
+        for (int t = 0; t < NQT; ++t) sacc[t][0] = sacc[t][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const bf16x8 kf = *reinterpret_cast<const bf16x8*>(st + (kt * KS + ks) * 512 + lane * 8);
+#pragma unroll
+                for (int t = 0; t < NQT; ++t)
+                    sacc[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[t][ks], sacc[t][kt], 0, 0, 0);
+            }
+        bf16x8 pf[NQT];
+#pragma unroll
+        for (int t = 0; t < NQT; ++t) {
+            float sv[8];
+            // lane (col, g): key kb + g*8 + e is row g*4 + e%4 of tile e/4
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sv[e] = sacc[t][e >> 2][e & 3];
+            if (kb + 31 > t_min_pos[t] || kb < t_max_lo[t]) {   // the slice touches an edge of some column
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int j = kb + kg * 8 + e;
+                    if (!(j >= c_lo[t] && j <= c_pos[t])) sv[e] = -INFINITY;
+                }
+            }
+            float mt = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
+                             fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+            mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            const float m_new = fmaxf(m_run[t], mt);          // maxima are kept in raw score units
+            const float mb = m_new == -INFINITY ? 0.f : m_new * sl2;
+            const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((m_run[t] - m_new) * sl2);
+            float ps = 0.f;
+            bf16x8 pv;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float p = __builtin_amdgcn_exp2f(fmaf(sv[e], sl2, -mb));   // 2^-inf = 0 for masked scores
+                ps += p;
+                pv[e] = (bf16_t)p;
+            }
+            pf[t] = pv;
+            l_run[t] = l_run[t] * alpha + ps;
+            m_run[t] = m_new;
+            if (__any(alpha != 1.f)) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    oacc[t][dt][0] *= alpha; oacc[t][dt][1] *= alpha;
+                    oacc[t][dt][2] *= alpha; oacc[t][dt][3] *= alpha;
+                }
+            }
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const bf16x8 vfr = *reinterpret_cast<const bf16x8*>(st + (KFR + dt) * 512 + lane * 8);
+#pragma unroll
+            for (int t = 0; t < NQT; ++t)
+                oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfr, pf[t], oacc[t][dt], 0, 0, 0);
+        }
+    }
+#undef ATTN_ISSUE
+#undef ATTN_PAGE
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm0());   // the copies past the end must not outlive the block
+
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+        float l = l_run[t];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        if (!c_ok[t]) continue;
+        const float inv = 1.0f / l;
+        bf16_t* op = out + ((size_t)c_tok[t] * nq + c_head[t]) * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            union { bf16_t h[4]; uint2 u; } pk;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pk.h[i] = (bf16_t)(oacc[t][dt][i] * inv);
+            *reinterpret_cast<uint2*>(op + dt * 16 + kg * 4) = pk.u;
+        }
+    }
+}
+
 template <int DT>
 static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o, float* part_ml,
                        const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* block_tables,
@@ -294,10 +539,19 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
                        const int32_t* work, int num_work, int tiles_per_entry, int cols_per_wave,
                        int splits, int nq, int nkv, int page_size, int window, float scale,
                        int T_total, hipStream_t s) {
+    int page_shift = -1;
+    if ((page_size & (page_size - 1)) == 0)
+        for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
+    if (cols_per_wave == 128) {   // blocks of four waves, two column tiles each
+        attn_mfma_block_kernel<DT, 2><<<dim3(num_work, nkv), 256, 0, s>>>(
+            q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work, nq,
+            nkv, page_size, page_shift, window, scale);
+        return tff_check_launch("attention_mfma_block");
+    }
     const dim3 grid(num_work, nkv, splits);
 #define TFF_ATTN_ARGS                                                                              \
     q, q_stride, out, part_o, part_ml, k_cache, v_cache, block_tables, bt_stride, cu_tokens,       \
-        start_pos, work, tiles_per_entry, nq, nkv, page_size, window, scale, T_total
+        start_pos, work, tiles_per_entry, nq, nkv, page_size, page_shift, window, scale, T_total
     if (splits > 1) {
         if (cols_per_wave == 16)
             attn_mfma_kernel<DT, 1, true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
@@ -339,7 +593,10 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                 "kernel (head sizes 16..128 in steps of 16, 192, 256; pages a multiple of 8)", d, page_size);
     TFF_REQUIRE(q_stride >= nq * d && q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0,
                 "attention_mfma: query rows must be 16-byte aligned (stride %d)", q_stride);
-    TFF_REQUIRE(cols_per_wave == 16 || cols_per_wave == 32, "attention_mfma: bad tile width %d", cols_per_wave);
+    TFF_REQUIRE(cols_per_wave == 16 || cols_per_wave == 32 || cols_per_wave == 128,
+                "attention_mfma: bad tile width %d", cols_per_wave);
+    TFF_REQUIRE(cols_per_wave != 128 || (work && splits == 1),
+                "attention_mfma: blocks of 128 columns take a work table and no key split");
     TFF_REQUIRE(splits >= 1 && splits <= 65535 && nkv <= 65535, "attention_mfma: bad split count %d", splits);
     TFF_REQUIRE(splits == 1 || (part_o && part_ml), "attention_mfma: split keys need a workspace");
     TFF_REQUIRE(work || tiles_per_entry >= 1, "attention_mfma: neither a work table nor a tile count");

@@ -370,7 +370,9 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
             part_ml = torch.empty(splits, T, nq, 2, dtype=torch.float32, device=q.device)
     else:
         tiles, splits = 1, 1
-        cols = 32 if batch.max_new_tokens * G > 16 else 16
+        # long portions: blocks of four waves that share their keys through LDS (128 columns);
+        # short ones: a wave of its own per 32 or 16 columns
+        cols = 128 if batch.max_new_tokens * G > 64 else (32 if batch.max_new_tokens * G > 16 else 16)
         work = _attention_work(batch, G, cols, q.device)
         num_work = work.shape[0]
     dest = out
