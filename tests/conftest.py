@@ -19,3 +19,11 @@ def model_dirs(tmp_path_factory):
     from helpers import TINY_CONFIGS, make_model_dir
     base = tmp_path_factory.mktemp("models")
     return {name: make_model_dir(str(base / name), cfg, seed) for name, (cfg, seed) in TINY_CONFIGS.items()}
+
+
+@pytest.fixture(autouse=True)
+def _seeded():
+    """Every test draws the same random inputs in every run."""
+    import torch
+    torch.manual_seed(1234)
+    yield

@@ -306,6 +306,142 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     }
 }
 
+// ------------------------------------------ tiled, async copy, k-steps of 32 ---
+// For large wave tiles (up to 128 x 128 per wave) LDS bandwidth and latency
+// decide: a stage holds one k-step (32 k) only, so four stages fit beside
+// 256 x 256 tiles, and a wave reads the operands of k-step kt + 1 into a second
+// set of registers while the matrix cores work on k-step kt.  One barrier per
+// k-step: after it, the copies of k-step kt + 1 are visible to all, and the
+// stage of k-step kt - 1 is free for the copy of k-step kt + STAGES - 1.
+template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU, typename TC>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_pipe_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
+    int K, int lda, int KB, int n_out) {
+    constexpr int NW = WGM * WGN;
+    constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
+    constexpr int AF = BM / 16, WF = BN / 16;   // fragments per stage and operand (one k-step)
+    constexpr int FR = AF + WF;
+    constexpr int LPW = FR / NW;
+    static_assert(FR % NW == 0, "fragments are dealt to the waves evenly");
+    static_assert(STAGES >= 3 && (STAGES - 3) * LPW < 64, "vmcnt has 6 bits");
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[STAGES * FR * 512];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int fr = lane & 15, fg = lane >> 4;
+    const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+    const int NB = (N + 15) / 16;
+
+    floatx4 acc[WTN][WTM];
+#pragma unroll
+    for (int i = 0; i < WTN; ++i)
+#pragma unroll
+        for (int j = 0; j < WTM; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const bf16_t* src[LPW];
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) {
+        const int f = wave + NW * j;
+        if (f < AF) src[j] = A + (size_t)min(m0 + f * 16 + fr, M - 1) * lda;
+        else src[j] = Wp + (size_t)min(n0 / 16 + (f - AF), NB - 1) * KB * 512 + lane * 8;
+    }
+    // k-steps past the end are copied as the last one (into stages nobody reads any more), so
+    // that the number of copies in flight is the same in every iteration
+#define TFF_ISSUE_STEP(step)                                                                       \
+    {                                                                                              \
+        const int ks_ = min((step), KB - 1);                                                       \
+        const int st_ = (step) % STAGES;                                                           \
+        _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                          \
+            const int f = wave + NW * j;                                                           \
+            const bf16_t* g_ = f < AF ? src[j] + min(ks_ * 32 + fg * 8, K - 8)                     \
+                                      : src[j] + (size_t)ks_ * 512;                                \
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)g_, (lds_ptr_t)(smem + (st_ * FR + f) * 512), 16, 0, 0); \
+        }                                                                                          \
+    }
+#define TFF_READ_FRAGS(step, FW, FA)                                                               \
+    {                                                                                              \
+        const bf16_t* st_ = smem + ((step) % STAGES) * FR * 512;                                   \
+        _Pragma("unroll") for (int i = 0; i < WTN; ++i)                                            \
+            FW[i] = *reinterpret_cast<const bf16x8*>(st_ + (AF + wn * WTN + i) * 512 + lane * 8);  \
+        _Pragma("unroll") for (int j = 0; j < WTM; ++j)                                            \
+            FA[j] = *reinterpret_cast<const bf16x8*>(st_ + (wm * WTM + j) * 512 + lane * 8);       \
+    }
+#define TFF_MFMA_STEP(FW, FA)                                                                      \
+    {                                                                                              \
+        _Pragma("unroll") for (int i = 0; i < WTN; ++i)                                            \
+            _Pragma("unroll") for (int j = 0; j < WTM; ++j)                                        \
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(FW[i], FA[j], acc[i][j], 0, 0, 0); \
+    }
+
+    bf16x8 fw0[WTN], fa0[WTM], fw1[WTN], fa1[WTM];
+#pragma unroll
+    for (int t = 0; t < STAGES - 1; ++t) TFF_ISSUE_STEP(t)
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * LPW));   // k-step 0 is in
+    __syncthreads();
+    TFF_READ_FRAGS(0, fw0, fa0)
+    // two k-steps per trip so that the register sets swap without copies
+    for (int kt = 0; kt < KB; kt += 2) {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * LPW));   // k-step kt + 1 is in
+        __syncthreads();
+        TFF_ISSUE_STEP(kt + STAGES - 1)
+        TFF_READ_FRAGS(kt + 1, fw1, fa1)
+        TFF_MFMA_STEP(fw0, fa0)
+        if (kt + 1 < KB) {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * LPW));
+            __syncthreads();
+            TFF_ISSUE_STEP(kt + STAGES)
+            TFF_READ_FRAGS(kt + 2, fw0, fa0)
+            TFF_MFMA_STEP(fw1, fa1)
+        }
+    }
+#undef TFF_ISSUE_STEP
+#undef TFF_READ_FRAGS
+#undef TFF_MFMA_STEP
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));   // the copies past the end must not outlive the block
+
+    if constexpr (GLU) {
+        static_assert(WTN % 2 == 0, "gate and up groups come in pairs");
+        const bool vec = (n_out % 4) == 0;
+#pragma unroll
+        for (int i = 0; i < WTN; i += 2) {
+            const int n = (n0 + (wn * WTN + i) * 16) / 2 + fg * 4;
+#pragma unroll
+            for (int j = 0; j < WTM; ++j) {
+                const int m = m0 + (wm * WTM + j) * 16 + fr;
+                if (m < M && n < n_out)
+                    store4<TC>(C + (size_t)m * n_out + n, silu_mul(acc[i][j], acc[i + 1][j]), n, n_out, vec);
+            }
+        }
+    } else {
+        const bool vec = (N % 4) == 0;
+#pragma unroll
+        for (int i = 0; i < WTN; ++i) {
+            const int n = n0 + (wn * WTN + i) * 16 + fg * 4;
+#pragma unroll
+            for (int j = 0; j < WTM; ++j) {
+                const int m = m0 + (wm * WTM + j) * 16 + fr;
+                if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, acc[i][j], n, N, vec);
+            }
+        }
+    }
+}
+
+template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU = false>
+static int launch_pipe(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
+                       int c_dtype, int n_out, hipStream_t s) {
+    const int KB = (K + 31) / 32;
+    constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
+    const dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN);
+    TFF_REQUIRE(grid.y <= 65535, "gemm: too many columns N=%d", N);
+    if (c_dtype == TFF_F32)
+        gemm_bf16_pipe_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, float>
+            <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
+    else
+        gemm_bf16_pipe_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, bf16_t>
+            <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
+    return tff_check_launch("gemm_bf16_pipe");
+}
+
 template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU = false>
 static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
                           int c_dtype, int n_out, hipStream_t s) {
@@ -345,7 +481,7 @@ static int launch_async(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N
 // that, not W, is most of a wave's traffic.  With GLU, sets 2p and 2p+1 hold a
 // gate group and the up group that follows it in W; the epilogue writes
 // silu(gate) * up.
-template <int MT, int R, int UNROLL, int KSPLIT, int NSETS, bool GLU, typename TC>
+template <int MT, int R, int UNROLL, int KSPLIT, int NSETS, bool GLU, typename TC, bool RING = false>
 __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
     int K, int lda, int KB, int n_out) {
@@ -380,7 +516,44 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
 
     const int full_end = min(s_end, K / 32);   // steps below K / 32 have all their 32 k in A
     int s0 = s_begin;
-    for (; s0 + UNROLL <= full_end; s0 += UNROLL) {
+    if constexpr (RING) {
+        // A ring of UNROLL k-steps in registers: a slot is loaded again as soon as it has been
+        // used, so the wave has UNROLL * (R + MT) KB in flight from its first step to its last.
+        // Loads come back in order, so the wait before a slot's use leaves the younger ones in
+        // flight.  Steps past the end load the last step again and are not used.
+        if (s0 < full_end) {
+            uint4 rw[UNROLL][R], ra[UNROLL][MT];
+            const int last = full_end - 1;
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int st = min(s0 + u, last);
+#pragma unroll
+                for (int r = 0; r < R; ++r) rw[u][r] = ld16(wfrag[r] + (size_t)st * 512);
+#pragma unroll
+                for (int t = 0; t < MT; ++t) ra[u][t] = ld16(arow[t] + st * 32 + fg * 8);
+            }
+            for (; s0 < full_end; s0 += UNROLL) {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    if (s0 + u < full_end) {
+#pragma unroll
+                        for (int r = 0; r < R; ++r)
+#pragma unroll
+                            for (int t = 0; t < MT; ++t)
+                                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                    as_frag(rw[u][r]), as_frag(ra[u][t]), acc[r][t], 0, 0, 0);
+                    }
+                    const int st = min(s0 + UNROLL + u, last);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) rw[u][r] = ld16(wfrag[r] + (size_t)st * 512);
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) ra[u][t] = ld16(arow[t] + st * 32 + fg * 8);
+                }
+            }
+            s0 = full_end;
+        }
+    }
+    for (; !RING && s0 + UNROLL <= full_end; s0 += UNROLL) {
         uint4 rw[UNROLL][R], ra[UNROLL][MT];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
@@ -459,17 +632,17 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
     }
 }
 
-template <int MT, int R, int UNROLL, int KSPLIT, int NSETS = 1, bool GLU = false>
+template <int MT, int R, int UNROLL, int KSPLIT, int NSETS = 1, bool GLU = false, bool RING = false>
 static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
                          int c_dtype, int n_out, hipStream_t s) {
     const int NB = (N + 15) / 16, KB = (K + 31) / 32;
     const int per_block = NSETS * R;
     const dim3 grid((NB + per_block - 1) / per_block);
     if (c_dtype == TFF_F32)
-        gemm_bf16_skinny_kernel<MT, R, UNROLL, KSPLIT, NSETS, GLU, float>
+        gemm_bf16_skinny_kernel<MT, R, UNROLL, KSPLIT, NSETS, GLU, float, RING>
             <<<grid, 64 * KSPLIT * NSETS, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
     else
-        gemm_bf16_skinny_kernel<MT, R, UNROLL, KSPLIT, NSETS, GLU, bf16_t>
+        gemm_bf16_skinny_kernel<MT, R, UNROLL, KSPLIT, NSETS, GLU, bf16_t, RING>
             <<<grid, 64 * KSPLIT * NSETS, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
     return tff_check_launch("gemm_bf16_skinny");
 }
@@ -502,7 +675,12 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
     if (glu_out > 0) {
         TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
                     "gemm: a gated weight of %d rows does not fit %d output columns", N, glu_out);
-        if (M <= 16) return launch_skinny<1, 1, 32, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
+        if (M <= 16) {
+            // with a thousand row groups and more, a wave takes a group's whole K through a ring
+            if (N >= 16 * 1024)
+                return launch_skinny<1, 1, 8, 1, 2, true, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
+            return launch_skinny<1, 1, 32, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
+        }
         if (M < 128) return launch_async<2, 4, 4, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
         if (M >= 512 && big_tiles >= 160)
             return launch_async_g<4, 4, 4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);

@@ -37,7 +37,33 @@ __device__ __forceinline__ int block_argmax(const float* __restrict__ x, int V, 
                                             int* redi, float* max_out) {
     float best = -INFINITY;
     int arg = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+    // One block reads the whole row, so what counts is loads in flight: eight 16-byte loads
+    // per thread are issued before the first is compared.
+    const int head = min(V, (int)(((16 - ((uintptr_t)x & 15)) & 15) / 4));   // up to a 16-byte boundary
+    const int nvec = (V - head) / 4;
+    const float4* x4 = reinterpret_cast<const float4*>(x + head);
+    constexpr int UN = 8;
+    for (int i0 = threadIdx.x; i0 < nvec; i0 += UN * blockDim.x) {
+        float4 v[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int j = i0 + u * blockDim.x;
+            v[u] = x4[min(j, nvec - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int j = i0 + u * blockDim.x;
+            if (j < nvec) {
+                const int i = head + 4 * j;
+                if (v[u].x > best || (v[u].x == best && i < arg)) { best = v[u].x; arg = i; }
+                if (v[u].y > best || (v[u].y == best && i + 1 < arg)) { best = v[u].y; arg = i + 1; }
+                if (v[u].z > best || (v[u].z == best && i + 2 < arg)) { best = v[u].z; arg = i + 2; }
+                if (v[u].w > best || (v[u].w == best && i + 3 < arg)) { best = v[u].w; arg = i + 3; }
+            }
+        }
+    }
+    for (int t = threadIdx.x; t < V - 4 * nvec; t += blockDim.x) {   // before and after the 16-byte part
+        const int i = t < head ? t : t + 4 * nvec;
         const float v = x[i];
         if (v > best || (v == best && i < arg)) { best = v; arg = i; }
     }
