@@ -271,6 +271,213 @@ __global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
     }
 }
 
+// ------------------------------------------------ one column tile per wave ---
+// Decoding (and portions of a few tokens): one wave, 16 columns.  What counts
+// here is bytes in flight.  The wave's part of the block table goes to LDS
+// first, so that no page number is waited for among the loads of keys and
+// values (loads come back in order: a wait for a page number would be a wait
+// for every load issued before it).  Keys and values of RING steps of 32 keys
+// are in flight at any time: a step's registers are loaded again as soon as
+// its arithmetic is done.  Within a step the 16 rows of key tile t are the keys
+// (r / 4) * 8 + t * 4 + r % 4, so lane (col, g) holds the scores of the eight
+// consecutive keys g*8 .. g*8+7 and reads its values as one 16-byte run.
+#define ATTN_WAVE_BT 1024
+template <int DT, bool SPLIT, int RING>
+__global__ __launch_bounds__(64, 1) void attn_wave_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int bt_stride,
+    const int32_t* __restrict__ cu_tokens, const int32_t* __restrict__ start_pos,
+    const int32_t* __restrict__ work, int tiles_per_entry, int nq, int nkv, int page_size,
+    int page_shift, int window, float scale, int T_total) {
+    constexpr int D = DT * 16;
+    constexpr int KS = (D + 31) / 32;
+    __shared__ int32_t bt_lds[ATTN_WAVE_BT];
+    const int lane = threadIdx.x, qc = lane & 15, kg = lane >> 4;
+    int r, col0;
+    if (work) {
+        r = work[2 * blockIdx.x];
+        col0 = work[2 * blockIdx.x + 1];
+    } else {
+        r = blockIdx.x / tiles_per_entry;
+        col0 = (blockIdx.x % tiles_per_entry) * 16;
+    }
+    const int g = blockIdx.y;
+    const int G = nq / nkv;
+    const int tok0 = cu_tokens[r];
+    const int n = cu_tokens[r + 1] - tok0;
+    const int P = start_pos[r];
+    const int ncols = n * G;
+    const int32_t* bt = block_tables + (size_t)r * bt_stride;
+
+    const int c = col0 + qc;
+    const bool c_ok = c < ncols;
+    const int cc = c_ok ? c : ncols - 1;
+    const int tl = cc / G;
+    const int c_tok = tok0 + tl;
+    const int c_head = g * G + (cc - tl * G);
+    const int c_pos = c_ok ? P + tl : -1;   // a missing column sees no key
+    const int c_lo = window > 0 ? max(0, P + tl - window + 1) : 0;
+    // keys any column of this wave can see
+    const int tl_first = col0 / G;
+    const int tl_last = (min(col0 + 16, ncols) - 1) / G;
+    const int kmin = window > 0 ? max(0, P + tl_first - window + 1) : 0;
+    const int kmax = P + tl_last;
+    const int kb0 = (kmin / 32) * 32;
+    const int nsteps = (kmax - kb0) / 32 + 1;
+    int s_begin = 0, s_end = nsteps;
+    if (SPLIT) {
+        const int per = (nsteps + (int)gridDim.z - 1) / (int)gridDim.z;
+        s_begin = (int)blockIdx.z * per;
+        s_end = min(nsteps, s_begin + per);
+    }
+
+    // the page numbers of this wave's keys
+    int pi0 = 0;
+    bool bt_in_lds = false;
+    if (s_begin < s_end) {
+        pi0 = page_index(kb0 + s_begin * 32, page_size, page_shift);
+        const int pi1 = page_index(min(kmax, kb0 + s_end * 32 - 1), page_size, page_shift);
+        bt_in_lds = pi1 - pi0 < ATTN_WAVE_BT;
+        if (bt_in_lds)
+            for (int i = lane; i <= pi1 - pi0; i += 64) bt_lds[i] = bt[pi0 + i];
+    }
+    __syncthreads();
+
+    bf16x8 qf[KS];
+    {
+        const bf16_t* qp = q + (size_t)c_tok * q_stride + (size_t)c_head * D;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int e = ks * 32 + kg * 8;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (c_ok && e < D) v = *reinterpret_cast<const uint4*>(qp + e);
+            qf[ks] = *reinterpret_cast<bf16x8*>(&v);
+        }
+    }
+
+    floatx4 oacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    bf16x8 kf[RING][2][KS];   // [ring slot][key tile][k-step]
+    bf16x8 vf[RING][DT];
+
+#define TFF_WAVE_PAGE(j) (bt_in_lds ? bt_lds[page_index((j), page_size, page_shift) - pi0]          \
+                                    : bt[page_index((j), page_size, page_shift)])
+#define TFF_WAVE_LOAD(buf, step)                                                                    \
+    {                                                                                               \
+        const int kb_ = kb0 + (step) * 32;                                                          \
+        _Pragma("unroll") for (int kt = 0; kt < 2; ++kt) {                                          \
+            /* rows past the last key repeat it; they are masked */                                 \
+            const int j_ = min(kb_ + (qc >> 2) * 8 + kt * 4 + (qc & 3), kmax);                      \
+            const int page_ = TFF_WAVE_PAGE(j_);                                                    \
+            const bf16_t* kp_ = k_cache + (((size_t)page_ * nkv + g) * page_size + page_slot(j_, page_size, page_shift)) * D; \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                     \
+                const int e_ = ks * 32 + kg * 8;                                                    \
+                uint4 v_ = make_uint4(0, 0, 0, 0);                                                  \
+                if (e_ < D) v_ = *reinterpret_cast<const uint4*>(kp_ + e_);                         \
+                kf[buf][kt][ks] = *reinterpret_cast<bf16x8*>(&v_);                                  \
+            }                                                                                       \
+        }                                                                                           \
+        /* the values of keys kb + g*8 .. +7: a run of 16 bytes in a page (pages hold a multiple */ \
+        /* of 8 keys); a run past the last key is read from the last key's run and masked */       \
+        const int j0_ = min(kb_ + kg * 8, (kmax >> 3) << 3);                                        \
+        const int vpage_ = TFF_WAVE_PAGE(j0_);                                                      \
+        const bf16_t* vrun_ = v_cache + ((size_t)vpage_ * nkv + g) * D * page_size + page_slot(j0_, page_size, page_shift); \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                         \
+            const uint4 v_ = *reinterpret_cast<const uint4*>(vrun_ + (size_t)(dt * 16 + qc) * page_size); \
+            vf[buf][dt] = *reinterpret_cast<const bf16x8*>(&v_);                                    \
+        }                                                                                           \
+    }
+#define TFF_WAVE_COMPUTE(buf, step)                                                                 \
+    {                                                                                               \
+        const int kb_ = kb0 + (step) * 32;                                                          \
+        floatx4 sacc_[2];                                                                           \
+        sacc_[0] = sacc_[1] = floatx4{0.f, 0.f, 0.f, 0.f};                                          \
+        _Pragma("unroll") for (int kt = 0; kt < 2; ++kt)                                            \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                       \
+                sacc_[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[buf][kt][ks], qf[ks], sacc_[kt], 0, 0, 0); \
+        float sv_[8];                                                                               \
+        float mt_ = -INFINITY;                                                                      \
+        _Pragma("unroll") for (int kt = 0; kt < 2; ++kt)                                            \
+            _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                         \
+                const int j = kb_ + kg * 8 + kt * 4 + i;                                            \
+                const bool vis = j >= c_lo && j <= c_pos;                                           \
+                const float x = vis ? sacc_[kt][i] * scale : -INFINITY;                             \
+                sv_[kt * 4 + i] = x;                                                                \
+                mt_ = fmaxf(mt_, x);                                                                \
+            }                                                                                       \
+        mt_ = fmaxf(mt_, __shfl_xor(mt_, 16, 64));                                                  \
+        mt_ = fmaxf(mt_, __shfl_xor(mt_, 32, 64));                                                  \
+        const float m_new_ = fmaxf(m_run, mt_);                                                     \
+        const float alpha_ = m_new_ == -INFINITY ? 1.f : __expf(m_run - m_new_);                    \
+        float ps_ = 0.f;                                                                            \
+        bf16x8 pv_;                                                                                 \
+        _Pragma("unroll") for (int e = 0; e < 8; ++e) {                                             \
+            const float p = sv_[e] == -INFINITY ? 0.f : __expf(sv_[e] - m_new_);                    \
+            ps_ += p;                                                                               \
+            pv_[e] = (bf16_t)p;                                                                     \
+        }                                                                                           \
+        l_run = l_run * alpha_ + ps_;                                                               \
+        m_run = m_new_;                                                                             \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                         \
+            oacc[dt][0] *= alpha_; oacc[dt][1] *= alpha_;                                           \
+            oacc[dt][2] *= alpha_; oacc[dt][3] *= alpha_;                                           \
+        }                                                                                           \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt)                                           \
+            oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[buf][dt], pv_, oacc[dt], 0, 0, 0); \
+    }
+
+    if (s_begin < s_end) {
+        // steps past the end load the last step again and are not used
+#pragma unroll
+        for (int u = 0; u < RING; ++u) TFF_WAVE_LOAD(u, min(s_begin + u, s_end - 1))
+        int s = s_begin;
+        for (; s_end - s > RING; s += RING) {
+#pragma unroll
+            for (int u = 0; u < RING; ++u) {
+                TFF_WAVE_COMPUTE(u, s + u)
+                TFF_WAVE_LOAD(u, min(s + u + RING, s_end - 1))
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < RING; ++u)
+            if (s + u < s_end) TFF_WAVE_COMPUTE(u, s + u)
+    }
+#undef TFF_WAVE_PAGE
+#undef TFF_WAVE_LOAD
+#undef TFF_WAVE_COMPUTE
+
+    float l = l_run;
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!c_ok) return;
+    if (SPLIT) {
+        const size_t row = ((size_t)blockIdx.z * T_total + c_tok) * nq + c_head;
+        float* po = part_o + row * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            *reinterpret_cast<float4*>(po + dt * 16 + kg * 4) =
+                make_float4(oacc[dt][0], oacc[dt][1], oacc[dt][2], oacc[dt][3]);
+        if (kg == 0) {
+            part_ml[row * 2] = m_run;
+            part_ml[row * 2 + 1] = l;
+        }
+    } else {
+        const float inv = 1.0f / l;
+        bf16_t* op = out + ((size_t)c_tok * nq + c_head) * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            union { bf16_t h[4]; uint2 u; } pk;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pk.h[i] = (bf16_t)(oacc[dt][i] * inv);
+            *reinterpret_cast<uint2*>(op + dt * 16 + kg * 4) = pk.u;
+        }
+    }
+}
+
 // merges the partial results of the key splits:
 //   m = max m_s, l = sum l_s e^(m_s - m), o = sum o_s e^(m_s - m) / l
 __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __restrict__ part_o,
@@ -554,12 +761,12 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
         start_pos, work, tiles_per_entry, nq, nkv, page_size, page_shift, window, scale, T_total
     if (splits > 1) {
         if (cols_per_wave == 16)
-            attn_mfma_kernel<DT, 1, true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
+            attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
         else
             attn_mfma_kernel<DT, 2, true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
     } else {
         if (cols_per_wave == 16)
-            attn_mfma_kernel<DT, 1, false><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
+            attn_wave_kernel<DT, false, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
         else
             attn_mfma_kernel<DT, 2, false><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
     }
