@@ -82,7 +82,7 @@ def test_rmsnorm_eps_position():
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 320, 96), (33, 200, 200), (130, 130, 72), (257, 96, 256),
-                                    (64, 4096, 512), (300, 1000, 1024)])
+                                    (64, 4096, 512), (300, 1000, 1024), (50, 203, 1000), (40, 1024, 2056)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_linear(M, N, K, dtype):
     ops = _ops()
@@ -435,7 +435,8 @@ def test_attention_mfma_long_portions(nq, nkv, d, ps, window):
 
 @pytest.mark.parametrize("nq,nkv,d,ps,window,splits", [
     (32, 8, 128, 16, 0, None), (32, 8, 128, 16, 0, 1), (32, 8, 128, 16, 0, 7), (4, 2, 16, 16, 0, 3),
-    (8, 2, 32, 8, 24, 4), (40, 2, 96, 8, 0, 5), (6, 3, 48, 8, 100, None), (16, 1, 64, 32, 0, 64)])
+    (8, 2, 32, 8, 24, 4), (40, 2, 96, 8, 0, 5), (6, 3, 48, 8, 100, None), (16, 1, 64, 32, 0, 64),
+    (4, 2, 192, 16, 0, 3), (2, 1, 256, 8, 0, None)])
 def test_attention_mfma_decode_split_keys(nq, nkv, d, ps, window, splits):
     ops = _ops()
     entries = [(0, 1), (1, 1), (31, 1), (32, 1), (700, 1), (255, 1), (64, 1)]
@@ -448,6 +449,27 @@ def test_attention_mfma_decode_split_keys(nq, nkv, d, ps, window, splits):
                        for r in range(T)])
     out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale, splits=splits)
     _close(out.reshape(T, nq, d), ref, 1.5e-2, "split-key decode attention")
+
+
+@pytest.mark.parametrize("splits", [1, 2, 5])
+def test_attention_mfma_decode_more_pages_than_the_wave_keeps(splits):
+    """A wave keeps 1024 page numbers at hand; with more pages in its run of keys it reads
+    them from the table in memory.  One key far back is made to dominate."""
+    ops = _ops()
+    nq, nkv, d, ps = 4, 2, 32, 8
+    P, far = 8300, 77
+    entries = [(P, 1), (40, 1)]
+    batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=21)
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(2, nq, d, generator=g).to(torch.bfloat16)
+    kfar = (30 * q[0, 0].float() / q[0, 0].float().norm()).to(torch.bfloat16)
+    kv.k_cache[int(kv.block_tables[0, far // ps]), 0, far % ps] = kfar.to(DEV)
+    ks[0][far, 0] = kfar
+    scale = 1 / math.sqrt(d)
+    ref = torch.stack([_attn_ref(q[r:r + 1], ks[r], vs[r], positions[r:r + 1], 0, scale)[0] for r in range(2)])
+    out = ops.attention_mfma(q.reshape(2, nq * d).to(DEV), nq, nkv, d, kv, batch, 0, scale, splits=splits)
+    _close(out.reshape(2, nq, d), ref, 1.5e-2, "decode attention over 1038 pages")
+    assert torch.allclose(out.reshape(2, nq, d)[0, 0].float().cpu(), vs[0][far, 0].float(), atol=5e-2)
 
 
 def test_attention_mfma_far_key_and_window_edge():

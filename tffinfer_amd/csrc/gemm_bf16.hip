@@ -198,7 +198,7 @@ constexpr int vmcnt_imm(int v) { return (v & 15) | (7 << 4) | (15 << 8) | ((v >>
 template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU, typename TC>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
-    int K, int lda, int KB, int n_out) {
+    int K, int lda, int KB, int n_out, float* __restrict__ part) {
     // WGM x WGN waves, each WTM x WTN MFMA tiles of 16 x 16
     constexpr int NW = WGM * WGN;
     constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
@@ -215,6 +215,11 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
     const int NB = (N + 15) / 16;
     const int nk = (K + 63) / 64;
+    // With gridDim.z > 1 the blocks of one tile split K among them and leave partial sums in
+    // part[z][M][N], which a second kernel adds up in a fixed order.
+    const int kt_per = (nk + (int)gridDim.z - 1) / (int)gridDim.z;
+    const int kt0 = (int)blockIdx.z * kt_per;
+    const int kt1 = min(nk, kt0 + kt_per);
 
     floatx4 acc[WTN][WTM];
 #pragma unroll
@@ -241,7 +246,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
 #define TFF_ISSUE_TILE(tile)                                                                       \
     {                                                                                              \
         const int kt_ = min((tile), nk - 1);                                                       \
-        const int st_ = (tile) % STAGES;                                                           \
+        const int st_ = ((tile) - kt0) % STAGES;                                                   \
         _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                          \
             const int f = wave + NW * j;                                                            \
             const bf16_t* g_;                                                                      \
@@ -252,12 +257,12 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     }
 
 #pragma unroll
-    for (int t = 0; t < STAGES - 1; ++t) TFF_ISSUE_TILE(t)
-    for (int kt = 0; kt < nk; ++kt) {
+    for (int t = 0; t < STAGES - 1; ++t) TFF_ISSUE_TILE(kt0 + t)
+    for (int kt = kt0; kt < kt1; ++kt) {
         __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * LPW));   // this wave's part of tile kt is in
         __syncthreads();                                             // ... and everybody else's
         TFF_ISSUE_TILE(kt + STAGES - 1)                              // into the stage read last iteration
-        const bf16_t* st = smem + (kt % STAGES) * FR * 512;
+        const bf16_t* st = smem + ((kt - kt0) % STAGES) * FR * 512;
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             if (2 * kt + ks < KB) {   // k-steps past the end of K are not in W
@@ -279,6 +284,20 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
 #undef TFF_ISSUE_TILE
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));   // the copies past the end must not outlive the block
 
+    if (part) {   // partial sums over this block's share of K, columns as W has them
+        float* P = part + (size_t)blockIdx.z * M * N;
+        const bool vec = (N % 4) == 0;
+#pragma unroll
+        for (int i = 0; i < WTN; ++i) {
+            const int n = n0 + (wn * WTN + i) * 16 + fg * 4;
+#pragma unroll
+            for (int j = 0; j < WTM; ++j) {
+                const int m = m0 + (wm * WTM + j) * 16 + fr;
+                if (m < M && n < N) store4<float>(P + (size_t)m * N + n, acc[i][j], n, N, vec);
+            }
+        }
+        return;
+    }
     if constexpr (GLU) {
         static_assert(WTN % 2 == 0, "gate and up groups come in pairs");
         const bool vec = (n_out % 4) == 0;
@@ -304,6 +323,46 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
             }
         }
     }
+}
+
+// Adds up the partial sums part[s][M][N] of a product whose blocks split K, s = 0, 1, ... in
+// turn, and writes C; with GLU, columns come as gate and up groups of 16 in turn and
+// C[m][j] = silu(gate) * up.  One thread makes four neighbouring outputs.
+template <bool GLU, typename TC>
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ part, int S,
+                                                                  int M, int N, TC* __restrict__ C,
+                                                                  int n_out) {
+    const int per_row = (n_out + 3) / 4;
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long)M * per_row) return;
+    const int m = (int)(idx / per_row), j = (int)(idx % per_row) * 4;
+    const size_t plane = (size_t)M * N;
+    floatx4 a = floatx4{0.f, 0.f, 0.f, 0.f}, b = a;
+    if constexpr (GLU) {
+        const int c = (j >> 4) * 32 + (j & 15);   // N is a multiple of 32 here: whole float4s
+        const float* p = part + (size_t)m * N + c;
+        for (int s = 0; s < S; ++s, p += plane) {
+            const float4 g = *reinterpret_cast<const float4*>(p);
+            const float4 u = *reinterpret_cast<const float4*>(p + 16);
+            a[0] += g.x; a[1] += g.y; a[2] += g.z; a[3] += g.w;
+            b[0] += u.x; b[1] += u.y; b[2] += u.z; b[3] += u.w;
+        }
+        a = silu_mul(a, b);
+    } else {
+        const float* p = part + (size_t)m * N + j;
+        const bool vec = (N % 4) == 0;
+        for (int s = 0; s < S; ++s, p += plane) {
+            if (vec) {
+                const float4 v = *reinterpret_cast<const float4*>(p);
+                a[0] += v.x; a[1] += v.y; a[2] += v.z; a[3] += v.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (j + e < N) a[e] += p[e];
+            }
+        }
+    }
+    store4<TC>(C + (size_t)m * n_out + j, a, j, n_out, (n_out % 4) == 0);
 }
 
 // ------------------------------------------ tiled, async copy, k-steps of 32 ---
@@ -442,20 +501,33 @@ static int launch_pipe(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N,
     return tff_check_launch("gemm_bf16_pipe");
 }
 
+// splits > 1: the blocks of a tile split K among them; part holds splits * M * N floats
 template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU = false>
 static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
-                          int c_dtype, int n_out, hipStream_t s) {
+                          int c_dtype, int n_out, hipStream_t s, int splits = 1, float* part = nullptr) {
     const int KB = (K + 31) / 32;
     constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
-    const dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN);
+    if (splits <= 1 || !part) { splits = 1; part = nullptr; }
+    const dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN, splits);
     TFF_REQUIRE(grid.y <= 65535, "gemm: too many columns N=%d", N);
     if (c_dtype == TFF_F32)
         gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, float>
-            <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
+            <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out, part);
     else
         gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, bf16_t>
-            <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
-    return tff_check_launch("gemm_bf16_async");
+            <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out, part);
+    if (int rc = tff_check_launch("gemm_bf16_async")) return rc;
+    if (splits > 1) {
+        const int No = GLU ? n_out : N;
+        const long threads = (long)M * ((No + 3) / 4);
+        const int blocks = (int)((threads + 255) / 256);
+        if (c_dtype == TFF_F32)
+            gemm_splitk_reduce_kernel<GLU, float><<<blocks, 256, 0, s>>>(part, splits, M, N, (float*)C, No);
+        else
+            gemm_splitk_reduce_kernel<GLU, bf16_t><<<blocks, 256, 0, s>>>(part, splits, M, N, (bf16_t*)C, No);
+        return tff_check_launch("gemm_splitk_reduce");
+    }
+    return 0;
 }
 
 // four waves in 2 x 2
@@ -662,8 +734,24 @@ static int launch_tiled(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N
 
 // glu_out > 0: W holds gate and up groups in turn (N = 2 * ceil16(glu_out) rows) and C is
 // [M, glu_out] = silu(gate) * up.
+// How many blocks share a tile's K for 16 < M <= 64: the tiled kernel with 64 x 128 tiles
+// wants some 400 blocks to pull on all of HBM.
+static int splitk_for(int M, int N, int K) {
+    if (M <= 16 || M > 64) return 1;
+    const int tiles = (N + 127) / 128, nk = (K + 63) / 64;
+    int S = 1;
+    while (S < 8 && tiles * S * 2 <= 400 && nk / (S * 2) >= 4) S *= 2;
+    return S;
+}
+
+TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype) {
+    if (ab_dtype != TFF_BF16) return 0;
+    const int S = splitk_for(M, N, K);
+    return S > 1 ? (size_t)S * M * N * sizeof(float) : 0;
+}
+
 int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
-                  int c_dtype, int glu_out, hipStream_t s) {
+                  int c_dtype, int glu_out, float* workspace, size_t workspace_bytes, hipStream_t s) {
     TFF_REQUIRE(K % 8 == 0 && lda % 8 == 0,
                 "gemm: the bfloat16 product needs the inner size (K=%d, row stride %d) to be a multiple of 8",
                 K, lda);
@@ -672,6 +760,7 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
     TFF_REQUIRE(c_dtype == TFF_F32 || c_dtype == TFF_BF16, "gemm: unknown output type %d", c_dtype);
     // The choices below were measured at the sizes of an 8B model on an MI355X.
     const long big_tiles = (long)((M + 255) / 256) * ((N + 255) / 256);
+    const int split = workspace ? splitk_for(M, N, K) : 1;
     if (glu_out > 0) {
         TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
                     "gemm: a gated weight of %d rows does not fit %d output columns", N, glu_out);
@@ -680,6 +769,10 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
             if (N >= 16 * 1024)
                 return launch_skinny<1, 1, 8, 1, 2, true, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
             return launch_skinny<1, 1, 32, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
+        }
+        if (M <= 64) {
+            const int S = workspace_bytes >= (size_t)split * M * N * sizeof(float) ? split : 1;
+            return launch_async_g<2, 2, 2, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         }
         if (M < 128) return launch_async<2, 4, 4, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
         if (M >= 512 && big_tiles >= 160)
@@ -694,9 +787,11 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
         return launch_skinny<1, 1, 8, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
     }
     if (M <= 64) {
-        // many columns: enough blocks for the tiled kernel with a deep pipeline; few columns: the
-        // streaming kernel, whose blocks split K among their waves
-        if (N >= 16 * 1024) return launch_async<2, 4, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+        // 64 x 128 tiles (72 KB of LDS: two blocks to a CU); with few columns the blocks of a
+        // tile split K and a second kernel adds their partial sums, if the caller brought the
+        // memory for them; else the streaming kernel, whose blocks split K among their waves
+        if (split == 1 || workspace_bytes >= (size_t)split * M * N * sizeof(float))
+            return launch_async_g<2, 2, 2, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, split, workspace);
         if (M <= 32) return launch_skinny<2, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
         return launch_skinny<4, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
     }
@@ -710,7 +805,8 @@ int tff_gemm_f32(const float* A, const float* W, void* C, int M, int N, int K, i
                  int c_dtype, hipStream_t s);
 
 TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda,
-                     int ab_dtype, int c_dtype, int w_packed, int glu_out, tff_stream_t stream) {
+                     int ab_dtype, int c_dtype, int w_packed, int glu_out, void* workspace,
+                     size_t workspace_bytes, tff_stream_t stream) {
     TFF_REQUIRE(A && W && C, "gemm: null pointer");
     TFF_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K, "gemm: bad sizes M=%d N=%d K=%d lda=%d", M, N, K, lda);
     if (M == 0) return 0;
@@ -721,7 +817,9 @@ TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K,
     }
     if (ab_dtype == TFF_BF16) {
         TFF_REQUIRE(w_packed, "gemm: the bfloat16 product takes a weight in fragment order");
-        return tff_gemm_bf16((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, c_dtype, glu_out, s);
+        TFF_REQUIRE(((uintptr_t)workspace % 16) == 0, "gemm: the workspace must be 16-byte aligned");
+        return tff_gemm_bf16((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, c_dtype, glu_out,
+                             (float*)workspace, workspace ? workspace_bytes : 0, s);
     }
     return tff_fail("gemm: unknown operand type %d", ab_dtype);
 }

@@ -38,8 +38,12 @@ TFF_API int tff_rmsnorm(const void* x, const float* weight, float eps, void* out
 // see tff_pack_weight).  glu_out > 0 (bfloat16 only): the 16-row groups of W
 // alternate between a gate and an up projection, N = 2 * ceil16(glu_out), and
 // C is [M, glu_out] = silu(gate) * up.
+// workspace (may be null): device memory of tff_gemm_workspace_bytes() bytes the
+// product may keep partial sums in; with less it takes a path that needs none.
 TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda,
-                     int ab_dtype, int c_dtype, int w_packed, int glu_out, tff_stream_t stream);
+                     int ab_dtype, int c_dtype, int w_packed, int glu_out, void* workspace,
+                     size_t workspace_bytes, tff_stream_t stream);
+TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype);
 
 // bfloat16 row-major [N, K] (K a multiple of 8) -> fragment order: tiles of
 // 16 rows x 32 k, each stored as the 1 KB operand of a 16x16x32 MFMA, element

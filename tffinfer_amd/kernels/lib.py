@@ -2,11 +2,11 @@
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class KernelLibraryError(RuntimeError):
@@ -17,13 +17,14 @@ class KernelError(RuntimeError):
     """An entry point refused its arguments or a launch failed."""
 
 
-_P, _I, _F = c_void_p, c_int, c_float
+_P, _I, _F, _Z = c_void_p, c_int, c_float, c_size_t
 
 _SIGNATURES = {
     "tff_embed": [_P, _P, _P, _I, _I, _I, _I, _P],
     "tff_add_rmsnorm": [_P, _P, _P, _F, _P, _P, _I, _I, _I, _P],
     "tff_rmsnorm": [_P, _P, _F, _P, _I, _I, _I, _P],
-    "tff_gemm": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+    "tff_gemm": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _Z, _P],
+    "tff_gemm_workspace_bytes": [_I, _I, _I, _I],
     "tff_pack_weight": [_P, _P, _I, _I, _P],
     "tff_embed_packed": [_P, _P, _P, _I, _I, _I, _P],
     "tff_qk_norm_rope_kv": [_P, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _I, _P, _P, _P, _P,
@@ -66,7 +67,7 @@ def load() -> ctypes.CDLL:
     for name, args in _SIGNATURES.items():
         fn = getattr(lib, name)
         fn.argtypes = args
-        fn.restype = c_int
+        fn.restype = c_size_t if name.endswith("_bytes") else c_int
     _lib = lib
     return lib
 

@@ -230,9 +230,12 @@ def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
         if tuple(out.shape) != (M, n_out):
             raise _lib.KernelError(f"linear out: shape {tuple(out.shape)} is not {(M, n_out)}")
     L = _lib.load()
+    # some shapes (a few dozen rows, few columns) split K over blocks and need room for partial sums
+    ws_bytes = L.tff_gemm_workspace_bytes(M, N, K, dtype_code(x.dtype)) if packed else 0
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=x.device) if ws_bytes else None
     _lib.check(L.tff_gemm(x.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K, lda,
                           dtype_code(x.dtype), dtype_code(out_dtype), 1 if packed else 0, glu_out,
-                          _stream()))
+                          _ptr(ws), ws_bytes, _stream()))
     return out
 
 
