@@ -82,7 +82,8 @@ def test_rmsnorm_eps_position():
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 320, 96), (33, 200, 200), (130, 130, 72), (257, 96, 256),
-                                    (64, 4096, 512), (300, 1000, 1024), (50, 203, 1000), (40, 1024, 2056)])
+                                    (64, 4096, 512), (300, 1000, 1024), (50, 203, 1000), (40, 1024, 2056),
+                                    (100, 203, 2048), (520, 264, 1544)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_linear(M, N, K, dtype):
     ops = _ops()

@@ -40,12 +40,6 @@ __device__ __forceinline__ void store4(TC* dst, const floatx4& v, int n, int N, 
     }
 }
 
-// ------------------------------------------------------------------ tiled ---
-// Block tile (WTM*32) x (WTN*32) x 64 with 4 waves in 2 x 2, each wave
-// WTM x WTN MFMA tiles.  Both operands go global -> registers -> LDS in
-// fragment order (linear 16-byte stores), double buffered; a wave reads a
-// fragment back as one linear 1 KB.  The padding of W to 32 k holds zeros, so
-// k past the end of A only has to be readable: what it multiplies is zero.
 // GLU: the 16-row groups of W alternate between a gate and an up projection
 // (group 2p gate, group 2p+1 up); the epilogue writes silu(gate) * up, N / 2 columns.
 __device__ __forceinline__ floatx4 silu_mul(const floatx4& g, const floatx4& u) {
@@ -55,139 +49,15 @@ __device__ __forceinline__ floatx4 silu_mul(const floatx4& g, const floatx4& u) 
     return o;
 }
 
-template <int WTM, int WTN, bool GLU, typename TC>
-__global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __restrict__ A,
-                                                               const bf16_t* __restrict__ Wp,
-                                                               TC* __restrict__ C, int M, int N,
-                                                               int K, int lda, int KB, int n_out) {
-    constexpr int BM = WTM * 32, BN = WTN * 32;
-    constexpr int AF = BM / 16 * 2, WF = BN / 16 * 2;   // fragments per operand tile (2 k-steps)
-    constexpr int AL = AF / 4, WL = WF / 4;             // 16-byte loads per thread and operand
-    __shared__ __attribute__((aligned(16))) bf16_t As[2][AF * 512];
-    __shared__ __attribute__((aligned(16))) bf16_t Ws[2][WF * 512];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int fr = lane & 15, fg = lane >> 4;
-    // blocks that run at the same time differ in m first: they share their W tiles out of L2
-    const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
-    const int NB = (N + 15) / 16;
-
-    floatx4 acc[WTN][WTM];
-#pragma unroll
-    for (int i = 0; i < WTN; ++i)
-#pragma unroll
-        for (int j = 0; j < WTM; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    // a thread's share of a tile: fragments f = wave + 4 j (f = row group * 2 + k-step), this
-    // lane's 16 bytes of each
-    const bf16_t* a_src[AL];
-    int a_koff[AL];
-#pragma unroll
-    for (int j = 0; j < AL; ++j) {
-        const int f = wave + 4 * j;
-        const int row = min(m0 + (f >> 1) * 16 + fr, M - 1);   // rows past the end repeat the last
-        a_koff[j] = (f & 1) * 32 + fg * 8;
-        a_src[j] = A + (size_t)row * lda;
-    }
-    const bf16_t* w_src[WL];
-    int w_ks[WL];
-#pragma unroll
-    for (int j = 0; j < WL; ++j) {
-        const int f = wave + 4 * j;
-        const int nb = min(n0 / 16 + (f >> 1), NB - 1);
-        w_ks[j] = f & 1;
-        w_src[j] = Wp + (size_t)nb * KB * 512 + lane * 8;
-    }
-    uint4 ra[AL], rw[WL];
-    const int nk = (K + 63) / 64;
-
-#define TFF_LOAD_TILE(kt)                                                                          \
-    {                                                                                              \
-        const int k0_ = (kt) * 64;                                                                 \
-        if (k0_ + 64 <= K) {                                                                       \
-            _Pragma("unroll") for (int j = 0; j < AL; ++j) ra[j] = ld16(a_src[j] + k0_ + a_koff[j]); \
-            _Pragma("unroll") for (int j = 0; j < WL; ++j)                                         \
-                rw[j] = ld16(w_src[j] + (size_t)(2 * (kt) + w_ks[j]) * 512);                       \
-        } else { /* the last, partial tile: clamp what does not exist */                           \
-            _Pragma("unroll") for (int j = 0; j < AL; ++j)                                         \
-                ra[j] = ld16(a_src[j] + min(k0_ + a_koff[j], K - 8));                              \
-            _Pragma("unroll") for (int j = 0; j < WL; ++j) {                                       \
-                const int ks_ = 2 * (kt) + w_ks[j];                                                \
-                const uint4 v_ = ld16(w_src[j] + (size_t)min(ks_, KB - 1) * 512);                  \
-                rw[j] = ks_ < KB ? v_ : make_uint4(0, 0, 0, 0);                                    \
-            }                                                                                      \
-        }                                                                                          \
-    }
-#define TFF_STORE_LDS(buf)                                                                         \
-    {                                                                                              \
-        _Pragma("unroll") for (int j = 0; j < AL; ++j)                                             \
-            *reinterpret_cast<uint4*>(&As[buf][(wave + 4 * j) * 512 + lane * 8]) = ra[j];          \
-        _Pragma("unroll") for (int j = 0; j < WL; ++j)                                             \
-            *reinterpret_cast<uint4*>(&Ws[buf][(wave + 4 * j) * 512 + lane * 8]) = rw[j];          \
-    }
-
-    TFF_LOAD_TILE(0)
-    TFF_STORE_LDS(0)
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) TFF_LOAD_TILE(kt + 1)
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            bf16x8 fw[WTN], fa[WTM];
-#pragma unroll
-            for (int i = 0; i < WTN; ++i)
-                fw[i] = *reinterpret_cast<const bf16x8*>(&Ws[buf][((wn * WTN + i) * 2 + ks) * 512 + lane * 8]);
-#pragma unroll
-            for (int j = 0; j < WTM; ++j)
-                fa[j] = *reinterpret_cast<const bf16x8*>(&As[buf][((wm * WTM + j) * 2 + ks) * 512 + lane * 8]);
-#pragma unroll
-            for (int i = 0; i < WTN; ++i)
-#pragma unroll
-                for (int j = 0; j < WTM; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[i], fa[j], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < nk) TFF_STORE_LDS(buf ^ 1)
-        __syncthreads();
-    }
-#undef TFF_LOAD_TILE
-#undef TFF_STORE_LDS
-
-    // lane holds C[m][n .. n+3], n = n0 + (wn*WTN + i)*16 + fg*4, m = m0 + (wm*WTM + j)*16 + fr
-    if constexpr (GLU) {
-        static_assert(WTN % 2 == 0, "gate and up groups come in pairs");
-        const int No = n_out;
-        const bool vec = (No % 4) == 0;
-#pragma unroll
-        for (int i = 0; i < WTN; i += 2) {
-            const int n = (n0 + (wn * WTN + i) * 16) / 2 + fg * 4;
-#pragma unroll
-            for (int j = 0; j < WTM; ++j) {
-                const int m = m0 + (wm * WTM + j) * 16 + fr;
-                if (m < M && n < No)
-                    store4<TC>(C + (size_t)m * No + n, silu_mul(acc[i][j], acc[i + 1][j]), n, No, vec);
-            }
-        }
-    } else {
-        const bool vec = (N % 4) == 0;
-#pragma unroll
-        for (int i = 0; i < WTN; ++i) {
-            const int n = n0 + (wn * WTN + i) * 16 + fg * 4;
-#pragma unroll
-            for (int j = 0; j < WTM; ++j) {
-                const int m = m0 + (wm * WTM + j) * 16 + fr;
-                if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, acc[i][j], n, N, vec);
-            }
-        }
-    }
-}
-
 // ------------------------------------------------------- tiled, async copy ---
-// The same tiling with the copies global -> LDS done by the load unit itself
-// (global_load_lds_dwordx4: every lane's 16 bytes land at LDS base + lane * 16,
-// which is exactly fragment order), so no register and no LDS store instruction
-// is spent on staging, and STAGES - 1 tiles are in flight while one is worked on.
+// Block tile (WGM*WTM*16) x (WGN*WTN*16) x 64 on WGM x WGN waves, each wave
+// WTM x WTN MFMA tiles.  Both operands are staged in LDS in fragment order; the
+// padding of W to 32 k holds zeros, so k past the end of A only has to be
+// readable: what it multiplies is zero.  The copies global -> LDS are done by
+// the load unit itself (global_load_lds_dwordx4: every lane's 16 bytes land at
+// LDS base + lane * 16, which is exactly fragment order), so no register and no
+// LDS store instruction is spent on staging, and STAGES - 1 tiles are in flight
+// while one is worked on.
 // A wave waits for its own copies of the tile it is about to read
 // (s_waitcnt vmcnt), the barrier that follows makes the other waves' visible.
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -365,142 +235,6 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
     store4<TC>(C + (size_t)m * n_out + j, a, j, n_out, (n_out % 4) == 0);
 }
 
-// ------------------------------------------ tiled, async copy, k-steps of 32 ---
-// For large wave tiles (up to 128 x 128 per wave) LDS bandwidth and latency
-// decide: a stage holds one k-step (32 k) only, so four stages fit beside
-// 256 x 256 tiles, and a wave reads the operands of k-step kt + 1 into a second
-// set of registers while the matrix cores work on k-step kt.  One barrier per
-// k-step: after it, the copies of k-step kt + 1 are visible to all, and the
-// stage of k-step kt - 1 is free for the copy of k-step kt + STAGES - 1.
-template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU, typename TC>
-__global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_pipe_kernel(
-    const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
-    int K, int lda, int KB, int n_out) {
-    constexpr int NW = WGM * WGN;
-    constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
-    constexpr int AF = BM / 16, WF = BN / 16;   // fragments per stage and operand (one k-step)
-    constexpr int FR = AF + WF;
-    constexpr int LPW = FR / NW;
-    static_assert(FR % NW == 0, "fragments are dealt to the waves evenly");
-    static_assert(STAGES >= 3 && (STAGES - 3) * LPW < 64, "vmcnt has 6 bits");
-    __shared__ __attribute__((aligned(1024))) bf16_t smem[STAGES * FR * 512];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WGN, wn = wave % WGN;
-    const int fr = lane & 15, fg = lane >> 4;
-    const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
-    const int NB = (N + 15) / 16;
-
-    floatx4 acc[WTN][WTM];
-#pragma unroll
-    for (int i = 0; i < WTN; ++i)
-#pragma unroll
-        for (int j = 0; j < WTM; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    const bf16_t* src[LPW];
-#pragma unroll
-    for (int j = 0; j < LPW; ++j) {
-        const int f = wave + NW * j;
-        if (f < AF) src[j] = A + (size_t)min(m0 + f * 16 + fr, M - 1) * lda;
-        else src[j] = Wp + (size_t)min(n0 / 16 + (f - AF), NB - 1) * KB * 512 + lane * 8;
-    }
-    // k-steps past the end are copied as the last one (into stages nobody reads any more), so
-    // that the number of copies in flight is the same in every iteration
-#define TFF_ISSUE_STEP(step)                                                                       \
-    {                                                                                              \
-        const int ks_ = min((step), KB - 1);                                                       \
-        const int st_ = (step) % STAGES;                                                           \
-        _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                          \
-            const int f = wave + NW * j;                                                           \
-            const bf16_t* g_ = f < AF ? src[j] + min(ks_ * 32 + fg * 8, K - 8)                     \
-                                      : src[j] + (size_t)ks_ * 512;                                \
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)g_, (lds_ptr_t)(smem + (st_ * FR + f) * 512), 16, 0, 0); \
-        }                                                                                          \
-    }
-#define TFF_READ_FRAGS(step, FW, FA)                                                               \
-    {                                                                                              \
-        const bf16_t* st_ = smem + ((step) % STAGES) * FR * 512;                                   \
-        _Pragma("unroll") for (int i = 0; i < WTN; ++i)                                            \
-            FW[i] = *reinterpret_cast<const bf16x8*>(st_ + (AF + wn * WTN + i) * 512 + lane * 8);  \
-        _Pragma("unroll") for (int j = 0; j < WTM; ++j)                                            \
-            FA[j] = *reinterpret_cast<const bf16x8*>(st_ + (wm * WTM + j) * 512 + lane * 8);       \
-    }
-#define TFF_MFMA_STEP(FW, FA)                                                                      \
-    {                                                                                              \
-        _Pragma("unroll") for (int i = 0; i < WTN; ++i)                                            \
-            _Pragma("unroll") for (int j = 0; j < WTM; ++j)                                        \
-                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(FW[i], FA[j], acc[i][j], 0, 0, 0); \
-    }
-
-    bf16x8 fw0[WTN], fa0[WTM], fw1[WTN], fa1[WTM];
-#pragma unroll
-    for (int t = 0; t < STAGES - 1; ++t) TFF_ISSUE_STEP(t)
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * LPW));   // k-step 0 is in
-    __syncthreads();
-    TFF_READ_FRAGS(0, fw0, fa0)
-    // two k-steps per trip so that the register sets swap without copies
-    for (int kt = 0; kt < KB; kt += 2) {
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * LPW));   // k-step kt + 1 is in
-        __syncthreads();
-        TFF_ISSUE_STEP(kt + STAGES - 1)
-        TFF_READ_FRAGS(kt + 1, fw1, fa1)
-        TFF_MFMA_STEP(fw0, fa0)
-        if (kt + 1 < KB) {
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * LPW));
-            __syncthreads();
-            TFF_ISSUE_STEP(kt + STAGES)
-            TFF_READ_FRAGS(kt + 2, fw0, fa0)
-            TFF_MFMA_STEP(fw1, fa1)
-        }
-    }
-#undef TFF_ISSUE_STEP
-#undef TFF_READ_FRAGS
-#undef TFF_MFMA_STEP
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));   // the copies past the end must not outlive the block
-
-    if constexpr (GLU) {
-        static_assert(WTN % 2 == 0, "gate and up groups come in pairs");
-        const bool vec = (n_out % 4) == 0;
-#pragma unroll
-        for (int i = 0; i < WTN; i += 2) {
-            const int n = (n0 + (wn * WTN + i) * 16) / 2 + fg * 4;
-#pragma unroll
-            for (int j = 0; j < WTM; ++j) {
-                const int m = m0 + (wm * WTM + j) * 16 + fr;
-                if (m < M && n < n_out)
-                    store4<TC>(C + (size_t)m * n_out + n, silu_mul(acc[i][j], acc[i + 1][j]), n, n_out, vec);
-            }
-        }
-    } else {
-        const bool vec = (N % 4) == 0;
-#pragma unroll
-        for (int i = 0; i < WTN; ++i) {
-            const int n = n0 + (wn * WTN + i) * 16 + fg * 4;
-#pragma unroll
-            for (int j = 0; j < WTM; ++j) {
-                const int m = m0 + (wm * WTM + j) * 16 + fr;
-                if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, acc[i][j], n, N, vec);
-            }
-        }
-    }
-}
-
-template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU = false>
-static int launch_pipe(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
-                       int c_dtype, int n_out, hipStream_t s) {
-    const int KB = (K + 31) / 32;
-    constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
-    const dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN);
-    TFF_REQUIRE(grid.y <= 65535, "gemm: too many columns N=%d", N);
-    if (c_dtype == TFF_F32)
-        gemm_bf16_pipe_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, float>
-            <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
-    else
-        gemm_bf16_pipe_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, bf16_t>
-            <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
-    return tff_check_launch("gemm_bf16_pipe");
-}
-
 // splits > 1: the blocks of a tile split K among them; part holds splits * M * N floats
 template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU = false>
 static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
@@ -528,13 +262,6 @@ static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int
         return tff_check_launch("gemm_splitk_reduce");
     }
     return 0;
-}
-
-// four waves in 2 x 2
-template <int WTM, int WTN, int STAGES, bool GLU = false>
-static int launch_async(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
-                        int c_dtype, int n_out, hipStream_t s) {
-    return launch_async_g<2, 2, WTM, WTN, STAGES, GLU>(A, Wp, C, M, N, K, lda, c_dtype, n_out, s);
 }
 
 // ------------------------------------------------------------- skinny M ---
@@ -719,37 +446,34 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
     return tff_check_launch("gemm_bf16_skinny");
 }
 
-template <int WTM, int WTN, bool GLU = false>
-static int launch_tiled(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
-                        int c_dtype, int n_out, hipStream_t s) {
-    const int KB = (K + 31) / 32;
-    const dim3 grid((M + WTM * 32 - 1) / (WTM * 32), (N + WTN * 32 - 1) / (WTN * 32));
-    TFF_REQUIRE(grid.y <= 65535, "gemm: too many columns N=%d", N);
-    if (c_dtype == TFF_F32)
-        gemm_bf16_tiled_kernel<WTM, WTN, GLU, float><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
-    else
-        gemm_bf16_tiled_kernel<WTM, WTN, GLU, bf16_t><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
-    return tff_check_launch("gemm_bf16_tiled");
-}
-
-// glu_out > 0: W holds gate and up groups in turn (N = 2 * ceil16(glu_out) rows) and C is
-// [M, glu_out] = silu(gate) * up.
-// How many blocks share a tile's K for 16 < M <= 64: the tiled kernel with 64 x 128 tiles
-// wants some 400 blocks to pull on all of HBM.
-static int splitk_for(int M, int N, int K) {
-    if (M <= 16 || M > 64) return 1;
-    const int tiles = (N + 127) / 128, nk = (K + 63) / 64;
+// The tiled product's plan for M > 16: tiles of 64 x 128 (up to 64 rows), 128 x 128 (up to
+// 384) or 256 x 256, and into how many parts the blocks of a tile split K so that the launch
+// has blocks for all CUs (a CU holds two blocks of the smaller tiles, one of the largest).
+// Measured at the sizes of an 8B model on an MI355X.
+struct GemmPlan { int tile; int splits; };
+static GemmPlan plan_for(int M, int N, int K) {
+    if (M <= 16) return {0, 1};
+    const int tile = M <= 64 ? 64 : (M <= 384 ? 128 : 256);
+    const int bn = tile == 64 ? 128 : tile;
+    const long blocks = (long)((M + tile - 1) / tile) * ((N + bn - 1) / bn);
+    const int limit = tile == 64 ? 400 : (tile == 128 ? 576 : 288);
+    const int max_splits = tile == 64 ? 8 : 4;
+    const int min_tiles = tile == 64 ? 4 : 8;   // 64-k tiles a part keeps at least
+    const int nk = (K + 63) / 64;
     int S = 1;
-    while (S < 8 && tiles * S * 2 <= 400 && nk / (S * 2) >= 4) S *= 2;
-    return S;
+    while (S < max_splits && blocks * S * 2 <= limit && nk / (S * 2) >= min_tiles) S *= 2;
+    return {tile, S};
 }
 
 TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype) {
-    if (ab_dtype != TFF_BF16) return 0;
-    const int S = splitk_for(M, N, K);
-    return S > 1 ? (size_t)S * M * N * sizeof(float) : 0;
+    if (ab_dtype != TFF_BF16 || M <= 0 || N <= 0 || K <= 0) return 0;
+    const GemmPlan p = plan_for(M, N, K);
+    return p.splits > 1 ? (size_t)p.splits * M * N * sizeof(float) : 0;
 }
 
+// glu_out > 0: W holds gate and up groups in turn (N = 2 * ceil16(glu_out) rows) and C is
+// [M, glu_out] = silu(gate) * up.  workspace: room for partial sums (tff_gemm_workspace_bytes);
+// with less the blocks do not split K.
 int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
                   int c_dtype, int glu_out, float* workspace, size_t workspace_bytes, hipStream_t s) {
     TFF_REQUIRE(K % 8 == 0 && lda % 8 == 0,
@@ -758,9 +482,9 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
     TFF_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)Wp % 16) == 0 && ((uintptr_t)C % 16) == 0,
                 "gemm: operands must be 16-byte aligned");
     TFF_REQUIRE(c_dtype == TFF_F32 || c_dtype == TFF_BF16, "gemm: unknown output type %d", c_dtype);
-    // The choices below were measured at the sizes of an 8B model on an MI355X.
-    const long big_tiles = (long)((M + 255) / 256) * ((N + 255) / 256);
-    const int split = workspace ? splitk_for(M, N, K) : 1;
+    GemmPlan plan = plan_for(M, N, K);
+    if (!workspace || workspace_bytes < (size_t)plan.splits * M * N * sizeof(float)) plan.splits = 1;
+    const int S = plan.splits;
     if (glu_out > 0) {
         TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
                     "gemm: a gated weight of %d rows does not fit %d output columns", N, glu_out);
@@ -770,14 +494,11 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
                 return launch_skinny<1, 1, 8, 1, 2, true, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
             return launch_skinny<1, 1, 32, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
         }
-        if (M <= 64) {
-            const int S = workspace_bytes >= (size_t)split * M * N * sizeof(float) ? split : 1;
+        if (plan.tile == 64)
             return launch_async_g<2, 2, 2, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
-        }
-        if (M < 128) return launch_async<2, 4, 4, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
-        if (M >= 512 && big_tiles >= 160)
-            return launch_async_g<4, 4, 4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
-        return launch_async_g<2, 4, 4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
+        if (plan.tile == 128)
+            return launch_async_g<2, 2, 4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+        return launch_async_g<4, 4, 4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
     }
     if (M <= 16) {
         // more waves per block where there are few blocks (small N) or long rows (large K),
@@ -786,19 +507,18 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
         if (K >= 8192 || N <= 4096) return launch_skinny<1, 1, 4, 16>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
         return launch_skinny<1, 1, 8, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
     }
-    if (M <= 64) {
-        // 64 x 128 tiles (72 KB of LDS: two blocks to a CU); with few columns the blocks of a
-        // tile split K and a second kernel adds their partial sums, if the caller brought the
-        // memory for them; else the streaming kernel, whose blocks split K among their waves
-        if (split == 1 || workspace_bytes >= (size_t)split * M * N * sizeof(float))
-            return launch_async_g<2, 2, 2, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, split, workspace);
-        if (M <= 32) return launch_skinny<2, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
-        return launch_skinny<4, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+    if (plan.tile == 64) {
+        // few columns and no room for partial sums: the streaming kernel, whose blocks split K
+        // among their waves
+        if (S == 1 && plan_for(M, N, K).splits > 1) {
+            if (M <= 32) return launch_skinny<2, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+            return launch_skinny<4, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+        }
+        return launch_async_g<2, 2, 2, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace);
     }
-    // 256 x 256 tiles on 16 waves where they still give most CUs a block, else 128 x 256 on 8
-    if (M < 128) return launch_async<2, 4, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
-    if (M >= 512 && big_tiles >= 160) return launch_async_g<4, 4, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
-    return launch_async_g<2, 4, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+    if (plan.tile == 128)
+        return launch_async_g<2, 2, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace);
+    return launch_async_g<4, 4, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace);
 }
 
 int tff_gemm_f32(const float* A, const float* W, void* C, int M, int N, int K, int lda,
