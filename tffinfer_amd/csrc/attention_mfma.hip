@@ -520,29 +520,36 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __r
 #define ATTN_STAGES 4
 constexpr int attn_vmcnt_imm(int v) { return (v & 15) | (7 << 4) | (15 << 8) | ((v >> 4) << 14); }
 
-template <int DT, int NQT>
-__global__ __launch_bounds__(256, 2) void attn_mfma_block_kernel(
+template <int DT, int NQT, int NW>
+__global__ __launch_bounds__(64 * NW, (NW <= 4 ? 2 : 1)) void attn_mfma_block_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_tables, int bt_stride, const int32_t* __restrict__ cu_tokens,
-    const int32_t* __restrict__ start_pos, const int32_t* __restrict__ work, int nq, int nkv,
-    int page_size, int page_shift, int window, float scale) {
+    const int32_t* __restrict__ start_pos, const int32_t* __restrict__ work,
+    const int32_t* __restrict__ block_items, int nq, int nkv, int page_size, int page_shift,
+    int window, float scale) {
     constexpr int D = DT * 16;
     constexpr int KS = (D + 31) / 32;
     constexpr int KFR = 2 * KS, VFR = DT, FR = KFR + VFR;   // 1 KB fragments per slice
-    constexpr int LPW = (FR + 3) / 4;                        // copies a wave issues per slice
-    constexpr int BCOLS = 4 * NQT * 16;                      // columns of a block
+    constexpr int LPW = (FR + NW - 1) / NW;                  // copies a wave issues per slice
+    constexpr int BCOLS = NW * NQT * 16;                     // columns of a block
     constexpr int STAGES = ATTN_STAGES;                      // slices in LDS: one in use, the rest in flight
     __shared__ __attribute__((aligned(1024))) bf16_t smem[STAGES * FR * 512];
     __shared__ int32_t pages[ATTN_BT_LDS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int qc = lane & 15, kg = lane >> 4;
-    // the last blocks of a request see the most keys: they start first
-    const int bx = gridDim.x - 1 - blockIdx.x;
-    const int r = work[2 * bx];
-    const int bcol0 = work[2 * bx + 1];
     const int g = blockIdx.y;
     const int G = nq / nkv;
+    // A block works through the items block_items[b] .. block_items[b + 1] of the work table one
+    // after the other (the host deals items to blocks so that all blocks have about the same
+    // number of slices to go through); without that table block b has item b, the last ones,
+    // which see the most keys, first.
+    const int it_begin = block_items ? block_items[blockIdx.x] : (int)(gridDim.x - 1 - blockIdx.x);
+    const int it_end = block_items ? block_items[blockIdx.x + 1] : it_begin + 1;
+    for (int item = it_begin; item < it_end; ++item) {
+    if (item > it_begin) __syncthreads();   // the last item's slices and page numbers are read
+    const int r = work[2 * item];
+    const int bcol0 = work[2 * item + 1];
     const int tok0 = cu_tokens[r];
     const int n = cu_tokens[r + 1] - tok0;
     const int P = start_pos[r];
@@ -575,7 +582,7 @@ __global__ __launch_bounds__(256, 2) void attn_mfma_block_kernel(
     const int npg = page_index(kmax, page_size, page_shift) - pg0 + 1;
     const bool bt_in_lds = npg <= ATTN_BT_LDS;
     if (bt_in_lds)
-        for (int i = tid; i < npg; i += 256) pages[i] = bt[pg0 + i];
+        for (int i = tid; i < npg; i += 64 * NW) pages[i] = bt[pg0 + i];
 
     bf16x8 qf[NQT][KS];
 #pragma unroll
@@ -611,7 +618,7 @@ __global__ __launch_bounds__(256, 2) void attn_mfma_block_kernel(
         const int kb_ = kb0 + min((step), nsteps - 1) * 32;                                         \
         const int st_ = (step) % STAGES;                                                            \
         _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                           \
-            const int f = min(wave + 4 * j, FR - 1);                                                \
+            const int f = min(wave + NW * j, FR - 1);                                               \
             {                                                                                       \
                 const bf16_t* g_;                                                                   \
                 if (f < KFR) {                                                                      \
@@ -737,22 +744,29 @@ __global__ __launch_bounds__(256, 2) void attn_mfma_block_kernel(
             *reinterpret_cast<uint2*>(op + dt * 16 + kg * 4) = pk.u;
         }
     }
+    }   // items
 }
 
 template <int DT>
 static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o, float* part_ml,
                        const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* block_tables,
                        int bt_stride, const int32_t* cu_tokens, const int32_t* start_pos,
-                       const int32_t* work, int num_work, int tiles_per_entry, int cols_per_wave,
+                       const int32_t* work, int num_work, const int32_t* block_items, int num_blocks,
+                       int block_variant, int tiles_per_entry, int cols_per_wave,
                        int splits, int nq, int nkv, int page_size, int window, float scale,
                        int T_total, hipStream_t s) {
     int page_shift = -1;
     if ((page_size & (page_size - 1)) == 0)
         for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
-    if (cols_per_wave == 128) {   // blocks of four waves, two column tiles each
-        attn_mfma_block_kernel<DT, 2><<<dim3(num_work, nkv), 256, 0, s>>>(
-            q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work, nq,
-            nkv, page_size, page_shift, window, scale);
+    if (cols_per_wave == 128) {   // blocks that share their keys through LDS
+        if (block_variant == 1)   // eight waves, one column tile each
+            attn_mfma_block_kernel<DT, 1, 8><<<dim3(num_blocks, nkv), 512, 0, s>>>(
+                q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
+                block_items, nq, nkv, page_size, page_shift, window, scale);
+        else                      // four waves, two column tiles each
+            attn_mfma_block_kernel<DT, 2, 4><<<dim3(num_blocks, nkv), 256, 0, s>>>(
+                q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
+                block_items, nq, nkv, page_size, page_shift, window, scale);
         return tff_check_launch("attention_mfma_block");
     }
     const dim3 grid(num_work, nkv, splits);
@@ -788,6 +802,7 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                const void* k_cache, const void* v_cache,
                                const int32_t* block_tables, int bt_stride, const int32_t* cu_tokens,
                                const int32_t* start_pos, const int32_t* work, int num_work,
+                               const int32_t* block_items, int num_blocks, int block_variant,
                                int tiles_per_entry, int cols_per_wave, int splits, int T_total,
                                int nq, int nkv, int d, int page_size, int num_pages, int window,
                                float scale, tff_stream_t stream) {
@@ -804,6 +819,12 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                 "attention_mfma: bad tile width %d", cols_per_wave);
     TFF_REQUIRE(cols_per_wave != 128 || (work && splits == 1),
                 "attention_mfma: blocks of 128 columns take a work table and no key split");
+    if (cols_per_wave == 128) {
+        if (!block_items) num_blocks = num_work;
+        TFF_REQUIRE(num_blocks >= 0 && num_blocks <= num_work && (block_variant == 0 || block_variant == 1),
+                    "attention_mfma: %d blocks for %d work items, variant %d", num_blocks, num_work, block_variant);
+        if (num_blocks == 0) return 0;
+    }
     TFF_REQUIRE(splits >= 1 && splits <= 65535 && nkv <= 65535, "attention_mfma: bad split count %d", splits);
     TFF_REQUIRE(splits == 1 || (part_o && part_ml), "attention_mfma: split keys need a workspace");
     TFF_REQUIRE(work || tiles_per_entry >= 1, "attention_mfma: neither a work table nor a tile count");
@@ -814,7 +835,8 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
     case DTV * 16:                                                                                  \
         return launch_attn<DTV>((const bf16_t*)q, q_stride, (bf16_t*)out, part_o, part_ml,          \
                                 (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,       \
-                                bt_stride, cu_tokens, start_pos, work, num_work, tiles_per_entry,   \
+                                bt_stride, cu_tokens, start_pos, work, num_work, block_items,       \
+                                num_blocks, block_variant, tiles_per_entry,                         \
                                 cols_per_wave, splits, nq, nkv, page_size, window, scale, T_total, s);
     switch (d) {
         TFF_ATTN_CASE(1) TFF_ATTN_CASE(2) TFF_ATTN_CASE(3) TFF_ATTN_CASE(4) TFF_ATTN_CASE(5)

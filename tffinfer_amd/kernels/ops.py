@@ -330,6 +330,66 @@ def _attention_work(batch, G: int, cols: int, device) -> torch.Tensor:
     return cache[key]
 
 
+_cu_count = {}
+
+
+def _num_cus(device) -> int:
+    idx = torch.device(device).index or 0
+    if idx not in _cu_count:
+        _cu_count[idx] = torch.cuda.get_device_properties(idx).multi_processor_count
+    return _cu_count[idx]
+
+
+def _attention_block_work(batch, G: int, nkv: int, window: int, device, cols: int = 128,
+                          bins: int | None = None):
+    """Work table of the block kernel: items (entry, first column) of ``cols``
+    columns, dealt to blocks so that every block goes through about the same
+    number of 32-key slices (an item late in a long prompt sees many times the
+    keys of an early one).  There are at most as many blocks as the device
+    can hold at once, so none waits for another to end.  Returns (items
+    [n, 2], block_items [blocks + 1], blocks)."""
+    cache = getattr(batch, "_attn_work", None)
+    if cache is None:
+        cache = batch._attn_work = {}
+    if bins is None:
+        bins = max(1, _num_cus(device) // max(1, nkv))
+    key = ("blocks", G, nkv, cols, window, bins)
+    if key not in cache:
+        cu, P = batch.host_cu_tokens, batch.host_start_pos
+        items = []                       # (slices, entry, first column)
+        for r in range(len(cu) - 1):
+            ncols = (cu[r + 1] - cu[r]) * G
+            for c0 in range(0, ncols, cols):
+                first = P[r] + c0 // G
+                last = P[r] + (min(c0 + cols, ncols) - 1) // G
+                lo = max(0, first - window + 1) if window > 0 else 0
+                items.append((last // 32 - lo // 32 + 1, r, c0))
+        if len(items) <= bins:
+            order = sorted(items, reverse=True)        # the longest start first
+            starts = list(range(len(order) + 1))
+        else:
+            # longest first, each to the block with the least to do so far
+            import heapq
+            loads = [(0, b) for b in range(bins)]
+            heapq.heapify(loads)
+            per_bin = [[] for _ in range(bins)]
+            for it in sorted(items, reverse=True):
+                load, b = heapq.heappop(loads)
+                per_bin[b].append(it)
+                heapq.heappush(loads, (load + it[0], b))
+            order, starts = [], [0]
+            for lst in per_bin:
+                order.extend(lst)
+                starts.append(len(order))
+        flat = [x for it in order for x in it[1:]]
+        cache[key] = (torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(device),
+                      torch.tensor(starts, dtype=torch.int32).to(device), len(starts) - 1)
+    return cache[key]
+
+
+_BLOCK_VARIANT = int(__import__('os').environ.get('TFF_ATTN_BLOCK_VARIANT', '1'))
+
+
 def pick_splits(waves: int, max_context: int) -> int:
     """Into how many runs the keys of a decoding request are split so that
     the launch has enough waves to pull on all of HBM: about 1024 waves, at
@@ -338,9 +398,12 @@ def pick_splits(waves: int, max_context: int) -> int:
 
 
 def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,
-                   scale: float | None = None, splits: int | None = None) -> torch.Tensor:
+                   scale: float | None = None, splits: int | None = None,
+                   block_bins: int | None = None) -> torch.Tensor:
     """bfloat16 attention of the step's tokens on the matrix cores; decode-only
-    steps split each request's keys over several waves and merge them."""
+    steps split each request's keys over several waves and merge them.
+    ``splits`` and ``block_bins`` (blocks per kv head that share the work of
+    long portions) override the choices made from the step's sizes."""
     _req(q, "attention q", torch.bfloat16, 2)
     T = q.shape[0]
     if q.shape[1] < nq * d:
@@ -362,7 +425,8 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
         scale = 1.0 / math.sqrt(d)
     out = torch.empty(T, nq * d, dtype=q.dtype, device=q.device)
     L = _lib.load()
-    part_o = part_ml = None
+    part_o = part_ml = block_items = None
+    num_blocks = 0
     if batch.max_new_tokens == 1:
         tiles = -(-G // 16)
         work, num_work, cols = None, R * tiles, 16
@@ -376,13 +440,18 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
         # long portions: blocks of four waves that share their keys through LDS (128 columns);
         # short ones: a wave of its own per 32 or 16 columns
         cols = 128 if batch.max_new_tokens * G > 64 else (32 if batch.max_new_tokens * G > 16 else 16)
-        work = _attention_work(batch, G, cols, q.device)
+        if cols == 128:
+            work, block_items, num_blocks = _attention_block_work(batch, G, nkv, int(window), q.device,
+                                                                  bins=block_bins)
+        else:
+            work = _attention_work(batch, G, cols, q.device)
         num_work = work.shape[0]
     dest = out
     _lib.check(L.tff_attention_mfma(
         q.data_ptr(), q.stride(0), dest.data_ptr(), _ptr(part_o), _ptr(part_ml), k_cache.data_ptr(),
         v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(),
-        batch.start_pos.data_ptr(), _ptr(work), num_work, tiles, cols, splits, T, nq, nkv, d,
+        batch.start_pos.data_ptr(), _ptr(work), num_work, _ptr(block_items), num_blocks,
+        _BLOCK_VARIANT, tiles, cols, splits, T, nq, nkv, d,
         k_cache.shape[2], k_cache.shape[0], int(window), float(scale), _stream()))
     if splits > 1:
         _lib.check(L.tff_attention_split_reduce(part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(),
