@@ -103,6 +103,37 @@ def test_linear(M, N, K, dtype):
     _close(out_s, wide[:, :K].double().cpu() @ w.double().T, 2e-6 if dtype == torch.float32 else 2e-5, "strided")
 
 
+@pytest.mark.parametrize("M,N,K", [(40, 1024, 2056), (520, 264, 1544), (8, 64, 64)])
+def test_linear_partial_sums_feed_the_norm(M, N, K):
+    """Where the product splits K over blocks it can hand out the partial sums; the fused
+    residual sum and norm adds them up itself, in order, to what the whole product gives."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(M + N)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(N, K, generator=g) * 0.1).to(torch.bfloat16)
+    pw = ops.pack_weight(w.to(DEV))
+    whole = ops.linear(x, pw, out_dtype=torch.float32)
+    parts = ops.linear(x, pw, out_dtype=torch.float32, partials=True)
+    if M == 8:
+        assert parts.dim() == 2          # nothing to split here: the plain result
+    else:
+        assert parts.dim() == 3 and parts.shape[0] > 1 and tuple(parts.shape[1:]) == (M, N)
+        acc = parts[0].clone()
+        for p in parts[1:]:
+            acc += p
+        assert torch.equal(acc, whole)
+    resid = torch.randn(M, N, generator=g).to(DEV)
+    nw = (1 + 0.1 * torch.randn(N, generator=g)).to(DEV)
+    r1, r2 = resid.clone(), resid.clone()
+    y1 = ops.add_rmsnorm(r1, whole, nw, 1e-6, torch.float32)
+    y2 = ops.add_rmsnorm(r2, parts, nw, 1e-6, torch.float32)
+    assert torch.equal(r1, r2) and torch.equal(y1, y2)
+    rows = torch.tensor([M - 1, 0], dtype=torch.int32, device=DEV)
+    z1 = ops.add_rmsnorm(resid.clone(), whole, nw, 1e-6, torch.bfloat16, rows=rows)
+    z2 = ops.add_rmsnorm(resid.clone(), parts, nw, 1e-6, torch.bfloat16, rows=rows)
+    assert torch.equal(z1, z2)
+
+
 def test_linear_identity_and_layout():
     """[out, in] layout: a non-square weight picks input columns."""
     ops = _ops()

@@ -23,7 +23,7 @@ int tff_check_launch(const char* what) {
     return 0;
 }
 TFF_API const char* tff_last_error() { return g_error; }
-TFF_API int tff_abi_version() { return 7; }
+TFF_API int tff_abi_version() { return 8; }
 
 // ----------------------------------------------------------------- embed ---
 // x[t, :] = E[token[t], :]   (reference: src/kernel/cpu/embedding.cpp:34-49,
@@ -60,10 +60,12 @@ TFF_API int tff_embed(const void* table, const int32_t* ids, float* out, int T, 
 // y_j = v_j * rsqrt(mean(v^2) + eps) * w_j, v = resid (+ delta)
 // (reference: src/kernel/cuda/norm.cu:31-48; the residual sum of
 // src/kernel/cuda/binary.cu:16-29 is folded in).
+// delta may come as `planes` partial sums, `plane` elements apart, which are added up first,
+// plane 0, 1, ... in turn.
 template <typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __restrict__ delta,
-                                   const float* __restrict__ w, float eps, TO* __restrict__ out,
-                                   const int32_t* __restrict__ rows, int H) {
+                                   int planes, size_t plane, const float* __restrict__ w, float eps,
+                                   TO* __restrict__ out, const int32_t* __restrict__ rows, int H) {
     __shared__ float red[17];
     const int i = blockIdx.x;
     const int r = rows ? rows[i] : i;
@@ -73,7 +75,11 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __res
     float ss = 0.f;
     for (int j = threadIdx.x; j < H; j += blockDim.x) {
         float v = x[j];
-        if (dl) v += dl[j];
+        if (dl) {
+            float d = dl[j];
+            for (int p = 1; p < planes; ++p) d += dl[p * plane + j];
+            v += d;
+        }
         if (store) x[j] = v;
         ss = fmaf(v, v, ss);
     }
@@ -82,7 +88,11 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __res
     TO* o = out + (size_t)i * H;
     for (int j = threadIdx.x; j < H; j += blockDim.x) {
         float v = x[j];
-        if (dl && !store) v += dl[j];
+        if (dl && !store) {
+            float d = dl[j];
+            for (int p = 1; p < planes; ++p) d += dl[p * plane + j];
+            v += d;
+        }
         o[j] = from_f32<TO>(v * rr * w[j]);
     }
 }
@@ -100,12 +110,23 @@ __device__ __forceinline__ void store_out4<bf16_t>(bf16_t* o, float4 v) {
     *reinterpret_cast<uint2*>(o) = pk.u;
 }
 
+__device__ __forceinline__ float4 delta_sum4(const float4* d4, int j, int planes, size_t plane4) {
+    float4 d = d4[j];
+    for (int p = 1; p < planes; ++p) {
+        const float4 e = d4[p * plane4 + j];
+        d.x += e.x; d.y += e.y; d.z += e.z; d.w += e.w;
+    }
+    return d;
+}
+
 template <typename TO>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid,
                                                                const float* __restrict__ delta,
+                                                               int planes, size_t plane,
                                                                const float* __restrict__ w, float eps,
                                                                TO* __restrict__ out,
                                                                const int32_t* __restrict__ rows, int H) {
+    const size_t plane4 = plane >> 2;
     __shared__ float red[17];
     const int i = blockIdx.x, tid = threadIdx.x;
     const int r = rows ? rows[i] : i;
@@ -121,7 +142,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
         const int j = tid + it * 256;
         if (j < H4) {
             float4 v = x4[j];
-            if (d4) { const float4 dv = d4[j]; v.x += dv.x; v.y += dv.y; v.z += dv.z; v.w += dv.w; }
+            if (d4) { const float4 dv = delta_sum4(d4, j, planes, plane4); v.x += dv.x; v.y += dv.y; v.z += dv.z; v.w += dv.w; }
             if (store) x4[j] = v;
             cache[it] = v;
             ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
@@ -129,7 +150,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     }
     for (int j = tid + 1024; j < H4; j += 256) {
         float4 v = x4[j];
-        if (d4) { const float4 dv = d4[j]; v.x += dv.x; v.y += dv.y; v.z += dv.z; v.w += dv.w; }
+        if (d4) { const float4 dv = delta_sum4(d4, j, planes, plane4); v.x += dv.x; v.y += dv.y; v.z += dv.z; v.w += dv.w; }
         if (store) x4[j] = v;
         ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
     }
@@ -146,17 +167,21 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     }
     for (int j = tid + 1024; j < H4; j += 256) {
         float4 v = x4[j];
-        if (d4 && !store) { const float4 dv = d4[j]; v.x += dv.x; v.y += dv.y; v.z += dv.z; v.w += dv.w; }
+        if (d4 && !store) { const float4 dv = delta_sum4(d4, j, planes, plane4); v.x += dv.x; v.y += dv.y; v.z += dv.z; v.w += dv.w; }
         const float4 wv = w4[j];
         store_out4<TO>(o + 4 * j, make_float4(v.x * rr * wv.x, v.y * rr * wv.y, v.z * rr * wv.z, v.w * rr * wv.w));
     }
 }
 
-TFF_API int tff_add_rmsnorm(float* resid, const float* delta, const float* weight, float eps,
-                            void* out, const int32_t* rows, int n, int H, int out_dtype,
-                            tff_stream_t stream) {
+TFF_API int tff_add_rmsnorm(float* resid, const float* delta, int delta_planes, size_t delta_plane,
+                            const float* weight, float eps, void* out, const int32_t* rows, int n,
+                            int H, int out_dtype, tff_stream_t stream) {
     TFF_REQUIRE(resid && weight && out, "add_rmsnorm: null pointer");
     TFF_REQUIRE(n >= 0 && H > 0, "add_rmsnorm: bad sizes n=%d H=%d", n, H);
+    TFF_REQUIRE(!delta || (delta_planes >= 1 && (delta_planes == 1 || delta_plane % 4 == 0)),
+                "add_rmsnorm: %d planes of partial sums, %zu elements apart", delta_planes, delta_plane);
+    const int planes = delta ? delta_planes : 0;
+    const size_t plane = delta_plane;
     if (n == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     TFF_REQUIRE(out_dtype == TFF_F32 || out_dtype == TFF_BF16, "add_rmsnorm: unknown dtype %d", out_dtype);
@@ -164,16 +189,16 @@ TFF_API int tff_add_rmsnorm(float* resid, const float* delta, const float* weigh
                      ((uintptr_t)out % 16) == 0 && (!delta || ((uintptr_t)delta % 16) == 0);
     if (vec) {
         if (out_dtype == TFF_F32)
-            add_rmsnorm_vec_kernel<float><<<n, 256, 0, s>>>(resid, delta, weight, eps, (float*)out, rows, H);
+            add_rmsnorm_vec_kernel<float><<<n, 256, 0, s>>>(resid, delta, planes, plane, weight, eps, (float*)out, rows, H);
         else
-            add_rmsnorm_vec_kernel<bf16_t><<<n, 256, 0, s>>>(resid, delta, weight, eps, (bf16_t*)out, rows, H);
+            add_rmsnorm_vec_kernel<bf16_t><<<n, 256, 0, s>>>(resid, delta, planes, plane, weight, eps, (bf16_t*)out, rows, H);
         return tff_check_launch("add_rmsnorm");
     }
     const int threads = H >= 2048 ? 1024 : 256;
     if (out_dtype == TFF_F32)
-        add_rmsnorm_kernel<float><<<n, threads, 0, s>>>(resid, delta, weight, eps, (float*)out, rows, H);
+        add_rmsnorm_kernel<float><<<n, threads, 0, s>>>(resid, delta, planes, plane, weight, eps, (float*)out, rows, H);
     else
-        add_rmsnorm_kernel<bf16_t><<<n, threads, 0, s>>>(resid, delta, weight, eps, (bf16_t*)out, rows, H);
+        add_rmsnorm_kernel<bf16_t><<<n, threads, 0, s>>>(resid, delta, planes, plane, weight, eps, (bf16_t*)out, rows, H);
     return tff_check_launch("add_rmsnorm");
 }
 

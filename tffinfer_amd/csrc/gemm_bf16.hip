@@ -82,7 +82,16 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
     const int fr = lane & 15, fg = lane >> 4;
-    const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+    // Blocks are handed to the eight XCDs in turn, and each XCD has an L2 of its own: block b
+    // of the launch runs on XCD b % 8.  Column tiles are therefore dealt to the XCDs (tile t to
+    // XCD t % 8), and the blocks an XCD runs one after the other walk the row tiles of one
+    // column tile before the next: a tile of W is fetched into one L2 only, and the (smaller) A
+    // is what every L2 holds.
+    const int TM = (M + BM - 1) / BM;
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int tn = (seq / TM) * 8 + xcd, tm = seq % TM;
+    if (tn * BN >= N) return;   // the launch is padded to whole groups of eight column tiles
+    const int m0 = tm * BM, n0 = tn * BN;
     const int NB = (N + 15) / 16;
     const int nk = (K + 63) / 64;
     // With gridDim.z > 1 the blocks of one tile split K among them and leave partial sums in
@@ -238,12 +247,14 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
 // splits > 1: the blocks of a tile split K among them; part holds splits * M * N floats
 template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU = false>
 static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
-                          int c_dtype, int n_out, hipStream_t s, int splits = 1, float* part = nullptr) {
+                          int c_dtype, int n_out, hipStream_t s, int splits = 1, float* part = nullptr,
+                          bool reduce = true) {
     const int KB = (K + 31) / 32;
     constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
     if (splits <= 1 || !part) { splits = 1; part = nullptr; }
-    const dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN, splits);
-    TFF_REQUIRE(grid.y <= 65535, "gemm: too many columns N=%d", N);
+    const long tiles = (long)((M + BM - 1) / BM) * (((N + BN - 1) / BN + 7) / 8 * 8);
+    TFF_REQUIRE(tiles < (1L << 31), "gemm: too many tiles for M=%d N=%d", M, N);
+    const dim3 grid((unsigned)tiles, 1, splits);
     if (c_dtype == TFF_F32)
         gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, float>
             <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out, part);
@@ -251,7 +262,7 @@ static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int
         gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, bf16_t>
             <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out, part);
     if (int rc = tff_check_launch("gemm_bf16_async")) return rc;
-    if (splits > 1) {
+    if (splits > 1 && reduce) {
         const int No = GLU ? n_out : N;
         const long threads = (long)M * ((No + 3) / 4);
         const int blocks = (int)((threads + 255) / 256);
@@ -474,8 +485,11 @@ TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype) {
 // glu_out > 0: W holds gate and up groups in turn (N = 2 * ceil16(glu_out) rows) and C is
 // [M, glu_out] = silu(gate) * up.  workspace: room for partial sums (tff_gemm_workspace_bytes);
 // with less the blocks do not split K.
+// keep_partials: where the plan splits K, the partial sums stay in the workspace
+// ([splits, M, N] float32) for the caller to add up, and C is not written.
 int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
-                  int c_dtype, int glu_out, float* workspace, size_t workspace_bytes, hipStream_t s) {
+                  int c_dtype, int glu_out, float* workspace, size_t workspace_bytes,
+                  int keep_partials, hipStream_t s) {
     TFF_REQUIRE(K % 8 == 0 && lda % 8 == 0,
                 "gemm: the bfloat16 product needs the inner size (K=%d, row stride %d) to be a multiple of 8",
                 K, lda);
@@ -485,6 +499,9 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
     GemmPlan plan = plan_for(M, N, K);
     if (!workspace || workspace_bytes < (size_t)plan.splits * M * N * sizeof(float)) plan.splits = 1;
     const int S = plan.splits;
+    const bool red = !keep_partials;
+    TFF_REQUIRE(!keep_partials || (glu_out == 0 && c_dtype == TFF_F32),
+                "gemm: partial sums are kept for a plain float32 result only");
     if (glu_out > 0) {
         TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
                     "gemm: a gated weight of %d rows does not fit %d output columns", N, glu_out);
@@ -514,11 +531,11 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
             if (M <= 32) return launch_skinny<2, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
             return launch_skinny<4, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
         }
-        return launch_async_g<2, 2, 2, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace);
+        return launch_async_g<2, 2, 2, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     }
     if (plan.tile == 128)
-        return launch_async_g<2, 2, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace);
-    return launch_async_g<4, 4, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace);
+        return launch_async_g<2, 2, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+    return launch_async_g<4, 4, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
 }
 
 int tff_gemm_f32(const float* A, const float* W, void* C, int M, int N, int K, int lda,
@@ -526,20 +543,21 @@ int tff_gemm_f32(const float* A, const float* W, void* C, int M, int N, int K, i
 
 TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda,
                      int ab_dtype, int c_dtype, int w_packed, int glu_out, void* workspace,
-                     size_t workspace_bytes, tff_stream_t stream) {
+                     size_t workspace_bytes, int keep_partials, tff_stream_t stream) {
     TFF_REQUIRE(A && W && C, "gemm: null pointer");
     TFF_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K, "gemm: bad sizes M=%d N=%d K=%d lda=%d", M, N, K, lda);
     if (M == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (ab_dtype == TFF_F32) {
-        TFF_REQUIRE(!w_packed && glu_out == 0, "gemm: the float32 product takes a plain row-major weight");
+        TFF_REQUIRE(!w_packed && glu_out == 0 && !keep_partials,
+                    "gemm: the float32 product takes a plain row-major weight and keeps no partial sums");
         return tff_gemm_f32((const float*)A, (const float*)W, C, M, N, K, lda, c_dtype, s);
     }
     if (ab_dtype == TFF_BF16) {
         TFF_REQUIRE(w_packed, "gemm: the bfloat16 product takes a weight in fragment order");
         TFF_REQUIRE(((uintptr_t)workspace % 16) == 0, "gemm: the workspace must be 16-byte aligned");
         return tff_gemm_bf16((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, c_dtype, glu_out,
-                             (float*)workspace, workspace ? workspace_bytes : 0, s);
+                             (float*)workspace, workspace ? workspace_bytes : 0, keep_partials, s);
     }
     return tff_fail("gemm: unknown operand type %d", ab_dtype);
 }

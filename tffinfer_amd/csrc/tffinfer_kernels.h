@@ -23,9 +23,11 @@ TFF_API int tff_embed(const void* table, const int32_t* ids, float* out,
 //   v = resid[r] + (delta ? delta[r] : 0);  out[i] = v * rsqrt(mean(v^2)+eps) * w
 // rows == null: r = i for i < n, and resid[r] = v is stored back.
 // rows != null: r = rows[i]; resid is left as it is (norm of gathered rows).
-TFF_API int tff_add_rmsnorm(float* resid, const float* delta, const float* weight,
-                            float eps, void* out, const int32_t* rows, int n, int H,
-                            int out_dtype, tff_stream_t stream);
+// delta may come as delta_planes partial sums, delta_plane elements apart (what
+// tff_gemm leaves with keep_partials); they are added up first, plane 0, 1, ...
+TFF_API int tff_add_rmsnorm(float* resid, const float* delta, int delta_planes, size_t delta_plane,
+                            const float* weight, float eps, void* out, const int32_t* rows, int n,
+                            int H, int out_dtype, tff_stream_t stream);
 
 // RMS norm of a plain [n, H] tensor of `dtype` with a float32 weight.
 TFF_API int tff_rmsnorm(const void* x, const float* weight, float eps, void* out,
@@ -40,9 +42,13 @@ TFF_API int tff_rmsnorm(const void* x, const float* weight, float eps, void* out
 // C is [M, glu_out] = silu(gate) * up.
 // workspace (may be null): device memory of tff_gemm_workspace_bytes() bytes the
 // product may keep partial sums in; with less it takes a path that needs none.
+// keep_partials (float32 result, no GLU): if the workspace is used, that is, if
+// tff_gemm_workspace_bytes() > 0 and the workspace has that size, the partial
+// sums [bytes / (M * N * 4), M, N] are left there for the caller to add up
+// (tff_add_rmsnorm takes them as they are) and C is not written.
 TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda,
                      int ab_dtype, int c_dtype, int w_packed, int glu_out, void* workspace,
-                     size_t workspace_bytes, tff_stream_t stream);
+                     size_t workspace_bytes, int keep_partials, tff_stream_t stream);
 TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype);
 
 // bfloat16 row-major [N, K] (K a multiple of 8) -> fragment order: tiles of

@@ -158,17 +158,22 @@ def add_rmsnorm(resid: torch.Tensor, delta: torch.Tensor | None, weight: torch.T
                 out_dtype: torch.dtype, rows: torch.Tensor | None = None,
                 out: torch.Tensor | None = None) -> torch.Tensor:
     """``resid += delta`` (when given and ``rows`` is None) and the RMS norm of
-    the sum; with ``rows`` the norm of those rows only, ``resid`` untouched."""
+    the sum; with ``rows`` the norm of those rows only, ``resid`` untouched.
+    ``delta`` may be a stack [S, T, H] of partial sums (``linear`` with
+    ``partials=True``): they are added up first, in order."""
     _req(resid, "add_rmsnorm resid", torch.float32, 2)
     H = resid.shape[1]
     _req(weight, "add_rmsnorm weight", torch.float32, 1)
     if weight.numel() != H:
         raise _lib.KernelError(f"add_rmsnorm: weight has {weight.numel()} elements, rows have {H}")
+    planes, plane = 1, 0
     if delta is not None:
-        _req(delta, "add_rmsnorm delta", torch.float32, 2)
-        if delta.shape != resid.shape:
+        _req(delta, "add_rmsnorm delta", torch.float32, 3 if delta.dim() == 3 else 2)
+        if tuple(delta.shape[-2:]) != tuple(resid.shape):
             raise _lib.KernelError(
                 f"add_rmsnorm: delta {tuple(delta.shape)} does not match resid {tuple(resid.shape)}")
+        if delta.dim() == 3:
+            planes, plane = delta.shape[0], delta.stride(0)
     if rows is not None:
         _req(rows, "add_rmsnorm rows", torch.int32, 1)
         n = rows.numel()
@@ -181,7 +186,7 @@ def add_rmsnorm(resid: torch.Tensor, delta: torch.Tensor | None, weight: torch.T
         if tuple(out.shape) != (n, H):
             raise _lib.KernelError(f"add_rmsnorm out: shape {tuple(out.shape)} is not {(n, H)}")
     L = _lib.load()
-    _lib.check(L.tff_add_rmsnorm(resid.data_ptr(), _ptr(delta), weight.data_ptr(), float(eps),
+    _lib.check(L.tff_add_rmsnorm(resid.data_ptr(), _ptr(delta), planes, plane, weight.data_ptr(), float(eps),
                                  out.data_ptr(), _ptr(rows), n, H, dtype_code(out_dtype), _stream()))
     return out
 
@@ -201,9 +206,14 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
 
 
 def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
-           out: torch.Tensor | None = None) -> torch.Tensor:
+           out: torch.Tensor | None = None, partials: bool = False) -> torch.Tensor:
     """``x . weight^T`` for x [M, K] (rows may be strided) and weight [N, K]:
-    a row-major float32 tensor, or a PackedWeight for bfloat16."""
+    a row-major float32 tensor, or a PackedWeight for bfloat16.
+
+    ``partials=True`` (float32 result): where the product splits K over
+    blocks, the partial sums are returned as they are, [S, M, N], for a
+    consumer that adds them up anyway (``add_rmsnorm``); else the result is
+    [M, N] as always."""
     if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
         raise _lib.KernelError("linear x: expected a GPU matrix with unit inner stride")
     packed = isinstance(weight, PackedWeight)
@@ -223,19 +233,22 @@ def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
     out_dtype = out_dtype or x.dtype
     glu_out = weight.glu_out if packed else 0
     n_out = glu_out or N
-    if out is None:
+    L = _lib.load()
+    # some shapes (few columns for the rows) split K over blocks and need room for partial sums
+    ws_bytes = L.tff_gemm_workspace_bytes(M, N, K, dtype_code(x.dtype)) if packed else 0
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=x.device) if ws_bytes else None
+    keep = bool(partials and ws is not None and out is None and out_dtype == torch.float32 and not glu_out)
+    if keep:
+        out = ws.view(-1, M, N)
+    elif out is None:
         out = torch.empty(M, n_out, dtype=out_dtype, device=x.device)
     else:
         _req(out, "linear out", out_dtype, 2)
         if tuple(out.shape) != (M, n_out):
             raise _lib.KernelError(f"linear out: shape {tuple(out.shape)} is not {(M, n_out)}")
-    L = _lib.load()
-    # some shapes (a few dozen rows, few columns) split K over blocks and need room for partial sums
-    ws_bytes = L.tff_gemm_workspace_bytes(M, N, K, dtype_code(x.dtype)) if packed else 0
-    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=x.device) if ws_bytes else None
     _lib.check(L.tff_gemm(x.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K, lda,
                           dtype_code(x.dtype), dtype_code(out_dtype), 1 if packed else 0, glu_out,
-                          _ptr(ws), ws_bytes, _stream()))
+                          _ptr(ws), ws_bytes, 1 if keep else 0, _stream()))
     return out
 
 

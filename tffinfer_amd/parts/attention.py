@@ -80,4 +80,4 @@ class GQAttention(Mixer):
         ops.qk_norm_rope_kv(qkv, nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0,
                             table, pairing, b.positions, kv.slot_mapping, kv.k_cache, kv.v_cache)
         o = ops.paged_attention(qkv, nq, nkv, d, kv, b, self.window, self.scale)
-        return ops.linear(o, self.w_o, out_dtype=torch.float32)
+        return ops.linear(o, self.w_o, out_dtype=torch.float32, partials=True)

@@ -89,7 +89,10 @@ class Norm(Part):
                 rows: torch.Tensor | None = None) -> torch.Tensor:
         """Adds ``delta`` into the float32 residual stream ``resid`` (when
         ``rows`` is None) and returns the norm of the sum in the activation
-        type; with ``rows`` returns the norm of those rows only."""
+        type; with ``rows`` returns the norm of those rows only.  ``delta`` is
+        what a mixer or feed-forward returned: [T, hidden], or a stack
+        [S, T, hidden] of partial sums to be added up (``ops.add_rmsnorm``
+        takes both)."""
         raise NotImplementedError
 
 
@@ -104,13 +107,15 @@ class Mixer(Part):
 
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
         """x [T, hidden] in the activation type -> float32 [T, hidden] to be
-        added to the residual stream."""
+        added to the residual stream (or [S, T, hidden], whose sum over S is:
+        what ``ops.linear(..., partials=True)`` returns)."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
-        """x [T, hidden] in the activation type -> float32 [T, hidden]."""
+        """x [T, hidden] in the activation type -> float32 [T, hidden] (or a
+        stack of partial sums [S, T, hidden], as for a mixer)."""
         raise NotImplementedError
 
 

@@ -47,4 +47,4 @@ class SwiGLU(FeedForward):
     def forward(self, ctx, x):
         gu = ctx.ops.linear(x, self.w_gate_up)
         m = gu if getattr(self.w_gate_up, "glu_out", 0) else ctx.ops.swiglu(gu)
-        return ctx.ops.linear(m, self.w_down, out_dtype=torch.float32)
+        return ctx.ops.linear(m, self.w_down, out_dtype=torch.float32, partials=True)
