@@ -508,10 +508,14 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __r
 }
 
 // ------------------------------------------------- prompt portions, by block ---
-// For portions of many tokens a block of four waves shares its keys and values:
+// For portions of many tokens a block of NW waves shares its keys and values:
 // every 32-key slice is copied once from the pages into LDS (by the load unit,
-// global_load_lds_dwordx4, in MFMA operand order, two slices in flight) and read
-// from there by all four waves, each of which works on NQT column tiles.
+// global_load_lds_dwordx4, in MFMA operand order, three slices in flight) and
+// read from there by all waves, each of which works on NQT column tiles.  Under
+// a causal mask the last columns of a prompt see many times the keys of the
+// first; so that no CU idles while another works through a long run, a block
+// is given several work items with about the same total of slices as every
+// other block's.
 //
 // Within a slice the 16 rows of key tile t are the keys (r / 4) * 8 + t * 4 + r % 4:
 // lane (col, g) then holds the scores of the 8 consecutive keys g*8 .. g*8+7,
@@ -752,21 +756,16 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
                        const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* block_tables,
                        int bt_stride, const int32_t* cu_tokens, const int32_t* start_pos,
                        const int32_t* work, int num_work, const int32_t* block_items, int num_blocks,
-                       int block_variant, int tiles_per_entry, int cols_per_wave,
+                       int tiles_per_entry, int cols_per_wave,
                        int splits, int nq, int nkv, int page_size, int window, float scale,
                        int T_total, hipStream_t s) {
     int page_shift = -1;
     if ((page_size & (page_size - 1)) == 0)
         for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
-    if (cols_per_wave == 128) {   // blocks that share their keys through LDS
-        if (block_variant == 1)   // eight waves, one column tile each
-            attn_mfma_block_kernel<DT, 1, 8><<<dim3(num_blocks, nkv), 512, 0, s>>>(
-                q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
-                block_items, nq, nkv, page_size, page_shift, window, scale);
-        else                      // four waves, two column tiles each
-            attn_mfma_block_kernel<DT, 2, 4><<<dim3(num_blocks, nkv), 256, 0, s>>>(
-                q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
-                block_items, nq, nkv, page_size, page_shift, window, scale);
+    if (cols_per_wave == 128) {   // blocks of eight waves that share their keys through LDS
+        attn_mfma_block_kernel<DT, 1, 8><<<dim3(num_blocks, nkv), 512, 0, s>>>(
+            q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
+            block_items, nq, nkv, page_size, page_shift, window, scale);
         return tff_check_launch("attention_mfma_block");
     }
     const dim3 grid(num_work, nkv, splits);
@@ -802,7 +801,7 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                const void* k_cache, const void* v_cache,
                                const int32_t* block_tables, int bt_stride, const int32_t* cu_tokens,
                                const int32_t* start_pos, const int32_t* work, int num_work,
-                               const int32_t* block_items, int num_blocks, int block_variant,
+                               const int32_t* block_items, int num_blocks,
                                int tiles_per_entry, int cols_per_wave, int splits, int T_total,
                                int nq, int nkv, int d, int page_size, int num_pages, int window,
                                float scale, tff_stream_t stream) {
@@ -821,8 +820,8 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                 "attention_mfma: blocks of 128 columns take a work table and no key split");
     if (cols_per_wave == 128) {
         if (!block_items) num_blocks = num_work;
-        TFF_REQUIRE(num_blocks >= 0 && num_blocks <= num_work && (block_variant == 0 || block_variant == 1),
-                    "attention_mfma: %d blocks for %d work items, variant %d", num_blocks, num_work, block_variant);
+        TFF_REQUIRE(num_blocks >= 0 && num_blocks <= num_work,
+                    "attention_mfma: %d blocks for %d work items", num_blocks, num_work);
         if (num_blocks == 0) return 0;
     }
     TFF_REQUIRE(splits >= 1 && splits <= 65535 && nkv <= 65535, "attention_mfma: bad split count %d", splits);
@@ -836,7 +835,7 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
         return launch_attn<DTV>((const bf16_t*)q, q_stride, (bf16_t*)out, part_o, part_ml,          \
                                 (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,       \
                                 bt_stride, cu_tokens, start_pos, work, num_work, block_items,       \
-                                num_blocks, block_variant, tiles_per_entry,                         \
+                                num_blocks, tiles_per_entry,                                        \
                                 cols_per_wave, splits, nq, nkv, page_size, window, scale, T_total, s);
     switch (d) {
         TFF_ATTN_CASE(1) TFF_ATTN_CASE(2) TFF_ATTN_CASE(3) TFF_ATTN_CASE(4) TFF_ATTN_CASE(5)

@@ -94,17 +94,16 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out,
 // gets tiles_per_entry waves.  splits > 1 cuts each request's keys into runs
 // whose partial results (part_o [splits, T, nq, d], part_ml [splits, T, nq, 2],
 // float32) tff_attention_split_reduce merges.  cols_per_wave 128: work items
-// are runs of 128 columns for a block that stages keys and values in LDS
-// (block_variant 0: four waves with two column tiles each, 1: eight waves with
-// one); block b works through items block_items[b] .. block_items[b + 1] of
-// the work table (block_items null: item b).  Head sizes 16..128 in steps of
+// are runs of 128 columns for a block of eight waves that stages keys and
+// values in LDS; block b works through items block_items[b] ..
+// block_items[b + 1] of the work table (block_items null: item b).  Head sizes 16..128 in steps of
 // 16, 192 and 256; pages a multiple of 8; values transposed in their pages.
 TFF_API int tff_attention_mfma_supported(int d, int page_size);
 TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* part_o, float* part_ml,
                                const void* k_cache, const void* v_cache,
                                const int32_t* block_tables, int bt_stride, const int32_t* cu_tokens,
                                const int32_t* start_pos, const int32_t* work, int num_work,
-                               const int32_t* block_items, int num_blocks, int block_variant,
+                               const int32_t* block_items, int num_blocks,
                                int tiles_per_entry, int cols_per_wave, int splits, int T_total,
                                int nq, int nkv, int d, int page_size, int num_pages, int window,
                                float scale, tff_stream_t stream);

@@ -400,9 +400,6 @@ def _attention_block_work(batch, G: int, nkv: int, window: int, device, cols: in
     return cache[key]
 
 
-_BLOCK_VARIANT = int(__import__('os').environ.get('TFF_ATTN_BLOCK_VARIANT', '1'))
-
-
 def pick_splits(waves: int, max_context: int) -> int:
     """Into how many runs the keys of a decoding request are split so that
     the launch has enough waves to pull on all of HBM: about 1024 waves, at
@@ -463,8 +460,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
     _lib.check(L.tff_attention_mfma(
         q.data_ptr(), q.stride(0), dest.data_ptr(), _ptr(part_o), _ptr(part_ml), k_cache.data_ptr(),
         v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(),
-        batch.start_pos.data_ptr(), _ptr(work), num_work, _ptr(block_items), num_blocks,
-        _BLOCK_VARIANT, tiles, cols, splits, T, nq, nkv, d,
+        batch.start_pos.data_ptr(), _ptr(work), num_work, _ptr(block_items), num_blocks, tiles, cols, splits, T, nq, nkv, d,
         k_cache.shape[2], k_cache.shape[0], int(window), float(scale), _stream()))
     if splits > 1:
         _lib.check(L.tff_attention_split_reduce(part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(),
