@@ -129,6 +129,48 @@ def test_eos_stops(model_dirs):
     assert stop.output == full[:cut] and stop.finish_reason == "stop"
 
 
+@pytest.mark.parametrize("dtype,use_graphs", [("float32", True), ("bfloat16", True), ("bfloat16", False)])
+def test_steps_launched_ahead_give_the_same_tokens(model_dirs, dtype, use_graphs):
+    """Decode steps launched before the tokens of the step in flight are read: the same
+    outputs as with one step at a time, with requests that end at different lengths, one
+    that ends on a token of its own choosing, more requests than slots and a pool that
+    runs out."""
+    from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
+    d = model_dirs["B"]
+    V = read_config(d)["vocab_size"]
+    prompts = [random_tokens(n, V, 170 + n) for n in (3, 17, 31, 9, 26, 5)]
+    sc = [SamplingConfig("random", temperature=0.7, seed=30 + i) if i % 2 else SamplingConfig() for i in range(6)]
+    lens = [24, 7, 30, 16, 1, 21]
+    outs = {}
+    for ahead in (False, True):
+        opt = EngineOptions(dtype=dtype, page_size=8, num_pages=24, max_num_seqs=4, max_num_batched_tokens=48,
+                            prefill_chunk=24, run_ahead=ahead, use_graphs=use_graphs)
+        eng = LLMEngine.from_model_dir(d, opt)
+        eos = None
+        if ahead:   # request 2 stops at the token it chose as its 12th
+            eos = outs[False][2][11]
+        for i, (p, s, n) in enumerate(zip(prompts, sc, lens)):
+            eng.add_request(p, s, max_new_tokens=n, ignore_eos=not (ahead and i == 2),
+                            eos_token_id=eos if i == 2 else None, request_id=i)
+        got = {i: [] for i in range(6)}
+        fin = {}
+        while eng.has_work:
+            for rid, tok, done in eng.step():
+                got[rid].append(tok)
+                if done:
+                    fin[rid] = True
+        assert len(fin) == 6
+        assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
+        assert (eng.steps_ahead > 10) == ahead
+        outs[ahead] = got
+    for i in range(6):
+        want = outs[False][i]
+        if i == 2:
+            want = want[:want.index(want[11]) + 1]
+        assert outs[True][i] == want, f"request {i}"
+        assert len(outs[False][i]) == lens[i]
+
+
 def test_command_line(model_dirs):
     d = model_dirs["A"]
     prompt = [7, 8, 9, 10, 11]

@@ -165,10 +165,14 @@ class DecodeGraph:
         torch.cuda.current_stream(rn.device).wait_stream(side)
         torch.cuda.synchronize(rn.device)
 
-    def run(self, entries) -> torch.Tensor:
+    def run(self, entries, token_source: torch.Tensor | None = None) -> torch.Tensor:
+        """``token_source``: int32 [len(entries)] on the device with the step's tokens, for a
+        step that is launched before the host knows them."""
         self.fill(entries)
         self.dev.copy_(self.host, non_blocking=True)
         self._copied.record()
+        if token_source is not None:
+            self.dev[self.offs[0]:self.offs[0] + len(entries)].copy_(token_source)
         self.graph.replay()
         return self.logits
 

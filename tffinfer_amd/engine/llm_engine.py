@@ -39,6 +39,18 @@ class EngineOptions:
     max_model_len: int | None = None
     memory_fraction: float = 0.85
     use_graphs: bool = True
+    #: launch a decode step before the host has read the tokens of the one before it
+    run_ahead: bool = True
+
+
+@dataclass
+class _Launched:
+    """A step whose kernels are queued and whose tokens the host has not read yet."""
+    plan: list
+    rows: list                      # the requests that sample, in the order of the logit rows
+    tokens: torch.Tensor | None     # int32 [rows] on the device
+    host: torch.Tensor | None       # the same in pinned host memory, valid after ``ready``
+    ready: torch.cuda.Event | None
 
 
 @dataclass
@@ -79,6 +91,8 @@ class LLMEngine:
         self._ids = itertools.count()
         self.keep_logits = False
         self._results: dict = {}
+        self._ahead: _Launched | None = None   # a decode step launched ahead of its predecessor's tokens
+        self.steps_ahead = 0                   # how many steps were launched that way
 
     @classmethod
     def from_model_dir(cls, model_dir: str, options: EngineOptions | None = None) -> "LLMEngine":
@@ -121,35 +135,108 @@ class LLMEngine:
 
     @property
     def has_work(self) -> bool:
-        return self.scheduler.has_work
+        return self.scheduler.has_work or self._ahead is not None
 
     # ---- one step --------------------------------------------------------
-    def step(self) -> list[tuple]:
-        """Plans and runs one step.  Returns (request id, new token, finished)
-        for every request that got a token."""
-        plan = self.scheduler.schedule()
-        if not plan:
-            return []
-        entries, sampling_rows = [], []
+    # Decoding one token per request leaves the device idle from the moment the host reads the
+    # sampled tokens until the next step's kernels are queued: a quarter of a millisecond of
+    # planning, table writing and graph launch per step.  While the batch only decodes, the
+    # next step is therefore launched *before* the tokens of the step in flight are read: its
+    # input tokens go from the sampler's output to the step's token table on the device, and
+    # everything else about it (positions, pages, random draws) the host knows beforehand.
+    # A request that turns out to have ended with the token just read (end of sequence) has
+    # one token computed in vain; it is dropped when that step completes.
+    def _launch(self, plan, token_source=None) -> _Launched:
+        entries, rows = [], []
         for p in plan:
-            toks = p.request.tokens[p.start:p.start + p.count]
+            if token_source is None:
+                toks = p.request.tokens[p.start:p.start + p.count]
+            else:
+                toks = [0]            # in token_source
             entries.append(StepEntry(p.request.id, toks, [p.count - 1] if p.samples else []))
             if p.samples:
-                sampling_rows.append(p.request)
-        logits = self.runner.step(entries)
+                rows.append(p.request)
+        logits = self.runner.step(entries, token_source)
+        if not rows:
+            return _Launched(plan, rows, None, None, None)
+        if self.keep_logits:
+            host = logits.float().cpu()
+            for r, req in enumerate(rows):
+                self._results.setdefault(req.id, []).append(host[r].clone())
+        ahead = 0 if token_source is None else 1      # outputs the host has not appended yet
+        tokens = self.sampler.sample_on_device(
+            logits, [r.sampling for r in rows], [len(r.output) + ahead for r in rows],
+            [r.tokens for r in rows])
+        host = torch.empty(len(rows), dtype=torch.int32, pin_memory=True)
+        host.copy_(tokens, non_blocking=True)
+        ready = torch.cuda.Event()
+        ready.record()
+        return _Launched(plan, rows, tokens, host, ready)
+
+    def _complete(self, st: _Launched) -> list[tuple]:
+        """Reads the step's tokens and tells the scheduler.  Requests that ended
+        or were taken away while the step ran are passed over."""
+        plan = [p for p in st.plan if p.request.status == "running"]
         sampled = {}
-        if sampling_rows:
-            if self.keep_logits:
-                host = logits.float().cpu()
-                for r, req in enumerate(sampling_rows):
-                    self._results.setdefault(req.id, []).append(host[r].clone())
-            toks = self.sampler.sample(
-                logits, [r.sampling for r in sampling_rows], [len(r.output) for r in sampling_rows],
-                [r.tokens for r in sampling_rows])
-            sampled = {req.id: t for req, t in zip(sampling_rows, toks)}
+        if st.rows:
+            st.ready.synchronize()
+            for req, t in zip(st.rows, st.host.tolist()):
+                if req.status == "running":
+                    sampled[req.id] = t
         finished = self.scheduler.update(plan, sampled)
         done = {r.id for r in finished}
         return [(rid, tok, rid in done) for rid, tok in sampled.items()]
+
+    def _plan_ahead(self, st: _Launched):
+        """The decode step after ``st``, planned without its tokens: every request
+        of ``st`` that its length does not end goes on.  None when the step after
+        needs the scheduler (admissions, prompts, pages running out, a penalty on
+        seen tokens)."""
+        if not self.options.run_ahead or self.keep_logits or not st.rows:
+            return None
+        sch = self.scheduler
+        if any(p.count != 1 or not p.samples for p in st.plan) or len(st.plan) != len(sch.running):
+            return None
+        if sch.waiting and len(sch.running) < sch.opt.max_num_seqs and self.runner.cache.slots.num_free > 0:
+            return None     # somebody may be admitted
+        plan = []
+        for p in st.plan:
+            req = p.request
+            if req.status != "running" or req.sampling.repetition_penalty != 1.0:
+                return None
+            n_out = len(req.output) + 1           # with the token in flight
+            if n_out >= req.max_new_tokens or len(req.prompt) + n_out >= sch.max_model_len:
+                continue                          # that token is its last
+            plan.append(type(p)(req, p.start + 1, 1, True))
+        if not plan:
+            return None
+        need = [0] * len(self.runner.cache.groups)
+        for p in plan:
+            for gi, k in enumerate(self.runner.cache.pages_needed(p.request.id, 1)):
+                need[gi] += k
+        if any(k > g.pool.num_free for k, g in zip(need, self.runner.cache.groups)):
+            return None
+        return plan
+
+    def step(self) -> list[tuple]:
+        """Plans and runs one step.  Returns (request id, new token, finished)
+        for every request that got a token."""
+        st = self._ahead
+        self._ahead = None
+        if st is None:
+            plan = self.scheduler.schedule()
+            if not plan:
+                return []
+            st = self._launch(plan)
+        nxt = self._plan_ahead(st)
+        if nxt is not None:
+            src = st.tokens
+            if len(nxt) != len(st.rows):          # some requests end with the token in flight
+                keep = [i for i, r in enumerate(st.rows) if any(p.request is r for p in nxt)]
+                src = st.tokens[torch.tensor(keep, device=st.tokens.device)]
+            self._ahead = self._launch(nxt, src)
+            self.steps_ahead += 1
+        return self._complete(st)
 
     # ---- whole generations ----------------------------------------------
     def generate(self, prompts, sampling=None, max_new_tokens: int = 64, eos_token_id: int | None = None,
@@ -164,7 +251,7 @@ class LLMEngine:
             rid = self.add_request(prompt, sc, max_new_tokens, eos_token_id, ignore_eos)
             reqs.append(self.scheduler.waiting[-1])
             assert reqs[-1].id == rid
-        while self.scheduler.has_work:
+        while self.has_work:
             self.step()
         return [GenerationResult(r.id, r.prompt, r.output, r.finish_reason, r.num_preemptions,
                                  self._results.pop(r.id, [])) for r in reqs]

@@ -131,25 +131,38 @@ class ModelRunner:
             self.cache.reserve(e.req, len(e.tokens))
 
     @torch.no_grad()
-    def step(self, entries: list[StepEntry]) -> torch.Tensor:
+    def step(self, entries: list[StepEntry], token_source: torch.Tensor | None = None) -> torch.Tensor:
         """Logits (float32 [wanted, vocab], on the device) at the wanted places,
-        in the order of the entries and of their ``want``."""
+        in the order of the entries and of their ``want``.
+
+        ``token_source`` (int32 [len(entries)], on the device) serves a step in
+        which every entry brings one token that the host does not know yet (it
+        was sampled by a step still running): entry i's token is
+        token_source[i], whatever ``entries[i].tokens`` holds in its place."""
         if not entries:
             return torch.empty(0, self.vocab_size, dtype=torch.float32, device=self.device)
         self._validate(entries)
+        if token_source is not None:
+            if any(len(e.tokens) != 1 for e in entries):
+                raise StepError("tokens can come from the device only in a step of one token per request")
+            if token_source.dtype != torch.int32 or tuple(token_source.shape) != (len(entries),) \
+                    or token_source.device != torch.device(self.device):
+                raise StepError("token_source must be int32 [entries] on the runner's device")
         self.reserve(entries)
         if self._graph_buckets and len(entries) <= self._graph_buckets[-1] \
                 and all(len(e.tokens) == 1 for e in entries):
-            return self._step_graph(entries)
+            return self._step_graph(entries, token_source)
         with torch.cuda.device(self.device):
             batch = build_step_batch(entries, self.cache, self.device)
+            if token_source is not None:
+                batch.token_ids[:len(entries)].copy_(token_source)
             ctx = StepContext(self.ops, self.act_dtype, batch, self.max_model_len, self._calls, self.cache)
             logits = self.model.forward(ctx)
         for e in entries:
             self.cache.commit(e.req, len(e.tokens))
         return logits
 
-    def _step_graph(self, entries) -> torch.Tensor:
+    def _step_graph(self, entries, token_source=None) -> torch.Tensor:
         """A decode-only step through the HIP graph of its batch size bucket.
         The logits live in a tensor the next such step overwrites."""
         R = len(entries)
@@ -159,7 +172,7 @@ class ModelRunner:
             if g is None:
                 g = self._graphs[bucket] = DecodeGraph(self, bucket)
                 g.capture()
-            logits = g.run(entries)
+            logits = g.run(entries, token_source)
             rows = [r for r, e in enumerate(entries) if e.want]
             if len(rows) == R:
                 out = logits[:R]

@@ -34,9 +34,15 @@ class Sampler:
         row r decides (the counter of its random draw); ``seen[r]`` the tokens
         of its prompt and output so far (needed only with a repetition penalty).
         ``logits`` may be changed in place by the penalty."""
-        R = logits.shape[0]
-        if R == 0:
+        if logits.shape[0] == 0:
             return []
+        return self.sample_on_device(logits, configs, indices, seen).tolist()
+
+    def sample_on_device(self, logits: torch.Tensor, configs: list[SamplingConfig], indices: list[int],
+                         seen: list | None = None) -> torch.Tensor:
+        """As ``sample``, but the tokens stay on the device (int32 [rows]) and
+        nothing waits for them: the caller reads them when it needs them."""
+        R = logits.shape[0]
         assert len(configs) == R and len(indices) == R
         if any(c.repetition_penalty != 1.0 for c in configs):
             flat, cu = [], [0]
@@ -50,7 +56,7 @@ class Sampler:
                 torch.tensor(cu, dtype=torch.int32, device=dev),
                 torch.tensor([c.repetition_penalty for c in configs], dtype=torch.float32, device=dev))
         if all(c.greedy for c in configs):
-            return self.ops.argmax(logits).tolist()
+            return self.ops.argmax(logits)
         eff = [c.effective() for c in configs]
         dev = self.device
         temperature = torch.tensor([e[0] for e in eff], dtype=torch.float32, device=dev)
@@ -59,4 +65,4 @@ class Sampler:
         min_p = torch.tensor([e[3] for e in eff], dtype=torch.float32, device=dev)
         u = torch.tensor([uniform_at(c.seed, i) for c, i in zip(configs, indices)],
                          dtype=torch.float32, device=dev)
-        return self.ops.sample(logits, temperature, u, top_k, top_p, min_p).tolist()
+        return self.ops.sample(logits, temperature, u, top_k, top_p, min_p)
