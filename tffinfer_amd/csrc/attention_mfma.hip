@@ -524,8 +524,8 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __r
 #define ATTN_STAGES 4
 constexpr int attn_vmcnt_imm(int v) { return (v & 15) | (7 << 4) | (15 << 8) | ((v >> 4) << 14); }
 
-template <int DT, int NQT, int NW>
-__global__ __launch_bounds__(64 * NW, (NW <= 4 ? 2 : 1)) void attn_mfma_block_kernel(
+template <int DT, int NQT, int NW, int KGRP>
+__global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn_mfma_block_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_tables, int bt_stride, const int32_t* __restrict__ cu_tokens,
@@ -535,12 +535,18 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 ? 2 : 1)) void attn_mfma_block_ke
     constexpr int D = DT * 16;
     constexpr int KS = (D + 31) / 32;
     constexpr int KFR = 2 * KS, VFR = DT, FR = KFR + VFR;   // 1 KB fragments per slice
-    constexpr int LPW = (FR + NW - 1) / NW;                  // copies a wave issues per slice
+    // KGRP groups of NW waves: group k works on the slices k, k + KGRP, ... of the same columns
+    // and the groups' results are merged at the end; a stage holds KGRP slices, one per group
+    constexpr int NWT = NW * KGRP, FRT = FR * KGRP;
+    constexpr int LPW = (FRT + NWT - 1) / NWT;               // copies a wave issues per stage
     constexpr int BCOLS = NW * NQT * 16;                     // columns of a block
-    constexpr int STAGES = ATTN_STAGES;                      // slices in LDS: one in use, the rest in flight
-    __shared__ __attribute__((aligned(1024))) bf16_t smem[STAGES * FR * 512];
+    constexpr int STAGES = ATTN_STAGES;                      // stages in LDS: one in use, the rest in flight
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[STAGES * FRT * 512];
     __shared__ int32_t pages[ATTN_BT_LDS];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    static_assert(KGRP == 1 || (size_t)STAGES * FRT * 1024 >= (size_t)NW * (DT * 1024 + 512),
+                  "the merge of the key groups borrows the stages");
+    const int tid = threadIdx.x, lane = tid & 63, wave_all = tid >> 6;
+    const int wave = wave_all % NW, kgi = wave_all / NW;     // column tile(s) and key group of this wave
     const int qc = lane & 15, kg = lane >> 4;
     const int g = blockIdx.y;
     const int G = nq / nkv;
@@ -586,7 +592,7 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 ? 2 : 1)) void attn_mfma_block_ke
     const int npg = page_index(kmax, page_size, page_shift) - pg0 + 1;
     const bool bt_in_lds = npg <= ATTN_BT_LDS;
     if (bt_in_lds)
-        for (int i = tid; i < npg; i += 64 * NW) pages[i] = bt[pg0 + i];
+        for (int i = tid; i < npg; i += 64 * NWT) pages[i] = bt[pg0 + i];
 
     bf16x8 qf[NQT][KS];
 #pragma unroll
@@ -619,10 +625,11 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 ? 2 : 1)) void attn_mfma_block_ke
     // wave and iteration, and one constant wait covers the slice about to be read.
 #define ATTN_ISSUE(step)                                                                            \
     {                                                                                               \
-        const int kb_ = kb0 + min((step), nsteps - 1) * 32;                                         \
         const int st_ = (step) % STAGES;                                                            \
         _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                           \
-            const int f = min(wave + NW * j, FR - 1);                                               \
+            const int F = min(wave_all + NWT * j, FRT - 1);                                         \
+            const int f = F % FR;                                                                   \
+            const int kb_ = kb0 + min((step) * KGRP + F / FR, nsteps - 1) * 32;                     \
             {                                                                                       \
                 const bf16_t* g_;                                                                   \
                 if (f < KFR) {                                                                      \
@@ -636,7 +643,7 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 ? 2 : 1)) void attn_mfma_block_ke
                     g_ = v_cache + (((size_t)ATTN_PAGE(j0) * nkv + g) * D + (f - KFR) * 16 + qc) * page_size + \
                          page_slot(j0, page_size, page_shift);                                      \
                 }                                                                                   \
-                __builtin_amdgcn_global_load_lds((glb_ptr_t)g_, (lds_ptr_t)(smem + (st_ * FR + f) * 512), 16, 0, 0); \
+                __builtin_amdgcn_global_load_lds((glb_ptr_t)g_, (lds_ptr_t)(smem + (st_ * FRT + F) * 512), 16, 0, 0); \
             }                                                                                       \
         }                                                                                           \
     }
@@ -662,12 +669,14 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 ? 2 : 1)) void attn_mfma_block_ke
 
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) ATTN_ISSUE(s)
-    for (int s = 0; s < nsteps; ++s) {
-        __builtin_amdgcn_s_waitcnt(attn_vmcnt_imm((STAGES - 2) * LPW));   // this wave's copies of slice s are in
-        __syncthreads();                            // ... and the other waves'; slice s - 1 is read
-        ATTN_ISSUE(s + STAGES - 1)                  // into the stage of slice s - 1
-        const int kb = kb0 + s * 32;
-        const bf16_t* st = smem + (s % STAGES) * FR * 512;
+    const int nsup = (nsteps + KGRP - 1) / KGRP;
+    for (int s = 0; s < nsup; ++s) {
+        __builtin_amdgcn_s_waitcnt(attn_vmcnt_imm((STAGES - 2) * LPW));   // this wave's copies of stage s are in
+        __syncthreads();                            // ... and the other waves'; stage s - 1 is read
+        ATTN_ISSUE(s + STAGES - 1)                  // into the stage of step s - 1
+        if (KGRP > 1 && s * KGRP + kgi >= nsteps) continue;   // past the last slice: nothing for this group
+        const int kb = kb0 + (s * KGRP + kgi) * 32;
+        const bf16_t* st = smem + ((s % STAGES) * FRT + kgi * FR) * 512;
         floatx4 sacc[NQT][2];
 #pragma unroll
         for (int t = 0; t < NQT; ++t) sacc[t][0] = sacc[t][1] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -732,6 +741,37 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 ? 2 : 1)) void attn_mfma_block_ke
 #undef ATTN_PAGE
     __builtin_amdgcn_s_waitcnt(vmcnt_imm0());   // the copies past the end must not outlive the block
 
+    if constexpr (KGRP > 1) {
+        // The second key group hands its maxima, sums and accumulators to the first through the
+        // stages (all copies have landed and all slices are read after the barrier).
+        static_assert(KGRP == 2 && NQT == 1, "the merge is written for two groups of single tiles");
+        float* mo = reinterpret_cast<float*>(smem) + wave * (DT * 256 + 128);
+        __syncthreads();
+        if (kgi == 1) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                *reinterpret_cast<float4*>(mo + dt * 256 + lane * 4) =
+                    make_float4(oacc[0][dt][0], oacc[0][dt][1], oacc[0][dt][2], oacc[0][dt][3]);
+            mo[DT * 256 + lane * 2] = m_run[0];
+            mo[DT * 256 + lane * 2 + 1] = l_run[0];
+        }
+        __syncthreads();
+        if (kgi == 1) continue;   // the next item, if any
+        const float m2 = mo[DT * 256 + lane * 2], l2 = mo[DT * 256 + lane * 2 + 1];
+        const float m = fmaxf(m_run[0], m2);
+        const float a1 = m_run[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m_run[0] - m) * sl2);
+        const float a2 = m2 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m2 - m) * sl2);
+        l_run[0] = l_run[0] * a1 + l2 * a2;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const float4 o2 = *reinterpret_cast<const float4*>(mo + dt * 256 + lane * 4);
+            oacc[0][dt][0] = oacc[0][dt][0] * a1 + o2.x * a2;
+            oacc[0][dt][1] = oacc[0][dt][1] * a1 + o2.y * a2;
+            oacc[0][dt][2] = oacc[0][dt][2] * a1 + o2.z * a2;
+            oacc[0][dt][3] = oacc[0][dt][3] * a1 + o2.w * a2;
+        }
+    }
+
 #pragma unroll
     for (int t = 0; t < NQT; ++t) {
         float l = l_run[t];
@@ -763,9 +803,15 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
     if ((page_size & (page_size - 1)) == 0)
         for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
     if (cols_per_wave == 128) {   // blocks of eight waves that share their keys through LDS
-        attn_mfma_block_kernel<DT, 1, 8><<<dim3(num_blocks, nkv), 512, 0, s>>>(
-            q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
-            block_items, nq, nkv, page_size, page_shift, window, scale);
+        // two groups of eight waves that take every other slice, where LDS holds their stages
+        if constexpr (DT <= 8)
+            attn_mfma_block_kernel<DT, 1, 8, 2><<<dim3(num_blocks, nkv), 1024, 0, s>>>(
+                q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
+                block_items, nq, nkv, page_size, page_shift, window, scale);
+        else
+            attn_mfma_block_kernel<DT, 1, 8, 1><<<dim3(num_blocks, nkv), 512, 0, s>>>(
+                q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
+                block_items, nq, nkv, page_size, page_shift, window, scale);
         return tff_check_launch("attention_mfma_block");
     }
     const dim3 grid(num_work, nkv, splits);
