@@ -371,6 +371,137 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_reg_kernel(
     }
 }
 
+// bfloat16, head sizes 16 .. 256 that are powers of two, the whole head rotated (or none of it):
+// a lane has 8 consecutive elements of a head (one 16-byte access), LPH = d / 8 lanes a head,
+// 64 / LPH heads a wave.  The sum of squares goes over the head's lanes by shuffles; with pairs
+// (i, i + d/2) a lane's partner is LPH / 2 lanes away, with pairs (2i, 2i+1) it is the lane itself.
+template <int LPH>
+__global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(
+    bf16_t* __restrict__ qkv, int nq, int nkv, const float* __restrict__ qw,
+    const float* __restrict__ kw, float eps, const float* __restrict__ cos_sin, int pairing,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ slot_mapping,
+    bf16_t* __restrict__ k_cache, int page_size) {
+    constexpr int D = LPH * 8, HPW = 64 / LPH;
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l = lane % LPH;
+    const int hh = (blockIdx.y * 4 + wave) * HPW + lane / LPH;
+    const bool valid = hh < nq + nkv;
+    const int h = valid ? hh : 0;
+    const bool is_k = h >= nq;
+    bf16_t* x = qkv + (size_t)t * (nq + 2 * nkv) * D + (size_t)h * D + l * 8;
+    union { uint4 u; bf16_t e[8]; } in, outv;
+    in.u = *reinterpret_cast<const uint4*>(x);
+    float v[8];
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        v[e] = (float)in.e[e];
+        ss = fmaf(v[e], v[e], ss);
+    }
+#pragma unroll
+    for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    const float* w = is_k ? kw : qw;
+    if (w) {
+        const float rr = rsqrtf(ss / (float)D + eps);
+        const float4 w0 = *reinterpret_cast<const float4*>(w + l * 8);
+        const float4 w1 = *reinterpret_cast<const float4*>(w + l * 8 + 4);
+        v[0] = v[0] * rr * w0.x; v[1] = v[1] * rr * w0.y; v[2] = v[2] * rr * w0.z; v[3] = v[3] * rr * w0.w;
+        v[4] = v[4] * rr * w1.x; v[5] = v[5] * rr * w1.y; v[6] = v[6] * rr * w1.z; v[7] = v[7] * rr * w1.w;
+    }
+    if (cos_sin) {
+        const float* cs = cos_sin + (size_t)positions[t] * D;   // [pos][pair][cos, sin]
+        if (pairing == 0) {
+            constexpr int HL = LPH / 2;
+            const float4* c4 = reinterpret_cast<const float4*>(cs + (l % HL) * 16);
+            const float4 q0 = c4[0], q1 = c4[1], q2 = c4[2], q3 = c4[3];
+            const float c[8] = {q0.x, q0.z, q1.x, q1.z, q2.x, q2.z, q3.x, q3.z};
+            const float sn[8] = {q0.y, q0.w, q1.y, q1.w, q2.y, q2.w, q3.y, q3.w};
+            const bool first = l < HL;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float pv = __shfl_xor(v[e], HL, 64);
+                // first half: a = v, b = pv -> a c - b s;  second half: a = pv, b = v -> a s + b c
+                v[e] = first ? v[e] * c[e] - pv * sn[e] : pv * sn[e] + v[e] * c[e];
+            }
+        } else {
+            const float4* c4 = reinterpret_cast<const float4*>(cs + l * 8);
+            const float4 q0 = c4[0], q1 = c4[1];
+            const float c[4] = {q0.x, q0.z, q1.x, q1.z};
+            const float sn[4] = {q0.y, q0.w, q1.y, q1.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float a = v[2 * i], b = v[2 * i + 1];
+                v[2 * i] = a * c[i] - b * sn[i];
+                v[2 * i + 1] = a * sn[i] + b * c[i];
+            }
+        }
+    }
+    if (!valid) return;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) outv.e[e] = (bf16_t)v[e];
+    if (!is_k) {
+        *reinterpret_cast<uint4*>(x) = outv.u;
+    } else {
+        const int slot = slot_mapping[t];
+        if (slot < 0) return;
+        const int page = slot / page_size, off = slot % page_size;
+        bf16_t* kdst = k_cache + (((size_t)page * nkv + (h - nq)) * page_size + off) * D + l * 8;
+        *reinterpret_cast<uint4*>(kdst) = outv.u;
+    }
+}
+
+// The values of 8 consecutive tokens and one kv head go to their (transposed) pages: where the 8
+// slots are consecutive and start at a multiple of 8 in a page, a thread writes one element's 8
+// tokens as one 16-byte run; else token by token.
+__global__ __launch_bounds__(128) void v_page_write_kernel(
+    const bf16_t* __restrict__ qkv, int T, int nq, int nkv, int d,
+    const int32_t* __restrict__ slot_mapping, bf16_t* __restrict__ v_cache, int page_size) {
+    __shared__ __attribute__((aligned(16))) bf16_t tile[8][QK_MAX_D];
+    __shared__ int32_t slots[8];
+    const int t0 = blockIdx.x * 8, head = blockIdx.y, tid = threadIdx.x;
+    const int width = (nq + 2 * nkv) * d;
+    const int cpr = d / 8;   // 16-byte chunks per row
+    if (tid < 8) slots[tid] = t0 + tid < T ? slot_mapping[t0 + tid] : -1;
+    for (int i = tid; i < 8 * cpr; i += 128) {
+        const int tk = i / cpr, c = i % cpr;
+        uint4 val = make_uint4(0, 0, 0, 0);
+        if (t0 + tk < T)
+            val = *reinterpret_cast<const uint4*>(qkv + (size_t)(t0 + tk) * width + (size_t)(nq + nkv + head) * d + c * 8);
+        *reinterpret_cast<uint4*>(&tile[tk][c * 8]) = val;
+    }
+    __syncthreads();
+    const int s0 = slots[0];
+    bool run = s0 >= 0 && (s0 & 7) == 0 && (s0 % page_size) + 8 <= page_size;
+#pragma unroll
+    for (int i = 1; i < 8; ++i) run = run && slots[i] == s0 + i;
+    if (run) {
+        bf16_t* vt = v_cache + ((size_t)(s0 / page_size) * nkv + head) * d * page_size + (s0 % page_size);
+        for (int e = tid; e < d; e += 128) {
+            union { uint4 u; bf16_t h[8]; } pk;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pk.h[i] = tile[i][e];
+            *reinterpret_cast<uint4*>(vt + (size_t)e * page_size) = pk.u;
+        }
+    } else {
+        for (int i = 0; i < 8; ++i) {
+            const int slot = slots[i];
+            if (slot < 0) continue;
+            bf16_t* vt = v_cache + ((size_t)(slot / page_size) * nkv + head) * d * page_size + (slot % page_size);
+            for (int e = tid; e < d; e += 128) vt[(size_t)e * page_size] = tile[i][e];
+        }
+    }
+}
+
+template <int LPH>
+static void launch_qk_vec(bf16_t* qkv, int T, int nq, int nkv, const float* qw, const float* kw, float eps,
+                          const float* cos_sin, int pairing, const int32_t* positions,
+                          const int32_t* slot_mapping, bf16_t* k_cache, int page_size, hipStream_t s) {
+    constexpr int HPB = 4 * (64 / LPH);
+    qk_norm_rope_vec_kernel<LPH><<<dim3(T, (nq + nkv + HPB - 1) / HPB), 256, 0, s>>>(
+        qkv, nq, nkv, qw, kw, eps, cos_sin, pairing, positions, slot_mapping, k_cache, page_size);
+}
+
 TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d, const float* q_weight,
                                 const float* k_weight, float eps, const float* cos_sin,
                                 int rot_dim, int pairing, int max_pos, const int32_t* positions,
@@ -398,6 +529,28 @@ TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d, const 
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     TFF_REQUIRE(dtype == TFF_F32 || dtype == TFF_BF16, "qk_norm_rope_kv: unknown dtype %d", dtype);
+    const bool pow2 = d >= 16 && d <= 256 && (d & (d - 1)) == 0;
+    // for prompt portions: two kernels with 16-byte accesses; a few tokens are done by one launch
+    if (T >= 32 && dtype == TFF_BF16 && pow2 && (!cos_sin || rot_dim == d) && ((uintptr_t)qkv % 16) == 0 &&
+        ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 16) == 0 &&
+        (!q_weight || (((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0)) &&
+        (!cos_sin || ((uintptr_t)cos_sin % 16) == 0)) {
+#define TFF_QK_VEC(L)                                                                               \
+    launch_qk_vec<L>((bf16_t*)qkv, T, nq, nkv, q_weight, k_weight, eps, cos_sin, pairing, positions, \
+                     slot_mapping, (bf16_t*)k_cache, page_size, s)
+        switch (d) {
+            case 16: TFF_QK_VEC(2); break;
+            case 32: TFF_QK_VEC(4); break;
+            case 64: TFF_QK_VEC(8); break;
+            case 128: TFF_QK_VEC(16); break;
+            default: TFF_QK_VEC(32); break;
+        }
+#undef TFF_QK_VEC
+        if (int rc = tff_check_launch("qk_norm_rope")) return rc;
+        v_page_write_kernel<<<dim3((T + 7) / 8, nkv), 128, 0, s>>>((const bf16_t*)qkv, T, nq, nkv, d, slot_mapping,
+                                                                 (bf16_t*)v_cache, page_size);
+        return tff_check_launch("v_page_write");
+    }
     if (!cos_sin || rot_dim == d) {
         dim3 grid4(T, (nq + 2 * nkv + 3) / 4);
         if (dtype == TFF_F32)
