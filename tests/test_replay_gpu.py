@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import replay_lib as rl
-from helpers import PAGE_SIZE, TOL, random_tokens, read_config
+from helpers import PAGE_SIZE, TOL, random_tokens, read_config, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -147,3 +147,46 @@ def test_midsize_model_long_prompt(tmp_path_factory, dtype):
         results = rl.run_steps_in_process(runner, steps)
         worst = rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
         print(f"mid {dtype}: worst rel. error {worst:.3e}")
+
+
+LARGE_SHAPES = {
+    # the layer sizes of larger members of the family, one layer each
+    "14b": dict(hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, head_dim=128, intermediate_size=17408),
+    "32b": dict(hidden_size=5120, num_attention_heads=64, num_key_value_heads=8, head_dim=128, intermediate_size=25600),
+}
+
+
+@pytest.mark.parametrize("shape", ["14b", "32b"])
+def test_bfloat16_against_float32_at_large_layer_sizes(shape):
+    """One layer with the widths of the 14B and 32B models (inner sizes that are no power of
+    two, 5 and 8 query heads to a key head): the bfloat16 kernels against the engine's own
+    float32 path (which the small configurations pin to the plain implementation), for a
+    prompt in portions beside another request, then steps of two decoding requests."""
+    from tffinfer_amd.engine.batch import StepEntry
+    from tffinfer_amd.engine.runner import ModelRunner
+    from tffinfer_amd.models import build_model_skeleton, config_from_dict
+    cfg = dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=1, vocab_size=5003,
+               max_position_embeddings=2048, rms_norm_eps=1e-6, rope_theta=1000000.0,
+               tie_word_embeddings=False, **LARGE_SHAPES[shape])
+    V = cfg["vocab_size"]
+    a, b = random_tokens(712, V, 5), random_tokens(47, V, 6)
+    steps = [[("a", a[:512], [0, 100, 511])], [("a", a[512:700], [187]), ("b", b[:40], [39])]]
+    steps += [[("a", [a[700 + i]], [0]), ("b", [b[40 + i]], [0])] for i in range(7)]
+    steps += [[("a", a[707:712], [0, 4])]]
+    out = {}
+    for dtype in (torch.float32, torch.bfloat16):
+        model = build_model_skeleton(config_from_dict(cfg))
+        model.init_random(11, dtype, "cuda:0", on_device=True)
+        runner = ModelRunner(model, page_size=16, num_pages=64, max_seqs=2)
+        runner.add_request("a")
+        runner.add_request("b")
+        rows = []
+        for st in steps:
+            rows.append(runner.step([StepEntry(r, list(t), list(w)) for r, t, w in st]).float().cpu())
+        out[dtype] = torch.cat(rows)
+        del runner, model
+        torch.cuda.empty_cache()
+    assert out[torch.float32].shape[0] == 3 + 2 + 14 + 2
+    worst = rel_err(out[torch.bfloat16], out[torch.float32])
+    print(f"{shape}: bfloat16 against float32, worst rel. error {worst:.3e}")
+    assert worst <= TOL["bfloat16"]
