@@ -499,6 +499,28 @@ def test_attention_mfma_decode_split_keys(nq, nkv, d, ps, window, splits):
     _close(out.reshape(T, nq, d), ref, 1.5e-2, "split-key decode attention")
 
 
+@pytest.mark.parametrize("nq,nkv,d,ps,window", [(32, 8, 128, 16, 0), (8, 2, 32, 8, 300), (40, 2, 96, 8, 0)])
+def test_attention_mfma_portions_beside_decoding_requests(nq, nkv, d, ps, window):
+    """A step of long portions and of requests that bring one token with a long context: the
+    latter go to the split-key kernel, the former to the block kernel, into the same output."""
+    ops = _ops()
+    entries = [(900, 1), (0, 300), (40, 1), (333, 150), (1500, 1), (7, 1)]
+    batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=nq + d)
+    T = batch.num_tokens
+    g = torch.Generator().manual_seed(8)
+    q = torch.randn(T, nq, d, generator=g).to(torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale)
+    gen = ops.attention_generic(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv.k_cache, kv.v_cache, kv.block_tables,
+                                batch.token_req, batch.positions, window, scale)
+    _close(out, gen.double(), 1.5e-2, "mixed step against the general kernel")
+    cu = batch.host_cu_tokens
+    for r, (P, n) in enumerate(entries):
+        mine = torch.tensor([cu[r], cu[r + 1] - 1])
+        ref = _attn_ref(q[mine], ks[r], vs[r], positions[mine], window, scale)
+        _close(out.reshape(T, nq, d)[mine], ref, 1.5e-2, f"request {r}")
+
+
 @pytest.mark.parametrize("splits", [1, 2, 5])
 def test_attention_mfma_decode_more_pages_than_the_wave_keeps(splits):
     """A wave keeps 1024 page numbers at hand; with more pages in its run of keys it reads

@@ -41,7 +41,7 @@ __device__ __forceinline__ int page_slot(int j, int page_size, int page_shift) {
     return page_shift >= 0 ? (j & (page_size - 1)) : j % page_size;
 }
 
-template <int DT, int NQT, bool SPLIT>
+template <int DT, int NQT>
 __global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const bf16_t* __restrict__ k_cache,
@@ -89,12 +89,7 @@ __global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
     const int kmax = P + tl_last;
     const int kb0 = (kmin / 32) * 32;
     const int nsteps = (kmax - kb0) / 32 + 1;
-    int s_begin = 0, s_end = nsteps;
-    if (SPLIT) {
-        const int per = (nsteps + (int)gridDim.z - 1) / (int)gridDim.z;
-        s_begin = (int)blockIdx.z * per;
-        s_end = min(nsteps, s_begin + per);
-    }
+    const int s_begin = 0, s_end = nsteps;
 
     // Q as second operand: lane (col, g) holds elements ks*32 + g*8 .. +8 of its column
     bf16x8 qf[NQT][KS];
@@ -246,18 +241,7 @@ __global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
         l += __shfl_xor(l, 16, 64);
         l += __shfl_xor(l, 32, 64);
         if (!c_ok[t]) continue;
-        if (SPLIT) {
-            const size_t row = ((size_t)blockIdx.z * T_total + c_tok[t]) * nq + c_head[t];
-            float* po = part_o + row * D;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-                *reinterpret_cast<float4*>(po + dt * 16 + kg * 4) =
-                    make_float4(oacc[t][dt][0], oacc[t][dt][1], oacc[t][dt][2], oacc[t][dt][3]);
-            if (kg == 0) {
-                part_ml[row * 2] = m_run[t];
-                part_ml[row * 2 + 1] = l;
-            }
-        } else {
+        {
             const float inv = 1.0f / l;
             bf16_t* op = out + ((size_t)c_tok[t] * nq + c_head[t]) * D;
 #pragma unroll
@@ -455,7 +439,8 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
     l += __shfl_xor(l, 32, 64);
     if (!c_ok) return;
     if (SPLIT) {
-        const size_t row = ((size_t)blockIdx.z * T_total + c_tok) * nq + c_head;
+        // keys are split for entries of one token only: partial results are kept by entry
+        const size_t row = ((size_t)blockIdx.z * T_total + r) * nq + c_head;
         float* po = part_o + row * D;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -483,13 +468,17 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
 __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __restrict__ part_o,
                                                                  const float* __restrict__ part_ml,
                                                                  bf16_t* __restrict__ out, int splits,
-                                                                 int T_total, int nq, int d) {
+                                                                 int R_total, int nq, int d,
+                                                                 const int32_t* __restrict__ rows) {
     __shared__ float w[256];
     __shared__ float red[17];
-    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    // rows: (entry, token) pairs; without them entry i is token i
+    const int r = rows ? rows[2 * blockIdx.x] : (int)blockIdx.x;
+    const int t = rows ? rows[2 * blockIdx.x + 1] : (int)blockIdx.x;
+    const int h = blockIdx.y, tid = threadIdx.x;
     float ms = -INFINITY, ls = 0.f;
     if (tid < splits) {
-        const float* ml = part_ml + (((size_t)tid * T_total + t) * nq + h) * 2;
+        const float* ml = part_ml + (((size_t)tid * R_total + r) * nq + h) * 2;
         ms = ml[0];
         ls = ml[1];
     }
@@ -502,7 +491,7 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __r
         float acc = 0.f;
 #pragma unroll 8
         for (int s = 0; s < splits; ++s)
-            acc = fmaf(part_o[(((size_t)s * T_total + t) * nq + h) * d + e], w[s], acc);
+            acc = fmaf(part_o[(((size_t)s * R_total + r) * nq + h) * d + e], w[s], acc);
         out[((size_t)t * nq + h) * d + e] = (bf16_t)(acc * inv);
     }
 }
@@ -819,15 +808,12 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
     q, q_stride, out, part_o, part_ml, k_cache, v_cache, block_tables, bt_stride, cu_tokens,       \
         start_pos, work, tiles_per_entry, nq, nkv, page_size, page_shift, window, scale, T_total
     if (splits > 1) {
-        if (cols_per_wave == 16)
-            attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
-        else
-            attn_mfma_kernel<DT, 2, true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
+        attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
     } else {
         if (cols_per_wave == 16)
             attn_wave_kernel<DT, false, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
         else
-            attn_mfma_kernel<DT, 2, false><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
+            attn_mfma_kernel<DT, 2><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
     }
 #undef TFF_ATTN_ARGS
     return tff_check_launch("attention_mfma");
@@ -872,6 +858,8 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
     }
     TFF_REQUIRE(splits >= 1 && splits <= 65535 && nkv <= 65535, "attention_mfma: bad split count %d", splits);
     TFF_REQUIRE(splits == 1 || (part_o && part_ml), "attention_mfma: split keys need a workspace");
+    TFF_REQUIRE(splits == 1 || cols_per_wave == 16,
+                "attention_mfma: keys are split for entries of one token (16 columns a wave) only");
     TFF_REQUIRE(work || tiles_per_entry >= 1, "attention_mfma: neither a work table nor a tile count");
     TFF_REQUIRE(bt_stride > 0 && num_pages > 0 && window >= 0 && T_total >= 0, "attention_mfma: bad geometry");
     if (num_work <= 0) return 0;
@@ -893,13 +881,16 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
 }
 
 TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml, void* out,
-                                       int splits, int T_total, int nq, int d, tff_stream_t stream) {
+                                       int splits, int R_total, int nq, int d, const int32_t* rows,
+                                       int num_rows, tff_stream_t stream) {
     TFF_REQUIRE(part_o && part_ml && out, "attention_split_reduce: null pointer");
-    TFF_REQUIRE(splits >= 1 && T_total >= 0 && nq > 0 && nq <= 65535 && d > 0,
+    TFF_REQUIRE(splits >= 1 && R_total >= 0 && nq > 0 && nq <= 65535 && d > 0,
                 "attention_split_reduce: bad sizes");
-    if (T_total == 0) return 0;
+    const int n = rows ? num_rows : R_total;
+    TFF_REQUIRE(n >= 0 && n <= R_total, "attention_split_reduce: %d rows of %d entries", n, R_total);
+    if (n == 0) return 0;
     TFF_REQUIRE(splits <= 256, "attention_split_reduce: at most 256 splits, got %d", splits);
-    attn_split_reduce_kernel<<<dim3(T_total, nq), 256, 0, (hipStream_t)stream>>>(
-        part_o, part_ml, (bf16_t*)out, splits, T_total, nq, d);
+    attn_split_reduce_kernel<<<dim3(n, nq), 256, 0, (hipStream_t)stream>>>(
+        part_o, part_ml, (bf16_t*)out, splits, R_total, nq, d, rows);
     return tff_check_launch("attention_split_reduce");
 }

@@ -91,9 +91,10 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out,
 // or 32) columns of one request and kv head; a column is a (token, q head of
 // the group) pair numbered token * G + head.  work != null: pairs (request,
 // first column) per wave; work == null: every request brings one token and
-// gets tiles_per_entry waves.  splits > 1 cuts each request's keys into runs
-// whose partial results (part_o [splits, T, nq, d], part_ml [splits, T, nq, 2],
-// float32) tff_attention_split_reduce merges.  cols_per_wave 128: work items
+// gets tiles_per_entry waves.  splits > 1 (entries of one token, 16 columns a
+// wave) cuts each request's keys into runs whose partial results (part_o
+// [splits, R, nq, d], part_ml [splits, R, nq, 2], float32, R = T_total the
+// number of entries) tff_attention_split_reduce merges.  cols_per_wave 128: work items
 // are runs of 128 columns for a block of eight waves that stages keys and
 // values in LDS; block b works through items block_items[b] ..
 // block_items[b + 1] of the work table (block_items null: item b).  Head sizes 16..128 in steps of
@@ -107,8 +108,11 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                int tiles_per_entry, int cols_per_wave, int splits, int T_total,
                                int nq, int nkv, int d, int page_size, int num_pages, int window,
                                float scale, tff_stream_t stream);
+// Merges partial results kept by entry (part_o [splits, R_total, nq, d]) into out rows:
+// rows (may be null: entry i is token i for all R_total) holds (entry, token) pairs.
 TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml, void* out,
-                                       int splits, int T_total, int nq, int d, tff_stream_t stream);
+                                       int splits, int R_total, int nq, int d, const int32_t* rows,
+                                       int num_rows, tff_stream_t stream);
 
 // out[t, i] = silu(gu[t, i]) * gu[t, I + i]
 TFF_API int tff_swiglu(const void* gu, void* out, int T, int I, int dtype, tff_stream_t stream);

@@ -326,17 +326,27 @@ def mfma_attention_supported(dtype: torch.dtype, d: int, page_size: int) -> bool
     return dtype == torch.bfloat16 and bool(_lib.load().tff_attention_mfma_supported(int(d), int(page_size)))
 
 
-def _attention_work(batch, G: int, cols: int, device) -> torch.Tensor:
+def _entries(batch, which: str) -> list[int]:
+    """Rows of the step's entries: all, those that bring one token, or the others."""
+    cu = batch.host_cu_tokens
+    rows = range(len(cu) - 1)
+    if which == "all":
+        return list(rows)
+    one = which == "single"
+    return [r for r in rows if (cu[r + 1] - cu[r] == 1) == one]
+
+
+def _attention_work(batch, G: int, cols: int, device, which: str = "all") -> torch.Tensor:
     """(entry, first column) of every wave's tile for the step's entries; a
     column is a (token, q head of the group) pair numbered token * G + head."""
     cache = getattr(batch, "_attn_work", None)
     if cache is None:
         cache = batch._attn_work = {}
-    key = (G, cols)
+    key = (G, cols, which)
     if key not in cache:
         cu = batch.host_cu_tokens
         flat = []
-        for r in range(len(cu) - 1):
+        for r in _entries(batch, which):
             for c0 in range(0, (cu[r + 1] - cu[r]) * G, cols):
                 flat.extend((r, c0))
         cache[key] = torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(device)
@@ -354,7 +364,7 @@ def _num_cus(device) -> int:
 
 
 def _attention_block_work(batch, G: int, nkv: int, window: int, device, cols: int = 128,
-                          bins: int | None = None):
+                          bins: int | None = None, which: str = "all"):
     """Work table of the block kernel: items (entry, first column) of ``cols``
     columns, dealt to blocks so that every block goes through about the same
     number of 32-key slices (an item late in a long prompt sees many times the
@@ -366,11 +376,11 @@ def _attention_block_work(batch, G: int, nkv: int, window: int, device, cols: in
         cache = batch._attn_work = {}
     if bins is None:
         bins = max(1, _num_cus(device) // max(1, nkv))
-    key = ("blocks", G, nkv, cols, window, bins)
+    key = ("blocks", G, nkv, cols, window, bins, which)
     if key not in cache:
         cu, P = batch.host_cu_tokens, batch.host_start_pos
         items = []                       # (slices, entry, first column)
-        for r in range(len(cu) - 1):
+        for r in _entries(batch, which):
             ncols = (cu[r + 1] - cu[r]) * G
             for c0 in range(0, ncols, cols):
                 first = P[r] + c0 // G
@@ -435,36 +445,55 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
         scale = 1.0 / math.sqrt(d)
     out = torch.empty(T, nq * d, dtype=q.dtype, device=q.device)
     L = _lib.load()
-    part_o = part_ml = block_items = None
-    num_blocks = 0
-    if batch.max_new_tokens == 1:
-        tiles = -(-G // 16)
-        work, num_work, cols = None, R * tiles, 16
-        if splits is None:
-            splits = getattr(batch, "attn_splits", None) or pick_splits(num_work * nkv, batch.max_context)
+    stream = _stream()
+
+    def launch(work, num_work, block_items, num_blocks, tiles, cols, splits, rows=None):
+        # partial results of split keys are kept by entry (split entries bring one token each)
+        part_o = part_ml = None
         if splits > 1:
-            part_o = torch.empty(splits, T, nq, d, dtype=torch.float32, device=q.device)
-            part_ml = torch.empty(splits, T, nq, 2, dtype=torch.float32, device=q.device)
+            part_o = torch.empty(splits, R, nq, d, dtype=torch.float32, device=q.device)
+            part_ml = torch.empty(splits, R, nq, 2, dtype=torch.float32, device=q.device)
+        _lib.check(L.tff_attention_mfma(
+            q.data_ptr(), q.stride(0), out.data_ptr(), _ptr(part_o), _ptr(part_ml), k_cache.data_ptr(),
+            v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(),
+            batch.start_pos.data_ptr(), _ptr(work), num_work, _ptr(block_items), num_blocks, tiles, cols,
+            splits, R if splits > 1 else T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window),
+            float(scale), stream))
+        if splits > 1:
+            _lib.check(L.tff_attention_split_reduce(
+                part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), splits, R, nq, d, _ptr(rows),
+                0 if rows is None else rows.shape[0], stream))
+
+    if batch.max_new_tokens == 1:
+        # decoding only: a wave per request, kv head and run of keys; sizes come from the tables
+        tiles = -(-G // 16)
+        if splits is None:
+            splits = getattr(batch, "attn_splits", None) or pick_splits(R * tiles * nkv, batch.max_context)
+        launch(None, R * tiles, None, 0, tiles, 16, splits)
+        return out
+    # long portions: blocks that share their keys through LDS (128 columns); short ones: a wave
+    # of its own per 32 or 16 columns
+    cols = 128 if batch.max_new_tokens * G > 64 else (32 if batch.max_new_tokens * G > 16 else 16)
+    which = "all"
+    single = _entries(batch, "single")
+    if cols == 128 and single and batch.max_context >= 256:
+        # Requests that decode beside the portions have one token each and possibly long
+        # contexts: they get the split-key kernel of their own rather than one block each.
+        which = "multi"
+        work = _attention_work(batch, G, 16, q.device, "single")
+        cache = batch._attn_work
+        if "single_rows" not in cache:
+            cu = batch.host_cu_tokens
+            cache["single_rows"] = torch.tensor([(r, cu[r]) for r in single], dtype=torch.int32).to(q.device)
+        sp = splits if splits is not None else pick_splits(work.shape[0] * nkv, batch.max_context)
+        launch(work, work.shape[0], None, 0, 1, 16, sp, cache["single_rows"])
+    if cols == 128:
+        work, block_items, num_blocks = _attention_block_work(batch, G, nkv, int(window), q.device,
+                                                              bins=block_bins, which=which)
+        launch(work, work.shape[0], block_items, num_blocks, 1, 128, 1)
     else:
-        tiles, splits = 1, 1
-        # long portions: blocks of four waves that share their keys through LDS (128 columns);
-        # short ones: a wave of its own per 32 or 16 columns
-        cols = 128 if batch.max_new_tokens * G > 64 else (32 if batch.max_new_tokens * G > 16 else 16)
-        if cols == 128:
-            work, block_items, num_blocks = _attention_block_work(batch, G, nkv, int(window), q.device,
-                                                                  bins=block_bins)
-        else:
-            work = _attention_work(batch, G, cols, q.device)
-        num_work = work.shape[0]
-    dest = out
-    _lib.check(L.tff_attention_mfma(
-        q.data_ptr(), q.stride(0), dest.data_ptr(), _ptr(part_o), _ptr(part_ml), k_cache.data_ptr(),
-        v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(),
-        batch.start_pos.data_ptr(), _ptr(work), num_work, _ptr(block_items), num_blocks, tiles, cols, splits, T, nq, nkv, d,
-        k_cache.shape[2], k_cache.shape[0], int(window), float(scale), _stream()))
-    if splits > 1:
-        _lib.check(L.tff_attention_split_reduce(part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(),
-                                                splits, T, nq, d, _stream()))
+        work = _attention_work(batch, G, cols, q.device)
+        launch(work, work.shape[0], None, 0, 1, cols, 1)
     return out
 
 
