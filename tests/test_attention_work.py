@@ -1,0 +1,51 @@
+"""The host side of the block attention kernel: work items dealt to blocks."""
+from types import SimpleNamespace
+
+import pytest
+
+
+def _batch(entries):
+    cu = [0]
+    for _, n in entries:
+        cu.append(cu[-1] + n)
+    return SimpleNamespace(host_cu_tokens=cu, host_start_pos=[p for p, _ in entries])
+
+
+def _slices(P, n, G, c0, cols, window):
+    ncols = n * G
+    first, last = P + c0 // G, P + (min(c0 + cols, ncols) - 1) // G
+    lo = max(0, first - window + 1) if window > 0 else 0
+    return last // 32 - lo // 32 + 1
+
+
+@pytest.mark.parametrize("window", [0, 300])
+@pytest.mark.parametrize("bins", [1, 3, 32, 500])
+def test_every_item_once_and_even_loads(bins, window):
+    from tffinfer_amd.kernels.ops import _attention_block_work
+    entries = [(0, 2048), (333, 200), (5, 1), (1000, 130), (0, 37)]
+    G, cols = 4, 128
+    batch = _batch(entries)
+    items, starts, blocks = _attention_block_work(batch, G, 8, window, "cpu", cols, bins=bins)
+    items, starts = items.tolist(), starts.tolist()
+    want = sorted((r, c0) for r, (P, n) in enumerate(entries) for c0 in range(0, n * G, cols))
+    assert sorted(map(tuple, items)) == want                      # no item lost, none twice
+    assert blocks == len(starts) - 1 == min(bins, len(want))
+    assert starts[0] == 0 and starts[-1] == len(items) and all(a < b for a, b in zip(starts, starts[1:]))
+    loads = []
+    for b in range(blocks):
+        loads.append(sum(_slices(*entries[r], G, c0, cols, window) for r, c0 in items[starts[b]:starts[b + 1]]))
+    biggest = max(_slices(*entries[r], G, c0, cols, window) for r, c0 in want)
+    # longest-first dealing: no block carries more than the mean plus one item
+    assert max(loads) <= sum(loads) / blocks + biggest
+    if blocks == len(want):
+        assert loads == sorted(loads, reverse=True)              # one item each, the longest first
+
+
+def test_entry_filters():
+    from tffinfer_amd.kernels.ops import _attention_block_work, _attention_work, _entries
+    batch = _batch([(900, 1), (0, 300), (40, 1), (333, 150)])
+    assert _entries(batch, "single") == [0, 2] and _entries(batch, "multi") == [1, 3]
+    items, starts, blocks = _attention_block_work(batch, 4, 2, 0, "cpu", 128, bins=64, which="multi")
+    assert {r for r, _ in items.tolist()} == {1, 3}
+    single = _attention_work(batch, 20, 16, "cpu", "single").tolist()     # 20 heads to a kv head: two tiles
+    assert single == [[0, 0], [0, 16], [2, 0], [2, 16]]
