@@ -42,6 +42,8 @@ def parse_args():
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="measure one phase only (for profiling); the JSON line then lacks the other")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--ceilings", action="store_true",
+                    help="measure streaming-read bandwidth and back-to-back MFMA rate on this machine and stop")
     return ap.parse_args()
 
 
@@ -129,6 +131,11 @@ def main():
     from tffinfer_amd.models import build_model_skeleton, config_from_dict
 
     kernel_lib.load()
+    if args.ceilings:
+        from tffinfer_amd.kernels import ops
+        print(json.dumps({"ceilings": ops.measure_ceilings("cuda:0"),
+                          "published": {"hbm_GBps": HBM_PEAK_GBS, "bf16_TFLOPs": MFMA_PEAK["bf16"] / 1e12}}))
+        return
     cfg = dict(QWEN3_8B)
     L_full = cfg["num_hidden_layers"]
     L = args.layers or L_full

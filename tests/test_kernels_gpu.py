@@ -585,3 +585,12 @@ def test_linear_with_gated_epilogue(M, I, K):
     _close(out, gt / (1 + torch.exp(-gt)) * up, 8e-3, "gated product")
     out32 = ops.linear(x.to(DEV), pw, out_dtype=torch.float32)
     _close(out32, gt / (1 + torch.exp(-gt)) * up, 3e-5, "gated product, float32 out")
+
+
+def test_measured_ceilings_are_plausible():
+    """The measuring kernels run and land where an MI355X can: well above a fraction of the
+    published peaks, never above them."""
+    c = _ops().measure_ceilings(DEV, gib=1.0)
+    assert 1000 < c["stream_read_GBps"] <= 8000
+    assert 300 < c["mfma_bf16_TFLOPs_1_waves_per_simd"] <= c["mfma_bf16_TFLOPs_4_waves_per_simd"] * 1.1 <= 2500 * 1.1
+

@@ -137,3 +137,8 @@ TFF_API int tff_sample(const float* logits, int32_t* out, int rows, int V,
                        const float* temperature, const int32_t* top_k, const float* top_p,
                        const float* min_p, const float* uniform, float* probs_out,
                        tff_stream_t stream);
+
+// Measuring kernels (csrc/probes.hip): stream `bytes` from src once; run blocks x 4 waves of
+// iters x 16 back-to-back 16x16x32 bfloat16 MFMAs.  The caller times them.
+TFF_API int tff_probe_stream_read(const void* src, size_t bytes, void* sink, int blocks, tff_stream_t stream);
+TFF_API int tff_probe_mfma(void* sink, int blocks, int iters, tff_stream_t stream);

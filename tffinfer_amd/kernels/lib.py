@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 
 class KernelLibraryError(RuntimeError):
@@ -40,6 +40,8 @@ _SIGNATURES = {
     "tff_argmax": [_P, _P, _I, _I, _P],
     "tff_repetition_penalty": [_P, _I, _I, _P, _P, _P, _P],
     "tff_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
+    "tff_probe_stream_read": [_P, _Z, _P, _I, _P],
+    "tff_probe_mfma": [_P, _I, _I, _P],
 }
 
 _lib = None

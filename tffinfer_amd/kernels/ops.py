@@ -581,6 +581,41 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tenso
     return (out, probs) if return_probs else out
 
 
+def measure_ceilings(device="cuda:0", gib: float = 4.0) -> dict:
+    """What this machine gives to kernels that do nothing else: streaming reads
+    from HBM into registers (a buffer of ``gib`` GiB, far larger than the
+    caches) and back-to-back bfloat16 MFMAs at 1, 2 and 4 waves per SIMD."""
+    L = _lib.load()
+    dev = torch.device(device)
+    cus = _num_cus(dev)
+    sink = torch.zeros(4, dtype=torch.float32, device=dev)
+    buf = torch.empty(int(gib * (1 << 30)) // 4, dtype=torch.int32, device=dev).fill_(1)
+    nbytes = buf.numel() * 4
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize(dev)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize(dev)
+        return e0.elapsed_time(e1) / 1e3 / reps
+
+    out = {"compute_units": cus}
+    with torch.cuda.device(dev):
+        st = _stream()
+        t = min(timed(lambda: _lib.check(L.tff_probe_stream_read(buf.data_ptr(), nbytes, sink.data_ptr(), cus * b, st)), 3)
+                for b in (8, 16, 32))
+        out["stream_read_GBps"] = round(nbytes / t / 1e9, 1)
+        iters = 20000
+        for waves in (1, 2, 4):
+            t = timed(lambda: _lib.check(L.tff_probe_mfma(sink.data_ptr(), cus * waves, iters, st)), 2)
+            out[f"mfma_bf16_TFLOPs_{waves}_waves_per_simd"] = round(cus * waves * 4 * iters * 16 * 16384 / t / 1e12, 1)
+    return out
+
+
 OP_TABLE = {
     "embed": embed,
     "add_rmsnorm": add_rmsnorm,
