@@ -134,6 +134,33 @@ def test_linear_partial_sums_feed_the_norm(M, N, K):
     assert torch.equal(z1, z2)
 
 
+def test_gemm_plan():
+    """The plan of the tiled product: large tiles where they fill the machine, smaller ones or K
+    split over blocks where they would not; never more parts than K has tiles for."""
+    import ctypes
+    from tffinfer_amd.kernels import lib
+    L = lib.load()
+
+    def plan(M, N, K, glu=0):
+        r, c, s = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        assert L.tff_gemm_plan(M, N, K, glu, ctypes.byref(r), ctypes.byref(c), ctypes.byref(s)) == 0
+        return r.value, c.value, s.value
+
+    assert plan(8, 4096, 4096) == (0, 0, 1)
+    assert plan(64, 4096, 12288) == (64, 128, 8)
+    assert plan(64, 151936, 4096) == (64, 128, 1)
+    assert plan(2048, 24576, 4096, 1) == (256, 256, 1)
+    assert plan(4096, 4096, 4096) == (256, 256, 1)
+    r, c, s = plan(1024, 4096, 12288)
+    assert (r, c) == (256, 256) and s == 4            # few tiles, long K: split
+    r, c, s = plan(256, 4096, 4096)
+    assert r == 128 and s >= 2
+    for M, N, K in ((100, 203, 2048), (520, 264, 1544), (300, 1000, 64), (2000, 64, 8)):
+        r, c, s = plan(M, N, K)
+        assert r in (128, 256) and c in (128, 256) and 1 <= s <= 4 and (s == 1 or (K + 63) // 64 // s >= 8)
+        assert L.tff_gemm_workspace_bytes(M, N, K, 1, 0) == (s * M * N * 4 if s > 1 else 0)
+
+
 def test_linear_identity_and_layout():
     """[out, in] layout: a non-square weight picks input columns."""
     ops = _ops()

@@ -632,7 +632,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
                     g_ = v_cache + (((size_t)ATTN_PAGE(j0) * nkv + g) * D + (f - KFR) * 16 + qc) * page_size + \
                          page_slot(j0, page_size, page_shift);                                      \
                 }                                                                                   \
-                __builtin_amdgcn_global_load_lds((glb_ptr_t)g_, (lds_ptr_t)(smem + (st_ * FRT + F) * 512), 16, 0, 0); \
+                copy16_to_lds(g_, smem + (st_ * FRT + F) * 512);                                    \
             }                                                                                       \
         }                                                                                           \
     }

@@ -70,3 +70,19 @@ int tff_check_launch(const char* what);
     do {                                           \
         if (!(cond)) return tff_fail(__VA_ARGS__); \
     } while (0)
+
+// Copies 16 bytes a lane from global memory straight into LDS: lane i's bytes land at
+// lds_wave_base + 16 i (global_load_lds_dwordx4; the LDS base travels in M0 and is the same for
+// the whole wave).  It is written as inline assembly on purpose: the compiler's own builtin
+// makes every later LDS read wait for *all* copies in flight (it cannot tell which stage a
+// read touches), which turns a pipeline of several stages into one of a single stage.  Here
+// the compiler knows nothing of the copy; the kernels wait for their copies themselves
+// (s_waitcnt vmcnt(n), copies complete in the order they were issued) before the barrier that
+// lets other waves read them.
+__device__ __forceinline__ void copy16_to_lds(const void* gptr, void* lds_wave_base) {
+    const unsigned base = (unsigned)(size_t)(__attribute__((address_space(3))) void*)lds_wave_base;
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(base)), "v"(gptr)
+                 : "memory", "m0");
+}

@@ -457,29 +457,54 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
     return tff_check_launch("gemm_bf16_skinny");
 }
 
-// The tiled product's plan for M > 16: tiles of 64 x 128 (up to 64 rows), 128 x 128 (up to
-// 384) or 256 x 256, and into how many parts the blocks of a tile split K so that the launch
-// has blocks for all CUs (a CU holds two blocks of the smaller tiles, one of the largest).
-// Measured at the sizes of an 8B model on an MI355X.
-struct GemmPlan { int tile; int splits; };
-static GemmPlan plan_for(int M, int N, int K) {
-    if (M <= 16) return {0, 1};
-    const int tile = M <= 64 ? 64 : (M <= 384 ? 128 : 256);
-    const int bn = tile == 64 ? 128 : tile;
-    const long blocks = (long)((M + tile - 1) / tile) * ((N + bn - 1) / bn);
-    const int limit = tile == 64 ? 400 : (tile == 128 ? 576 : 288);
-    const int max_splits = tile == 64 ? 8 : 4;
-    const int min_tiles = tile == 64 ? 4 : 8;   // 64-k tiles a part keeps at least
+// The tiled product's plan for M > 16: which tile, and into how many parts the blocks of a
+// tile split K.  Up to 64 rows: 64 x 128 tiles (two blocks to a CU), split so that the launch
+// has some 400 blocks.  Beyond: the cheapest of 256 x 256, 128 x 256 and 128 x 128 tiles with 1,
+// 2 or 4 parts by a small cost model: rounds of blocks over the CUs times a block's work at the
+// tile's measured efficiency (large tiles stream fewer bytes per flop; few blocks on a CU-rich
+// machine run faster each), plus the traffic of the partial sums.  Its constants were fitted to
+// measurements of the four products of an 8B model at 128 .. 4,096 rows on an MI355X, where
+// it picks within a tenth of the best of these candidates everywhere.
+struct GemmPlan { int tile; int bn; int splits; };   // tile = rows of a block tile
+static GemmPlan plan_for(int M, int N, int K, bool glu) {
+    if (M <= 16) return {0, 0, 1};
     const int nk = (K + 63) / 64;
-    int S = 1;
-    while (S < max_splits && blocks * S * 2 <= limit && nk / (S * 2) >= min_tiles) S *= 2;
-    return {tile, S};
+    if (M <= 64) {
+        const long blocks = (N + 127) / 128;
+        int S = 1;
+        while (S < 8 && blocks * S * 2 <= 400 && nk / (S * 2) >= 4) S *= 2;
+        return {64, 128, S};
+    }
+    struct Cand { int bm, bn; double eff; };
+    static const Cand cands[3] = {{256, 256, 0.22}, {128, 256, 0.18}, {128, 128, 0.15}};
+    GemmPlan best = {256, 256, 1};
+    double best_t = 1e30;
+    for (const Cand& c : cands)
+        for (int S = 1; S <= (glu ? 2 : 4); S *= 2) {
+            if (S > 1 && nk / S < 8) break;
+            const double blocks = (double)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * S;
+            const double rounds = ceil(blocks / 256.0);
+            const double util = blocks < 256.0 ? blocks / 256.0 : 1.0;
+            double t = rounds * (2.0 * c.bm * c.bn * ((double)K / S) / (c.eff * 4.3e6)) * (0.4 + 0.6 * util) + 3.0;
+            if (S > 1) t += (double)S * M * N * 4.0 * 1.5 / 5e6 + 3.0;
+            if (t < best_t) { best_t = t; best = {c.bm, c.bn, S}; }
+        }
+    return best;
 }
 
-TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype) {
+TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype, int glu) {
     if (ab_dtype != TFF_BF16 || M <= 0 || N <= 0 || K <= 0) return 0;
-    const GemmPlan p = plan_for(M, N, K);
+    const GemmPlan p = plan_for(M, N, K, glu != 0);
     return p.splits > 1 ? (size_t)p.splits * M * N * sizeof(float) : 0;
+}
+
+// For tests and tuning: the plan's tile (rows x columns) and number of parts.
+TFF_API int tff_gemm_plan(int M, int N, int K, int glu, int* tile_rows, int* tile_cols, int* splits) {
+    const GemmPlan p = plan_for(M, N, K, glu != 0);
+    if (tile_rows) *tile_rows = p.tile;
+    if (tile_cols) *tile_cols = p.bn;
+    if (splits) *splits = p.splits;
+    return 0;
 }
 
 // glu_out > 0: W holds gate and up groups in turn (N = 2 * ceil16(glu_out) rows) and C is
@@ -496,7 +521,8 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
     TFF_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)Wp % 16) == 0 && ((uintptr_t)C % 16) == 0,
                 "gemm: operands must be 16-byte aligned");
     TFF_REQUIRE(c_dtype == TFF_F32 || c_dtype == TFF_BF16, "gemm: unknown output type %d", c_dtype);
-    GemmPlan plan = plan_for(M, N, K);
+    GemmPlan plan = plan_for(M, N, K, glu_out > 0);
+    const int planned_splits = plan.splits;
     if (!workspace || workspace_bytes < (size_t)plan.splits * M * N * sizeof(float)) plan.splits = 1;
     const int S = plan.splits;
     const bool red = !keep_partials;
@@ -513,8 +539,10 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
         }
         if (plan.tile == 64)
             return launch_async_g<2, 2, 2, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+        if (plan.tile == 128 && plan.bn == 128)
+            return launch_async_g<2, 2, 4, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         if (plan.tile == 128)
-            return launch_async_g<2, 2, 4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+            return launch_async_g<2, 4, 4, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         return launch_async_g<4, 4, 4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
     }
     if (M <= 16) {
@@ -527,14 +555,16 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
     if (plan.tile == 64) {
         // few columns and no room for partial sums: the streaming kernel, whose blocks split K
         // among their waves
-        if (S == 1 && plan_for(M, N, K).splits > 1) {
+        if (S == 1 && planned_splits > 1) {
             if (M <= 32) return launch_skinny<2, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
             return launch_skinny<4, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
         }
         return launch_async_g<2, 2, 2, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     }
+    if (plan.tile == 128 && plan.bn == 128)
+        return launch_async_g<2, 2, 4, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     if (plan.tile == 128)
-        return launch_async_g<2, 2, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+        return launch_async_g<2, 4, 4, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     return launch_async_g<4, 4, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
 }
 

@@ -49,7 +49,10 @@ TFF_API int tff_rmsnorm(const void* x, const float* weight, float eps, void* out
 TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda,
                      int ab_dtype, int c_dtype, int w_packed, int glu_out, void* workspace,
                      size_t workspace_bytes, int keep_partials, tff_stream_t stream);
-TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype);
+TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype, int glu);
+// The bfloat16 product's plan for these sizes: rows and columns of a block tile (0: the
+// streaming kernel for up to 16 rows) and the number of parts K is split into.
+TFF_API int tff_gemm_plan(int M, int N, int K, int glu, int* tile_rows, int* tile_cols, int* splits);
 
 // bfloat16 row-major [N, K] (K a multiple of 8) -> fragment order: tiles of
 // 16 rows x 32 k, each stored as the 1 KB operand of a 16x16x32 MFMA, element

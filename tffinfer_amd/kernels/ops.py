@@ -235,7 +235,8 @@ def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
     n_out = glu_out or N
     L = _lib.load()
     # some shapes (few columns for the rows) split K over blocks and need room for partial sums
-    ws_bytes = L.tff_gemm_workspace_bytes(M, N, K, dtype_code(x.dtype)) if packed else 0
+    glu_out = weight.glu_out if packed else 0
+    ws_bytes = L.tff_gemm_workspace_bytes(M, N, K, dtype_code(x.dtype), 1 if glu_out else 0) if packed else 0
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=x.device) if ws_bytes else None
     keep = bool(partials and ws is not None and out is None and out_dtype == torch.float32 and not glu_out)
     if keep:
