@@ -291,7 +291,7 @@ def test_attention_far_key_stands_out():
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("pairing", ["half", "interleaved"])
-@pytest.mark.parametrize("T", [9, 75])
+@pytest.mark.parametrize("T", [9, 139])
 @pytest.mark.parametrize("nq,nkv,d,rot", [(4, 2, 16, 16), (3, 1, 48, 48), (8, 2, 128, 128), (2, 2, 64, 32),
                                            (5, 1, 32, 32), (3, 2, 256, 256), (9, 3, 64, 64)])
 def test_qk_norm_rope_kv(dtype, pairing, nq, nkv, d, rot, T):
@@ -309,11 +309,13 @@ def test_qk_norm_rope_kv(dtype, pairing, nq, nkv, d, rot, T):
         positions = torch.tensor([0, 1, 2, 17, 18, 40, 41, 42, 99], dtype=torch.int32)
         slots = torch.tensor([3, 47, 8, 9, 10, -1, 0, 1, 2], dtype=torch.int32)
     else:
-        num_pages = 20
+        num_pages = 40
         positions = torch.cat([torch.arange(5, 45), torch.tensor([0]), torch.arange(100, 120),
-                               torch.tensor([7, 99, 3, 64, 65, 66, 67, 68, 69, 70, 71, 2, 1, 127])]).to(torch.int32)
+                               torch.tensor([7, 99, 3, 64, 65, 66, 67, 68, 69, 70, 71, 2, 1, 127]),
+                               torch.arange(30, 94)]).to(torch.int32)
         slots = torch.cat([torch.arange(16, 56), torch.tensor([-1]), torch.arange(59, 79),
-                           torch.tensor([0, 9, 150, 96, 97, 98, 99, 100, 101, 102, 103, 159, 5, 88])]).to(torch.int32)
+                           torch.tensor([0, 9, 150, 96, 97, 98, 99, 100, 101, 102, 103, 159, 5, 88]),
+                           torch.arange(200, 264)]).to(torch.int32)
         assert len(positions) == T and len(slots) == T
     rope = RotaryEmbedding(d, theta, pairing, rotary_dim=rot)
     table = rope.table(128, DEV)

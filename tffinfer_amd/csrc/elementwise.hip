@@ -531,7 +531,7 @@ TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d, const 
     TFF_REQUIRE(dtype == TFF_F32 || dtype == TFF_BF16, "qk_norm_rope_kv: unknown dtype %d", dtype);
     const bool pow2 = d >= 16 && d <= 256 && (d & (d - 1)) == 0;
     // for prompt portions: two kernels with 16-byte accesses; a few tokens are done by one launch
-    if (T >= 32 && dtype == TFF_BF16 && pow2 && (!cos_sin || rot_dim == d) && ((uintptr_t)qkv % 16) == 0 &&
+    if (T >= 128 && dtype == TFF_BF16 && pow2 && (!cos_sin || rot_dim == d) && ((uintptr_t)qkv % 16) == 0 &&
         ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 16) == 0 &&
         (!q_weight || (((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0)) &&
         (!cos_sin || ((uintptr_t)cos_sin % 16) == 0)) {
