@@ -141,9 +141,9 @@ def test_gemm_plan():
     from tffinfer_amd.kernels import lib
     L = lib.load()
 
-    def plan(M, N, K, glu=0):
+    def plan(M, N, K, glu=0, keep=0):
         r, c, s = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
-        assert L.tff_gemm_plan(M, N, K, glu, ctypes.byref(r), ctypes.byref(c), ctypes.byref(s)) == 0
+        assert L.tff_gemm_plan(M, N, K, glu, keep, ctypes.byref(r), ctypes.byref(c), ctypes.byref(s)) == 0
         return r.value, c.value, s.value
 
     assert plan(8, 4096, 4096) == (0, 0, 1)
@@ -152,13 +152,14 @@ def test_gemm_plan():
     assert plan(2048, 24576, 4096, 1) == (256, 256, 1)
     assert plan(4096, 4096, 4096) == (256, 256, 1)
     r, c, s = plan(1024, 4096, 12288)
-    assert (r, c) == (256, 256) and s == 4            # few tiles, long K: split
+    assert r >= 128 and c == 256 and s >= 2           # few tiles, long K: split
     r, c, s = plan(256, 4096, 4096)
-    assert r == 128 and s >= 2
+    assert r <= 128 and s >= 2
     for M, N, K in ((100, 203, 2048), (520, 264, 1544), (300, 1000, 64), (2000, 64, 8)):
         r, c, s = plan(M, N, K)
-        assert r in (128, 256) and c in (128, 256) and 1 <= s <= 4 and (s == 1 or (K + 63) // 64 // s >= 8)
-        assert L.tff_gemm_workspace_bytes(M, N, K, 1, 0) == (s * M * N * 4 if s > 1 else 0)
+        assert r in (64, 128, 256) and c in (128, 256) and 1 <= s <= 8 and (s == 1 or (K + 63) // 64 // s >= 8)
+        assert L.tff_gemm_workspace_bytes(M, N, K, 1, 0, 0) == (s * M * N * 4 if s > 1 else 0)
+    assert plan(2048, 4096, 12288, keep=1)[2] >= plan(2048, 4096, 12288)[2]   # kept sums cost less
 
 
 def test_linear_identity_and_layout():
@@ -526,6 +527,94 @@ def test_attention_mfma_decode_split_keys(nq, nkv, d, ps, window, splits):
                        for r in range(T)])
     out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale, splits=splits)
     _close(out.reshape(T, nq, d), ref, 1.5e-2, "split-key decode attention")
+
+
+@pytest.mark.parametrize("with_norm,with_rope", [(True, True), (False, True), (True, False)])
+@pytest.mark.parametrize("nq,nkv,d,ps,window,splits,pairing", [
+    (32, 8, 128, 16, 0, None, "half"), (32, 8, 128, 16, 0, 1, "interleaved"), (4, 2, 16, 16, 0, 3, "interleaved"),
+    (8, 2, 32, 8, 24, 4, "interleaved"), (40, 2, 96, 8, 0, 5, "interleaved"), (6, 3, 48, 8, 100, None, "interleaved"),
+    (16, 1, 64, 32, 0, 64, "half"), (4, 2, 192, 16, 0, 3, "half"), (2, 1, 256, 8, 0, None, "half")])
+def test_attention_decode_fused(nq, nkv, d, ps, window, splits, pairing, with_norm, with_rope):
+    """Decode steps from the raw projection output: q/k norm, rotation, the token's key and value
+    into its page and attention in one kernel, against each part's formula; the slot of the new
+    token holds large numbers beforehand, which must not reach the result; nothing else in the
+    cache changes; with write_kv off the cache is read only."""
+    ops = _ops()
+    from tffinfer_amd.parts.position import RotaryEmbedding
+    eps, theta = 1e-5, 5000.0
+    entries = [(0, 1), (1, 1), (31, 1), (32, 1), (700, 1), (255, 1), (64, 1), (7, 1), (8, 1)]
+    batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=d + ps)
+    R = batch.num_tokens
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(R, (nq + 2 * nkv) * d, generator=g).to(torch.bfloat16)
+    qw = (1 + 0.1 * torch.randn(d, generator=g)) if with_norm else None
+    kw = (1 + 0.1 * torch.randn(d, generator=g)) if with_norm else None
+    table = RotaryEmbedding(d, theta, pairing).table(1024, DEV) if with_rope else None
+    pr = 1 if pairing == "interleaved" else 0
+    x = qkv.double()
+
+    def norm(a, w):
+        return a if w is None else a * torch.rsqrt((a * a).mean(-1, keepdim=True) + eps) * w.double()
+
+    def rotate(a):
+        if not with_rope:
+            return a
+        ang = positions.double()[:, None] * torch.exp(-(2.0 * torch.arange(d // 2).double() / d) * math.log(theta))
+        c, sn = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        out = a.clone()
+        if pairing == "half":
+            lo, hi = a[..., :d // 2], a[..., d // 2:]
+            out[..., :d // 2] = lo * c - hi * sn
+            out[..., d // 2:] = lo * sn + hi * c
+        else:
+            ev, od = a[..., 0::2], a[..., 1::2]
+            out[..., 0::2] = ev * c - od * sn
+            out[..., 1::2] = ev * sn + od * c
+        return out
+
+    q = rotate(norm(x[:, :nq * d].reshape(R, nq, d), qw)).to(torch.bfloat16)
+    k_new = rotate(norm(x[:, nq * d:(nq + nkv) * d].reshape(R, nkv, d), kw)).to(torch.bfloat16)
+    v_new = qkv[:, (nq + nkv) * d:].reshape(R, nkv, d)
+    scale = 1 / math.sqrt(d)
+    refs = []
+    for r, (P, _) in enumerate(entries):
+        k = torch.cat([ks[r][:P], k_new[r:r + 1]])
+        v = torch.cat([vs[r][:P], v_new[r:r + 1]])
+        refs.append(_attn_ref(q[r:r + 1], k, v, positions[r:r + 1], window, scale)[0])
+    ref = torch.stack(refs)
+    # the slots of the new tokens hold numbers that would wreck the result if they were read
+    bt = kv.block_tables.cpu()
+    kc0, vc0 = kv.k_cache.cpu().clone(), kv.v_cache.cpu().clone()
+    for r, (P, _) in enumerate(entries):
+        kc0[bt[r, P // ps], :, P % ps] = 300.0
+        vc0[bt[r, P // ps], :, :, P % ps] = -300.0
+    kv.k_cache, kv.v_cache = kc0.to(DEV), vc0.to(DEV)
+    w = (None if qw is None else qw.to(DEV), None if kw is None else kw.to(DEV))
+    assert ops.decode_fused_supported(qkv.to(DEV), d, ps, table, pr, batch)
+    out = ops.attention_decode_fused(qkv.to(DEV), nq, nkv, d, w[0], w[1], eps, table, pr, kv, batch, window, scale,
+                                     write_kv=True, splits=splits)
+    _close(out.reshape(R, nq, d), ref, 1.5e-2, "fused decode attention")
+    kc1, vc1 = kv.k_cache.cpu(), kv.v_cache.cpu()
+    expect_k, expect_v = kc0.clone(), vc0.clone()
+    for r, (P, _) in enumerate(entries):
+        _close(kc1[bt[r, P // ps], :, P % ps], k_new[r].double(), 8e-3, f"key of entry {r} in its page")
+        assert torch.equal(vc1[bt[r, P // ps], :, :, P % ps], v_new[r]), f"value of entry {r} in its page"
+        expect_k[bt[r, P // ps], :, P % ps] = kc1[bt[r, P // ps], :, P % ps]
+        expect_v[bt[r, P // ps], :, :, P % ps] = vc1[bt[r, P // ps], :, :, P % ps]
+    assert torch.equal(kc1, expect_k) and torch.equal(vc1, expect_v), "a slot of another token was written"
+    # a call that only reads: the pages hold the token already
+    out2 = ops.attention_decode_fused(qkv.to(DEV), nq, nkv, d, w[0], w[1], eps, table, pr, kv, batch, window, scale,
+                                      write_kv=False, splits=splits)
+    assert torch.equal(kv.k_cache.cpu(), kc1) and torch.equal(kv.v_cache.cpu(), vc1)
+    _close(out2.reshape(R, nq, d), ref, 1.5e-2, "fused decode attention, cache read only")
+    # the two-kernel path gives the same to rounding
+    kv.k_cache, kv.v_cache = kc0.to(DEV), vc0.to(DEV)
+    slots = torch.tensor([int(bt[r, P // ps]) * ps + P % ps for r, (P, _) in enumerate(entries)], dtype=torch.int32)
+    dq = qkv.to(DEV).clone()
+    ops.qk_norm_rope_kv(dq, nq, nkv, d, w[0], w[1], eps, table, pr, batch.positions, slots.to(DEV),
+                        kv.k_cache, kv.v_cache)
+    out3 = ops.attention_mfma(dq, nq, nkv, d, kv, batch, window, scale, splits=splits)
+    _close(out.reshape(R, nq, d), out3.reshape(R, nq, d).double().cpu(), 1.5e-2, "fused against two kernels")
 
 
 @pytest.mark.parametrize("nq,nkv,d,ps,window", [(32, 8, 128, 16, 0), (8, 2, 32, 8, 300), (40, 2, 96, 8, 0)])

@@ -266,17 +266,104 @@ __global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
 // (r / 4) * 8 + t * 4 + r % 4, so lane (col, g) holds the scores of the eight
 // consecutive keys g*8 .. g*8+7 and reads its values as one 16-byte run.
 #define ATTN_WAVE_BT 1024
-template <int DT, bool SPLIT, int RING>
+
+// What the decoding kernel needs to take q, k and v as the fused projection left them (one row
+// of (nq + 2 nkv) d elements per token) instead of a finished q and a cache that already holds
+// the token: the weights of the per-head RMS norms of q and k (null: no norm), the table of
+// rotation angles [position][pair][cos, sin] (null: no rotation; else the whole head is
+// rotated), the pairing (0: (i, i + d/2), 1: (2i, 2i+1)) and the caches to write the token's
+// key and value into (null: the cache holds them already and is only read).
+struct AttnFuse {
+    const float* q_weight;
+    const float* k_weight;
+    const float* cos_sin;
+    bf16_t* k_write;
+    bf16_t* v_write;
+    float eps;
+    int pairing;
+};
+
+// RMS norm over the head and rotation of one head held as MFMA operand fragments: lane group kg
+// has the elements ks * 32 + kg * 8 .. + 7 of every 32-element step ks, so with pairs (i, i + d/2)
+// (d a multiple of 64) both elements of a pair are in the same lane, KS / 2 steps apart, and with
+// pairs (2i, 2i+1) they are neighbours.  The four lane groups of a column add up the squares.
+// w and cs point into LDS (the kernel put the weights and the position's angles there).
+template <int DT>
+__device__ __forceinline__ void norm_rope_fragments(bf16x8 (&f)[(DT * 16 + 31) / 32], bool has_norm,
+                                                    const float* w, float eps, bool has_rope,
+                                                    const float* cs, int pairing, int kg) {
+    constexpr int D = DT * 16;
+    constexpr int KS = (D + 31) / 32;
+    float x[KS][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            x[ks][j] = (float)f[ks][j];
+            ss = fmaf(x[ks][j], x[ks][j], ss);
+        }
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    if (has_norm) {
+        const float rr = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int e = ks * 32 + kg * 8;
+            if (e < D) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) x[ks][j] = x[ks][j] * rr * w[e + j];
+            }
+        }
+    }
+    if (has_rope) {
+        if (pairing == 0) {
+            if constexpr (KS % 2 == 0) {
+#pragma unroll
+                for (int ks = 0; ks < KS / 2; ++ks)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const int p = ks * 32 + kg * 8 + j;
+                        const float c = cs[2 * p], sn = cs[2 * p + 1];
+                        const float a = x[ks][j], b = x[ks + KS / 2][j];
+                        x[ks][j] = a * c - b * sn;
+                        x[ks + KS / 2][j] = a * sn + b * c;
+                    }
+            }
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int e = ks * 32 + kg * 8;
+                if (e < D) {
+#pragma unroll
+                    for (int j = 0; j < 8; j += 2) {
+                        const int p = (e + j) >> 1;
+                        const float c = cs[2 * p], sn = cs[2 * p + 1];
+                        const float a = x[ks][j], b = x[ks][j + 1];
+                        x[ks][j] = a * c - b * sn;
+                        x[ks][j + 1] = a * sn + b * c;
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[ks][j] = (bf16_t)x[ks][j];
+}
+template <int DT, bool SPLIT, int RING, bool FUSED = false>
 __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int bt_stride,
     const int32_t* __restrict__ cu_tokens, const int32_t* __restrict__ start_pos,
     const int32_t* __restrict__ work, int tiles_per_entry, int nq, int nkv, int page_size,
-    int page_shift, int window, float scale, int T_total) {
+    int page_shift, int window, float scale, int T_total, AttnFuse fz) {
     constexpr int D = DT * 16;
     constexpr int KS = (D + 31) / 32;
     __shared__ int32_t bt_lds[ATTN_WAVE_BT];
+    __shared__ __attribute__((aligned(16))) float fz_lds[FUSED ? 3 * D : 4];   // q weight, k weight, (cos, sin) pairs
     const int lane = threadIdx.x, qc = lane & 15, kg = lane >> 4;
     int r, col0;
     if (work) {
@@ -316,6 +403,25 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
         s_end = min(nsteps, s_begin + per);
     }
 
+    // FUSED (entries of one token): q comes as the projection left it and is normalised and
+    // rotated here; the wave whose keys end with the token's own position does the same for
+    // the token's key, puts key and value into their page and works on them from registers.
+    // The norm weights and the position's angles go to LDS beside the page numbers; the raw q, k
+    // and v are loaded after the barrier and worked on once the first keys and values are on
+    // their way, so that they delay nothing.
+    const bool owns_new = FUSED && fz.k_write != nullptr && s_begin < s_end && s_end == nsteps;
+    const bool has_norm = FUSED && fz.q_weight != nullptr, has_rope = FUSED && fz.cos_sin != nullptr;
+
+    if constexpr (FUSED) {
+        for (int i = lane; i < D; i += 64) {
+            if (has_norm) {
+                fz_lds[i] = fz.q_weight[i];
+                fz_lds[D + i] = fz.k_weight[i];
+            }
+            if (has_rope) fz_lds[2 * D + i] = fz.cos_sin[(size_t)P * D + i];
+        }
+    }
+
     // the page numbers of this wave's keys
     int pi0 = 0;
     bool bt_in_lds = false;
@@ -337,6 +443,23 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
             uint4 v = make_uint4(0, 0, 0, 0);
             if (c_ok && e < D) v = *reinterpret_cast<const uint4*>(qp + e);
             qf[ks] = *reinterpret_cast<bf16x8*>(&v);
+        }
+    }
+    bf16x8 knew[KS];
+    bf16_t vnew[DT];
+    if constexpr (FUSED) {
+        if (owns_new) {
+            const bf16_t* kraw = q + (size_t)tok0 * q_stride + (size_t)(nq + g) * D;
+            const bf16_t* vraw = kraw + (size_t)nkv * D;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int e = ks * 32 + kg * 8;
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (e < D) v = *reinterpret_cast<const uint4*>(kraw + e);
+                knew[ks] = *reinterpret_cast<bf16x8*>(&v);
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vnew[dt] = vraw[dt * 16 + qc];
         }
     }
 
@@ -374,6 +497,20 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
             const uint4 v_ = *reinterpret_cast<const uint4*>(vrun_ + (size_t)(dt * 16 + qc) * page_size); \
             vf[buf][dt] = *reinterpret_cast<const bf16x8*>(&v_);                                    \
         }                                                                                           \
+    }
+    /* the token's own key and value (the last key of the last step): from registers, not from */
+    /* the page */
+#define TFF_WAVE_PATCH(buf, step)                                                                   \
+    {                                                                                               \
+        const int kb_ = kb0 + (step) * 32;                                                          \
+        _Pragma("unroll") for (int kt = 0; kt < 2; ++kt)                                            \
+            if (kb_ + (qc >> 2) * 8 + kt * 4 + (qc & 3) >= kmax) {                                  \
+                _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) kf[buf][kt][ks] = knew[ks];       \
+            }                                                                                       \
+        const int at_ = kmax - min(kb_ + kg * 8, (kmax >> 3) << 3);                                 \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt)                                           \
+            _Pragma("unroll") for (int e = 0; e < 8; ++e)                                           \
+                if (e == at_) vf[buf][dt][e] = vnew[dt];                                            \
     }
 #define TFF_WAVE_COMPUTE(buf, step)                                                                 \
     {                                                                                               \
@@ -418,6 +555,29 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
         // steps past the end load the last step again and are not used
 #pragma unroll
         for (int u = 0; u < RING; ++u) TFF_WAVE_LOAD(u, min(s_begin + u, s_end - 1))
+        if constexpr (FUSED) {   // while the first keys and values travel
+            if (has_norm || has_rope) norm_rope_fragments<DT>(qf, has_norm, fz_lds, fz.eps, has_rope, fz_lds + 2 * D, fz.pairing, kg);
+            if (owns_new) {
+                norm_rope_fragments<DT>(knew, has_norm, fz_lds + D, fz.eps, has_rope, fz_lds + 2 * D, fz.pairing, kg);
+                if (col0 == 0) {
+                    const int page = TFF_WAVE_PAGE(P);
+                    const int slot = page_slot(P, page_size, page_shift);
+                    if (qc == 0) {
+                        bf16_t* kd = fz.k_write + (((size_t)page * nkv + g) * page_size + slot) * D;
+#pragma unroll
+                        for (int ks = 0; ks < KS; ++ks) {
+                            const int e = ks * 32 + kg * 8;
+                            if (e < D) *reinterpret_cast<uint4*>(kd + e) = *reinterpret_cast<const uint4*>(&knew[ks]);
+                        }
+                    }
+                    if (kg == 0) {
+                        bf16_t* vd = fz.v_write + ((size_t)page * nkv + g) * D * page_size + slot;
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt) vd[(size_t)(dt * 16 + qc) * page_size] = vnew[dt];
+                    }
+                }
+            }
+        }
         int s = s_begin;
         for (; s_end - s > RING; s += RING) {
 #pragma unroll
@@ -428,9 +588,15 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
         }
 #pragma unroll
         for (int u = 0; u < RING; ++u)
-            if (s + u < s_end) TFF_WAVE_COMPUTE(u, s + u)
+            if (s + u < s_end) {
+                if constexpr (FUSED) {
+                    if (owns_new && s + u == s_end - 1) TFF_WAVE_PATCH(u, s + u)
+                }
+                TFF_WAVE_COMPUTE(u, s + u)
+            }
     }
 #undef TFF_WAVE_PAGE
+#undef TFF_WAVE_PATCH
 #undef TFF_WAVE_LOAD
 #undef TFF_WAVE_COMPUTE
 
@@ -787,7 +953,7 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
                        const int32_t* work, int num_work, const int32_t* block_items, int num_blocks,
                        int tiles_per_entry, int cols_per_wave,
                        int splits, int nq, int nkv, int page_size, int window, float scale,
-                       int T_total, hipStream_t s) {
+                       int T_total, hipStream_t s, const AttnFuse* fuse = nullptr) {
     int page_shift = -1;
     if ((page_size & (page_size - 1)) == 0)
         for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
@@ -804,14 +970,20 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
         return tff_check_launch("attention_mfma_block");
     }
     const dim3 grid(num_work, nkv, splits);
+    const AttnFuse fz = fuse ? *fuse : AttnFuse{nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
 #define TFF_ATTN_ARGS                                                                              \
     q, q_stride, out, part_o, part_ml, k_cache, v_cache, block_tables, bt_stride, cu_tokens,       \
         start_pos, work, tiles_per_entry, nq, nkv, page_size, page_shift, window, scale, T_total
-    if (splits > 1) {
-        attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
+    if (fuse) {
+        if (splits > 1)
+            attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 2), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
+        else
+            attn_wave_kernel<DT, false, (DT <= 8 ? 4 : 2), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
+    } else if (splits > 1) {
+        attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
     } else {
         if (cols_per_wave == 16)
-            attn_wave_kernel<DT, false, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
+            attn_wave_kernel<DT, false, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
         else
             attn_mfma_kernel<DT, 2><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
     }
@@ -878,6 +1050,58 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
     }
 #undef TFF_ATTN_CASE
     return tff_fail("attention_mfma: head size %d", d);
+}
+
+// Decoding steps (every entry brings one token) from the fused projection's output: q, k and v
+// of token r are row r of qkv ([R, (nq + 2 nkv) d]).  Per head, q and k get their RMS norm
+// (weights [d]; both null: none) and the rotation by the angles of the token's position
+// start_pos[r] (cos_sin [max_pos, d/2, 2]; null: none; the whole head is rotated; pairing 0:
+// (i, i + d/2), which needs d to be a multiple of 64, 1: (2i, 2i+1)); with write_kv the token's
+// key and value go to position start_pos[r] of the entry's pages, else the pages hold them
+// already.  Then attention as tff_attention_mfma does it for such a step.
+TFF_API int tff_attention_decode_fused(const void* qkv, int qkv_stride, void* out, float* part_o,
+                                       float* part_ml, void* k_cache, void* v_cache,
+                                       const int32_t* block_tables, int bt_stride,
+                                       const int32_t* cu_tokens, const int32_t* start_pos,
+                                       const float* q_weight, const float* k_weight, float eps,
+                                       const float* cos_sin, int max_pos, int pairing, int write_kv,
+                                       int splits, int R, int nq, int nkv, int d, int page_size,
+                                       int num_pages, int window, float scale, tff_stream_t stream) {
+    TFF_REQUIRE(qkv && out && k_cache && v_cache && block_tables && cu_tokens && start_pos,
+                "attention_decode_fused: null pointer");
+    TFF_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0,
+                "attention_decode_fused: %d query heads are not a multiple of %d key heads", nq, nkv);
+    TFF_REQUIRE(tff_attention_mfma_supported(d, page_size),
+                "attention_decode_fused: head size %d with pages of %d is not supported by the "
+                "matrix-core kernel", d, page_size);
+    TFF_REQUIRE(qkv_stride >= (nq + 2 * nkv) * d && qkv_stride % 8 == 0 && ((uintptr_t)qkv % 16) == 0,
+                "attention_decode_fused: rows of %d elements do not hold (nq + 2 nkv) d = %d, 16-byte aligned",
+                qkv_stride, (nq + 2 * nkv) * d);
+    TFF_REQUIRE((q_weight == nullptr) == (k_weight == nullptr),
+                "attention_decode_fused: q and k norm weights must both be given or both be absent");
+    TFF_REQUIRE(!cos_sin || ((pairing == 1 || (pairing == 0 && d % 64 == 0)) && max_pos > 0),
+                "attention_decode_fused: pairing %d with head size %d is not supported here", pairing, d);
+    TFF_REQUIRE(splits >= 1 && splits <= 256 && nkv <= 65535, "attention_decode_fused: bad split count %d", splits);
+    TFF_REQUIRE(splits == 1 || (part_o && part_ml), "attention_decode_fused: split keys need a workspace");
+    TFF_REQUIRE(bt_stride > 0 && num_pages > 0 && window >= 0 && R >= 0, "attention_decode_fused: bad geometry");
+    if (R == 0) return 0;
+    const int tiles = (nq / nkv + 15) / 16;
+    AttnFuse fz{q_weight, k_weight, cos_sin, write_kv ? (bf16_t*)k_cache : nullptr,
+                write_kv ? (bf16_t*)v_cache : nullptr, eps, pairing};
+    hipStream_t s = (hipStream_t)stream;
+#define TFF_ATTN_CASE(DTV)                                                                          \
+    case DTV * 16:                                                                                  \
+        return launch_attn<DTV>((const bf16_t*)qkv, qkv_stride, (bf16_t*)out, part_o, part_ml,      \
+                                (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,       \
+                                bt_stride, cu_tokens, start_pos, nullptr, R * tiles, nullptr, 0,    \
+                                tiles, 16, splits, nq, nkv, page_size, window, scale, R, s, &fz);
+    switch (d) {
+        TFF_ATTN_CASE(1) TFF_ATTN_CASE(2) TFF_ATTN_CASE(3) TFF_ATTN_CASE(4) TFF_ATTN_CASE(5)
+        TFF_ATTN_CASE(6) TFF_ATTN_CASE(7) TFF_ATTN_CASE(8) TFF_ATTN_CASE(12) TFF_ATTN_CASE(16)
+        default: break;
+    }
+#undef TFF_ATTN_CASE
+    return tff_fail("attention_decode_fused: head size %d", d);
 }
 
 TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml, void* out,

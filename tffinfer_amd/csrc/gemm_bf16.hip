@@ -131,7 +131,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
             const bf16_t* g_;                                                                      \
             if (f < AF) g_ = src[j] + min(kt_ * 64 + (f & 1) * 32 + fg * 8, K - 8);                \
             else g_ = src[j] + (size_t)min(2 * kt_ + ((f - AF) & 1), KB - 1) * 512;                \
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)g_, (lds_ptr_t)(smem + (st_ * FR + f) * 512), 16, 0, 0); \
+            copy16_to_lds(g_, smem + (st_ * FR + f) * 512);                                        \
         }                                                                                          \
     }
 
@@ -459,48 +459,55 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
 
 // The tiled product's plan for M > 16: which tile, and into how many parts the blocks of a
 // tile split K.  Up to 64 rows: 64 x 128 tiles (two blocks to a CU), split so that the launch
-// has some 400 blocks.  Beyond: the cheapest of 256 x 256, 128 x 256 and 128 x 128 tiles with 1,
-// 2 or 4 parts by a small cost model: rounds of blocks over the CUs times a block's work at the
-// tile's measured efficiency (large tiles stream fewer bytes per flop; few blocks on a CU-rich
-// machine run faster each), plus the traffic of the partial sums.  Its constants were fitted to
-// measurements of the four products of an 8B model at 128 .. 4,096 rows on an MI355X, where
-// it picks within a tenth of the best of these candidates everywhere.
+// has some 256 blocks.  Beyond: the cheapest of 256 x 256, 128 x 256, 128 x 128 and 64 x 128
+// tiles with 1 .. 8 parts by a small cost model: rounds of blocks over the CUs times a
+// block's work at the tile's measured rate (large tiles read fewer bytes of LDS per flop; a
+// last round that fills part of the machine costs between half and all of a full one), plus
+// the traffic of the partial sums (less where the caller takes them as they are).  Its constants were fitted to measurements of the four
+// products of an 8B model at 128 .. 2,048 rows on an MI355X, where it picks within a tenth of
+// the best of these candidates everywhere.
 struct GemmPlan { int tile; int bn; int splits; };   // tile = rows of a block tile
-static GemmPlan plan_for(int M, int N, int K, bool glu) {
+static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
     if (M <= 16) return {0, 0, 1};
     const int nk = (K + 63) / 64;
     if (M <= 64) {
         const long blocks = (N + 127) / 128;
         int S = 1;
-        while (S < 8 && blocks * S * 2 <= 400 && nk / (S * 2) >= 4) S *= 2;
+        while (S < 8 && blocks * S * 2 <= 256 && nk / (S * 2) >= 4) S *= 2;
         return {64, 128, S};
     }
-    struct Cand { int bm, bn; double eff; };
-    static const Cand cands[3] = {{256, 256, 0.22}, {128, 256, 0.18}, {128, 128, 0.15}};
+    // rate: flops a microsecond that a CU sustains on blocks of this tile; slots: blocks a CU holds
+    struct Cand { int bm, bn, slots; double rate; };
+    static const Cand cands[4] = {{256, 256, 1, 4.2e6}, {128, 256, 1, 3.8e6}, {128, 128, 1, 2.6e6}, {64, 128, 2, 2.6e6}};
     GemmPlan best = {256, 256, 1};
     double best_t = 1e30;
     for (const Cand& c : cands)
-        for (int S = 1; S <= (glu ? 2 : 4); S *= 2) {
+        for (int S = 1; S <= (glu ? 2 : 8); S *= 2) {
             if (S > 1 && nk / S < 8) break;
             const double blocks = (double)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * S;
-            const double rounds = ceil(blocks / 256.0);
-            const double util = blocks < 256.0 ? blocks / 256.0 : 1.0;
-            double t = rounds * (2.0 * c.bm * c.bn * ((double)K / S) / (c.eff * 4.3e6)) * (0.4 + 0.6 * util) + 3.0;
-            if (S > 1) t += (double)S * M * N * 4.0 * 1.5 / 5e6 + 3.0;
+            const double cap = 256.0 * c.slots;
+            const double rounds = ceil(blocks / cap);
+            const double last = (blocks - (rounds - 1.0) * cap) / cap;
+            const double round_us = 2.0 * c.bm * c.bn * ((double)K / S) * c.slots / c.rate;
+            double t = round_us * (rounds - 1.0 + 0.5 + 0.5 * last) + 3.0;
+            // the partial sums: written, read and added by a second kernel, or (kept) read by the
+            // consumer in place of one plane
+            if (S > 1) t += keep ? (S - 1.0) * M * N * 4.0 / 4e6 : (double)S * M * N * 4.0 / 2e6 + 3.0;
             if (t < best_t) { best_t = t; best = {c.bm, c.bn, S}; }
         }
     return best;
 }
 
-TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype, int glu) {
+TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype, int glu, int keep_partials) {
     if (ab_dtype != TFF_BF16 || M <= 0 || N <= 0 || K <= 0) return 0;
-    const GemmPlan p = plan_for(M, N, K, glu != 0);
+    const GemmPlan p = plan_for(M, N, K, glu != 0, keep_partials != 0);
     return p.splits > 1 ? (size_t)p.splits * M * N * sizeof(float) : 0;
 }
 
 // For tests and tuning: the plan's tile (rows x columns) and number of parts.
-TFF_API int tff_gemm_plan(int M, int N, int K, int glu, int* tile_rows, int* tile_cols, int* splits) {
-    const GemmPlan p = plan_for(M, N, K, glu != 0);
+TFF_API int tff_gemm_plan(int M, int N, int K, int glu, int keep_partials, int* tile_rows, int* tile_cols,
+                          int* splits) {
+    const GemmPlan p = plan_for(M, N, K, glu != 0, keep_partials != 0);
     if (tile_rows) *tile_rows = p.tile;
     if (tile_cols) *tile_cols = p.bn;
     if (splits) *splits = p.splits;
@@ -521,7 +528,7 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
     TFF_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)Wp % 16) == 0 && ((uintptr_t)C % 16) == 0,
                 "gemm: operands must be 16-byte aligned");
     TFF_REQUIRE(c_dtype == TFF_F32 || c_dtype == TFF_BF16, "gemm: unknown output type %d", c_dtype);
-    GemmPlan plan = plan_for(M, N, K, glu_out > 0);
+    GemmPlan plan = plan_for(M, N, K, glu_out > 0, keep_partials != 0);
     const int planned_splits = plan.splits;
     if (!workspace || workspace_bytes < (size_t)plan.splits * M * N * sizeof(float)) plan.splits = 1;
     const int S = plan.splits;
@@ -555,7 +562,7 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
     if (plan.tile == 64) {
         // few columns and no room for partial sums: the streaming kernel, whose blocks split K
         // among their waves
-        if (S == 1 && planned_splits > 1) {
+        if (S == 1 && planned_splits > 1 && M <= 64) {
             if (M <= 32) return launch_skinny<2, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
             return launch_skinny<4, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
         }

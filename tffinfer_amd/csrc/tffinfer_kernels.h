@@ -43,16 +43,18 @@ TFF_API int tff_rmsnorm(const void* x, const float* weight, float eps, void* out
 // workspace (may be null): device memory of tff_gemm_workspace_bytes() bytes the
 // product may keep partial sums in; with less it takes a path that needs none.
 // keep_partials (float32 result, no GLU): if the workspace is used, that is, if
-// tff_gemm_workspace_bytes() > 0 and the workspace has that size, the partial
+// tff_gemm_workspace_bytes() > 0 (asked with the same keep_partials: the plan counts the
+// cheaper hand-over) and the workspace has that size, the partial
 // sums [bytes / (M * N * 4), M, N] are left there for the caller to add up
 // (tff_add_rmsnorm takes them as they are) and C is not written.
 TFF_API int tff_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda,
                      int ab_dtype, int c_dtype, int w_packed, int glu_out, void* workspace,
                      size_t workspace_bytes, int keep_partials, tff_stream_t stream);
-TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype, int glu);
+TFF_API size_t tff_gemm_workspace_bytes(int M, int N, int K, int ab_dtype, int glu, int keep_partials);
 // The bfloat16 product's plan for these sizes: rows and columns of a block tile (0: the
 // streaming kernel for up to 16 rows) and the number of parts K is split into.
-TFF_API int tff_gemm_plan(int M, int N, int K, int glu, int* tile_rows, int* tile_cols, int* splits);
+TFF_API int tff_gemm_plan(int M, int N, int K, int glu, int keep_partials, int* tile_rows, int* tile_cols,
+                          int* splits);
 
 // bfloat16 row-major [N, K] (K a multiple of 8) -> fragment order: tiles of
 // 16 rows x 32 k, each stored as the 1 KB operand of a 16x16x32 MFMA, element
@@ -111,6 +113,22 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                int tiles_per_entry, int cols_per_wave, int splits, int T_total,
                                int nq, int nkv, int d, int page_size, int num_pages, int window,
                                float scale, tff_stream_t stream);
+// Decoding steps (every entry brings one token), bfloat16, from the fused projection's output:
+// row r of qkv ([R, (nq + 2 nkv) d], q heads first, then k, then v) is token r.  The kernel
+// does what tff_qk_norm_rope_kv and tff_attention_mfma do one after the other, in one pass:
+// per-head RMS norm of q and k (weights [d]; both null: none), rotation by the angles of the
+// token's position start_pos[r] (cos_sin [max_pos, d/2, 2]; null: none; the whole head is
+// rotated; pairing 0 needs d to be a multiple of 64), the token's key and value written to
+// their page (write_kv = 0: the pages hold them already), attention over the pages.  With
+// splits > 1 the partial results need tff_attention_split_reduce as there.
+TFF_API int tff_attention_decode_fused(const void* qkv, int qkv_stride, void* out, float* part_o,
+                                       float* part_ml, void* k_cache, void* v_cache,
+                                       const int32_t* block_tables, int bt_stride,
+                                       const int32_t* cu_tokens, const int32_t* start_pos,
+                                       const float* q_weight, const float* k_weight, float eps,
+                                       const float* cos_sin, int max_pos, int pairing, int write_kv,
+                                       int splits, int R, int nq, int nkv, int d, int page_size,
+                                       int num_pages, int window, float scale, tff_stream_t stream);
 // Merges partial results kept by entry (part_o [splits, R_total, nq, d]) into out rows:
 // rows (may be null: entry i is token i for all R_total) holds (entry, token) pairs.
 TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml, void* out,

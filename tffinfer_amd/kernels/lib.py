@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 
 class KernelLibraryError(RuntimeError):
@@ -24,8 +24,8 @@ _SIGNATURES = {
     "tff_add_rmsnorm": [_P, _P, _I, _Z, _P, _F, _P, _P, _I, _I, _I, _P],
     "tff_rmsnorm": [_P, _P, _F, _P, _I, _I, _I, _P],
     "tff_gemm": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _Z, _I, _P],
-    "tff_gemm_workspace_bytes": [_I, _I, _I, _I, _I],
-    "tff_gemm_plan": [_I, _I, _I, _I, _P, _P, _P],
+    "tff_gemm_workspace_bytes": [_I, _I, _I, _I, _I, _I],
+    "tff_gemm_plan": [_I, _I, _I, _I, _I, _P, _P, _P],
     "tff_pack_weight": [_P, _P, _I, _I, _P],
     "tff_embed_packed": [_P, _P, _P, _I, _I, _I, _P],
     "tff_qk_norm_rope_kv": [_P, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _I, _P, _P, _P, _P,
@@ -35,6 +35,8 @@ _SIGNATURES = {
     "tff_attention_mfma_supported": [_I, _I],
     "tff_attention_mfma": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I,
                            _I, _I, _I, _I, _I, _I, _F, _P],
+    "tff_attention_decode_fused": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _F, _P, _I, _I, _I,
+                                   _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "tff_attention_split_reduce": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _P],
     "tff_swiglu": [_P, _P, _I, _I, _I, _P],
     "tff_cast": [_P, _I, _P, _I, c_int64, _P],

@@ -235,10 +235,11 @@ def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
     n_out = glu_out or N
     L = _lib.load()
     # some shapes (few columns for the rows) split K over blocks and need room for partial sums
-    glu_out = weight.glu_out if packed else 0
-    ws_bytes = L.tff_gemm_workspace_bytes(M, N, K, dtype_code(x.dtype), 1 if glu_out else 0) if packed else 0
+    want = bool(partials and packed and out is None and out_dtype == torch.float32 and not glu_out)
+    ws_bytes = (L.tff_gemm_workspace_bytes(M, N, K, dtype_code(x.dtype), 1 if glu_out else 0, 1 if want else 0)
+                if packed else 0)
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=x.device) if ws_bytes else None
-    keep = bool(partials and ws is not None and out is None and out_dtype == torch.float32 and not glu_out)
+    keep = want and ws is not None
     if keep:
         out = ws.view(-1, M, N)
     elif out is None:
@@ -498,6 +499,90 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
     return out
 
 
+def decode_fused_supported(qkv: torch.Tensor, d: int, page_size: int, cos_sin, pairing: int, batch) -> bool:
+    """Whether :func:`attention_decode_fused` takes this step: bfloat16, a head
+    size of the matrix-core kernel, every entry one token, the whole head
+    rotated (or none of it) with a pairing the kernel has in one lane."""
+    if batch.max_new_tokens != 1 or not mfma_attention_supported(qkv.dtype, d, page_size):
+        return False
+    if cos_sin is None:
+        return True
+    return 2 * cos_sin.shape[1] == d and (pairing == 1 or d % 64 == 0)
+
+
+def attention_decode_fused(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, eps: float,
+                           cos_sin, pairing: int, kv, batch, window: int = 0, scale: float | None = None,
+                           write_kv: bool = True, splits: int | None = None) -> torch.Tensor:
+    """A decode-only step from the fused projection's output ``qkv`` [R, (nq +
+    2 nkv) d]: q/k norm, rotation, the new keys and values into their pages and
+    the attention over the pages, in one kernel (plus the merge of split keys)."""
+    _req(qkv, "attention_decode_fused qkv", torch.bfloat16, 2)
+    R = batch.num_reqs
+    if qkv.shape[0] != R or batch.num_tokens != R or batch.max_new_tokens != 1:
+        raise _lib.KernelError("attention_decode_fused: every entry of the step must bring one token")
+    if qkv.shape[1] != (nq + 2 * nkv) * d:
+        raise _lib.KernelError(
+            f"attention_decode_fused: rows of {qkv.shape[1]} are not (nq + 2 nkv) d = {(nq + 2 * nkv) * d}")
+    k_cache, v_cache = kv.k_cache, kv.v_cache
+    _req(k_cache, "k cache", qkv.dtype, 4)
+    _req(v_cache, "v cache", qkv.dtype, 4)
+    _check_cache(k_cache, v_cache, nkv, d, "attention_decode_fused")
+    bt = _req(kv.block_tables, "block tables", torch.int32, 2)
+    _req(batch.cu_tokens, "cu_tokens", torch.int32, 1)
+    _req(batch.start_pos, "start_pos", torch.int32, 1)
+    if batch.cu_tokens.numel() != R + 1 or batch.start_pos.numel() != R or bt.shape[0] != R:
+        raise _lib.KernelError("attention_decode_fused: the step's tables do not describe the same number of requests")
+    for w, nm in ((q_weight, "q norm weight"), (k_weight, "k norm weight")):
+        if w is not None:
+            _req(w, nm, torch.float32, 1)
+            if w.numel() != d:
+                raise _lib.KernelError(f"{nm}: {w.numel()} elements, head size {d}")
+    max_pos = 0
+    if cos_sin is not None:
+        _req(cos_sin, "rotation table", torch.float32, 3)
+        max_pos = cos_sin.shape[0]
+        if 2 * cos_sin.shape[1] != d or cos_sin.shape[2] != 2:
+            raise _lib.KernelError(f"attention_decode_fused: a rotation table of shape {tuple(cos_sin.shape)} "
+                                   f"does not rotate whole heads of {d}")
+    G = nq // nkv
+    tiles = -(-G // 16)
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    if splits is None:
+        splits = getattr(batch, "attn_splits", None) or pick_splits(R * tiles * nkv, batch.max_context)
+    out = torch.empty(R, nq * d, dtype=qkv.dtype, device=qkv.device)
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty(splits, R, nq, d, dtype=torch.float32, device=qkv.device)
+        part_ml = torch.empty(splits, R, nq, 2, dtype=torch.float32, device=qkv.device)
+    L = _lib.load()
+    stream = _stream()
+    _lib.check(L.tff_attention_decode_fused(
+        qkv.data_ptr(), qkv.stride(0), out.data_ptr(), _ptr(part_o), _ptr(part_ml), k_cache.data_ptr(),
+        v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(), batch.start_pos.data_ptr(),
+        _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin), max_pos, int(pairing), 1 if write_kv else 0,
+        splits, R, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale), stream))
+    if splits > 1:
+        _lib.check(L.tff_attention_split_reduce(part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), splits, R,
+                                                nq, d, None, 0, stream))
+    return out
+
+
+def qkv_attention(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, eps: float, cos_sin,
+                  pairing: int, kv, batch, window: int = 0, scale: float | None = None) -> torch.Tensor:
+    """From the fused projection's output to the attention's output [T, nq d]:
+    q/k norm and rotation, the step's keys and values into the cache (unless
+    ``kv.writes`` is false: the call reads a cache that another call fills),
+    attention over the cache.  Decode-only steps in bfloat16 are one kernel."""
+    writes = getattr(kv, "writes", True)
+    if decode_fused_supported(qkv, d, kv.k_cache.shape[2], cos_sin, pairing, batch):
+        return attention_decode_fused(qkv, nq, nkv, d, q_weight, k_weight, eps, cos_sin, pairing, kv, batch,
+                                      window, scale, write_kv=writes)
+    qk_norm_rope_kv(qkv, nq, nkv, d, q_weight, k_weight, eps, cos_sin, pairing, batch.positions,
+                    kv.slot_mapping, kv.k_cache, kv.v_cache)
+    return paged_attention(qkv, nq, nkv, d, kv, batch, window, scale)
+
+
 def paged_attention(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,
                     scale: float | None = None) -> torch.Tensor:
     """Attention of a step's tokens over the cache view ``kv`` (k_cache,
@@ -627,6 +712,8 @@ OP_TABLE = {
     "attention": paged_attention,
     "attention_generic": attention_generic,
     "attention_mfma": attention_mfma,
+    "attention_decode_fused": attention_decode_fused,
+    "qkv_attention": qkv_attention,
     "swiglu": swiglu,
     "cast": cast,
     "argmax": argmax,

@@ -77,7 +77,6 @@ class GQAttention(Mixer):
         qkv = ops.linear(x, self.w_qkv)
         table = self.position.table(ctx.max_positions, x.device) if self.position is not None else None
         pairing = 1 if (self.position is not None and self.position.pairing == "interleaved") else 0
-        ops.qk_norm_rope_kv(qkv, nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0,
-                            table, pairing, b.positions, kv.slot_mapping, kv.k_cache, kv.v_cache)
-        o = ops.paged_attention(qkv, nq, nkv, d, kv, b, self.window, self.scale)
+        o = ops.qkv_attention(qkv, nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0,
+                              table, pairing, kv, b, self.window, self.scale)
         return ops.linear(o, self.w_o, out_dtype=torch.float32, partials=True)
