@@ -50,7 +50,7 @@ __device__ __forceinline__ floatx4 silu_mul(const floatx4& g, const floatx4& u) 
 }
 
 // ------------------------------------------------------- tiled, async copy ---
-// Block tile (WGM*WTM*16) x (WGN*WTN*16) x 64 on WGM x WGN waves, each wave
+// Block tile (WGM*WTM*16) x (WGN*WTN*16) x (32 KPS) on WGM x WGN waves, each wave
 // WTM x WTN MFMA tiles.  Both operands are staged in LDS in fragment order; the
 // padding of W to 32 k holds zeros, so k past the end of A only has to be
 // readable: what it multiplies is zero.  The copies global -> LDS are done by
@@ -65,14 +65,14 @@ typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 
 constexpr int vmcnt_imm(int v) { return (v & 15) | (7 << 4) | (15 << 8) | ((v >> 4) << 14); }
 
-template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU, typename TC>
+template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU, typename TC, int KPS = 2>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
     int K, int lda, int KB, int n_out, float* __restrict__ part) {
     // WGM x WGN waves, each WTM x WTN MFMA tiles of 16 x 16
     constexpr int NW = WGM * WGN;
     constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
-    constexpr int AF = BM / 16 * 2, WF = BN / 16 * 2;   // fragments per operand tile (2 k-steps)
+    constexpr int AF = BM / 16 * KPS, WF = BN / 16 * KPS;   // fragments per operand tile (KPS k-steps of 32)
     constexpr int FR = AF + WF;                          // fragments per stage, 1 KB each
     constexpr int LPW = FR / NW;                         // copies a wave issues per tile
     static_assert(FR % NW == 0, "fragments are dealt to the waves evenly");
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     if (tn * BN >= N) return;   // the launch is padded to whole groups of eight column tiles
     const int m0 = tm * BM, n0 = tn * BN;
     const int NB = (N + 15) / 16;
-    const int nk = (K + 63) / 64;
+    const int nk = (K + 32 * KPS - 1) / (32 * KPS);
     // With gridDim.z > 1 the blocks of one tile split K among them and leave partial sums in
     // part[z][M][N], which a second kernel adds up in a fixed order.
     const int kt_per = (nk + (int)gridDim.z - 1) / (int)gridDim.z;
@@ -112,10 +112,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     for (int j = 0; j < LPW; ++j) {
         const int f = wave + NW * j;
         if (f < AF) {
-            const int row = min(m0 + (f >> 1) * 16 + fr, M - 1);   // rows past the end repeat the last
+            const int row = min(m0 + (f / KPS) * 16 + fr, M - 1);   // rows past the end repeat the last
             src[j] = A + (size_t)row * lda;
         } else {
-            const int nb = min(n0 / 16 + ((f - AF) >> 1), NB - 1);
+            const int nb = min(n0 / 16 + (f - AF) / KPS, NB - 1);
             src[j] = Wp + (size_t)nb * KB * 512 + lane * 8;
         }
     }
@@ -129,8 +129,8 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
         _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                          \
             const int f = wave + NW * j;                                                            \
             const bf16_t* g_;                                                                      \
-            if (f < AF) g_ = src[j] + min(kt_ * 64 + (f & 1) * 32 + fg * 8, K - 8);                \
-            else g_ = src[j] + (size_t)min(2 * kt_ + ((f - AF) & 1), KB - 1) * 512;                \
+            if (f < AF) g_ = src[j] + min((kt_ * KPS + f % KPS) * 32 + fg * 8, K - 8);                 \
+            else g_ = src[j] + (size_t)min(KPS * kt_ + (f - AF) % KPS, KB - 1) * 512;                  \
             copy16_to_lds(g_, smem + (st_ * FR + f) * 512);                                        \
         }                                                                                          \
     }
@@ -143,15 +143,15 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
         TFF_ISSUE_TILE(kt + STAGES - 1)                              // into the stage read last iteration
         const bf16_t* st = smem + ((kt - kt0) % STAGES) * FR * 512;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            if (2 * kt + ks < KB) {   // k-steps past the end of K are not in W
+        for (int ks = 0; ks < KPS; ++ks) {
+            if (KPS * kt + ks < KB) {   // k-steps past the end of K are not in W
                 bf16x8 fw[WTN], fa[WTM];
 #pragma unroll
                 for (int i = 0; i < WTN; ++i)
-                    fw[i] = *reinterpret_cast<const bf16x8*>(st + (AF + (wn * WTN + i) * 2 + ks) * 512 + lane * 8);
+                    fw[i] = *reinterpret_cast<const bf16x8*>(st + (AF + (wn * WTN + i) * KPS + ks) * 512 + lane * 8);
 #pragma unroll
                 for (int j = 0; j < WTM; ++j)
-                    fa[j] = *reinterpret_cast<const bf16x8*>(st + ((wm * WTM + j) * 2 + ks) * 512 + lane * 8);
+                    fa[j] = *reinterpret_cast<const bf16x8*>(st + ((wm * WTM + j) * KPS + ks) * 512 + lane * 8);
 #pragma unroll
                 for (int i = 0; i < WTN; ++i)
 #pragma unroll
@@ -245,7 +245,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
 }
 
 // splits > 1: the blocks of a tile split K among them; part holds splits * M * N floats
-template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU = false>
+template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU = false, int KPS = 2>
 static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
                           int c_dtype, int n_out, hipStream_t s, int splits = 1, float* part = nullptr,
                           bool reduce = true) {
@@ -256,10 +256,10 @@ static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int
     TFF_REQUIRE(tiles < (1L << 31), "gemm: too many tiles for M=%d N=%d", M, N);
     const dim3 grid((unsigned)tiles, 1, splits);
     if (c_dtype == TFF_F32)
-        gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, float>
+        gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, float, KPS>
             <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out, part);
     else
-        gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, bf16_t>
+        gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, bf16_t, KPS>
             <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out, part);
     if (int rc = tff_check_launch("gemm_bf16_async")) return rc;
     if (splits > 1 && reduce) {
