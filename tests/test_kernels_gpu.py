@@ -115,7 +115,8 @@ def test_linear_partial_sums_feed_the_norm(M, N, K):
     whole = ops.linear(x, pw, out_dtype=torch.float32)
     parts = ops.linear(x, pw, out_dtype=torch.float32, partials=True)
     if M == 8:
-        assert parts.dim() == 2          # nothing to split here: the plain result
+        assert isinstance(parts, ops.PendingProduct)   # a few rows: run by whoever consumes it
+        assert torch.equal(parts.run(), whole)
     else:
         assert parts.dim() == 3 and parts.shape[0] > 1 and tuple(parts.shape[1:]) == (M, N)
         acc = parts[0].clone()
@@ -132,6 +133,58 @@ def test_linear_partial_sums_feed_the_norm(M, N, K):
     z1 = ops.add_rmsnorm(resid.clone(), whole, nw, 1e-6, torch.bfloat16, rows=rows)
     z2 = ops.add_rmsnorm(resid.clone(), parts, nw, 1e-6, torch.bfloat16, rows=rows)
     assert torch.equal(z1, z2)
+
+
+@pytest.mark.parametrize("glu", [False, True])
+@pytest.mark.parametrize("M,H,K,N2", [(1, 64, 64, 96), (8, 4096, 4096, 6144), (5, 320, 96, 200), (16, 200, 1000, 72),
+                                       (3, 1000, 256, 33000), (7, 4096, 12288, 24576), (16, 40, 8200, 136)])
+def test_norm_taken_into_the_products_on_either_side(M, H, K, N2, glu):
+    """Up to 16 rows: the product before a norm adds to the residual stream, writes (sum * norm
+    weight) in bfloat16 and the sums of squares of its groups of 16 columns; the product after it
+    multiplies by the row's factor.  Against the three steps done one after the other, in float64,
+    with the norm's weights and a residual stream whose rows differ in size by orders of magnitude
+    (a factor applied to the wrong row, or a norm left out, would show)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(M * 7 + H)
+    eps = 1e-5
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w1 = (torch.randn(H, K, generator=g) * 0.05).to(torch.bfloat16)
+    resid = torch.randn(M, H, generator=g) * (10.0 ** torch.arange(M).remainder(4).float())[:, None]
+    nw = 1 + 0.3 * torch.randn(H, generator=g)
+    new_resid = resid.double() + x.double() @ w1.double().T
+    normed = new_resid * torch.rsqrt((new_resid * new_resid).mean(-1, keepdim=True) + eps) * nw.double()
+    if glu:
+        I = N2 // 2
+        gate = (torch.randn(I, H, generator=g) * 0.05).to(torch.bfloat16)
+        up = (torch.randn(I, H, generator=g) * 0.05).to(torch.bfloat16)
+        w2 = ops.pack_gate_up(gate.to(DEV), up.to(DEV))
+        a, b = normed @ gate.double().T, normed @ up.double().T
+        ref = a / (1 + torch.exp(-a)) * b
+    else:
+        w2d = (torch.randn(N2, H, generator=g) * 0.05).to(torch.bfloat16)
+        w2 = ops.pack_weight(w2d.to(DEV))
+        ref = normed @ w2d.double().T
+    r = resid.to(DEV).clone()
+    pending = ops.linear(x.to(DEV), ops.pack_weight(w1.to(DEV)), out_dtype=torch.float32, partials=True)
+    assert isinstance(pending, ops.PendingProduct)
+    rows = ops.add_rmsnorm(r, pending, nw.to(DEV), eps, torch.bfloat16, for_linear=True)
+    assert isinstance(rows, ops.ScaledRows)
+    _close(r, new_resid, 2e-5, "residual stream after the product")
+    y = ops.linear(rows, w2, out_dtype=torch.float32)
+    _close(y, ref, 1.2e-2, "product after the norm")
+    for m in range(M):     # row by row: a row's factor is its own
+        _close(y[m], ref[m], 1.5e-2, f"row {m}")
+    _close(rows.materialize(), normed, 8e-3, "normalised rows written out")
+    # the same through the separate kernels, to rounding
+    r2 = resid.to(DEV).clone()
+    z = ops.add_rmsnorm(r2, pending.run(), nw.to(DEV), eps, torch.bfloat16)
+    assert torch.allclose(r2, r, rtol=1e-6, atol=1e-6)
+    y2 = ops.linear(z, w2, out_dtype=torch.float32)
+    _close(y, y2.double().cpu(), 1.2e-2, "fused against separate kernels")
+    # without for_linear (or with rows to gather) the norm gives a plain tensor
+    r3 = resid.to(DEV).clone()
+    z3 = ops.add_rmsnorm(r3, pending, nw.to(DEV), eps, torch.bfloat16)
+    assert isinstance(z3, torch.Tensor) and torch.equal(z3, z) and torch.equal(r3, r2)
 
 
 def test_gemm_plan():

@@ -291,10 +291,35 @@ static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int
 // that, not W, is most of a wave's traffic.  With GLU, sets 2p and 2p+1 hold a
 // gate group and the up group that follows it in W; the epilogue writes
 // silu(gate) * up.
-template <int MT, int R, int UNROLL, int KSPLIT, int NSETS, bool GLU, typename TC, bool RING = false>
+//
+// An RMS norm between two such products costs a kernel of a few microseconds for a few rows.
+// Its per-row factor commutes with the product that follows it, so the two products take the
+// norm between them (EPI):
+//   2, the product before the norm (float32 result): its epilogue adds its result to the
+//      residual stream in place, writes the sum times the norm's weight as the bfloat16 input
+//      of the next product, *without* the factor rsqrt(mean of squares + eps), and leaves the
+//      sum of squares of its 16 columns of every row in ss_out[row][row group];
+//   1, the product after the norm: adds up the sums of squares of a row, in a fixed order, and
+//      multiplies its float32 accumulators by the row's factor before anything else is done
+//      to them.
+// The sum of squares is over the float32 residual stream, as in the norm's own kernel.
+struct SkinnyFuse {
+    const float* ss_in;     // EPI 1: [16][ss_stride] sums of squares, ss_count of them a row
+    int ss_stride, ss_count;
+    float inv_dim, eps;     // 1 / row length of the normalised tensor
+    float* resid;           // EPI 2: [M, N] float32, updated in place
+    const float* norm_w;    // [N]
+    bf16_t* x_out;          // [M, N]
+    float* ss_out;          // [16][ss_out_stride]
+    int ss_out_stride;
+};
+
+template <int MT, int R, int UNROLL, int KSPLIT, int NSETS, bool GLU, typename TC, bool RING = false, int EPI = 0>
 __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
-    int K, int lda, int KB, int n_out) {
+    int K, int lda, int KB, int n_out, SkinnyFuse fz) {
+    static_assert(EPI == 0 || MT == 1, "the fused norm is for up to 16 rows");
+    static_assert(EPI != 2 || (!GLU && R == 1), "the product before a norm has a plain float32 result");
     constexpr int SK_WAVES = KSPLIT * NSETS;
     static_assert(!GLU || (R == 1 && NSETS % 2 == 0), "a gate and its up group are one row group each");
     __shared__ floatx4 part[SK_WAVES][R * MT][64];
@@ -324,6 +349,58 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
 #pragma unroll
     for (int t = 0; t < MT; ++t) arow[t] = A + (size_t)min(t * 16 + fr, M - 1) * lda;
 
+    // What the epilogue needs from memory is asked for first, so that it has arrived long
+    // before the stream of W ends.
+    float row_scale = 1.f;
+    float4 resid_in = make_float4(0.f, 0.f, 0.f, 0.f), normw_in = resid_in;
+    // EPI 1: lane (fr, fg) of a set's first wave adds every fourth group of four sums of row fr,
+    // then the four lanes of a row meet: the same order in every block.  The loads are issued
+    // here and added up (TFF_ROW_SCALE) after the first loads of W are on their way.
+    constexpr int SSV = 16;   // 16-byte loads a lane keeps: rows of up to 64 * SSV sums
+    float4 ssv[EPI == 1 ? SSV : 1];
+    const bool scales = EPI == 1 && wave == 0;
+    if constexpr (EPI == 1) {
+        if (scales) {
+            const float* sp = fz.ss_in + (size_t)fr * fz.ss_stride;
+            const int vec_end = fz.ss_count & ~3;
+#pragma unroll
+            for (int u = 0; u < SSV; ++u) {
+                const int j = fg * 4 + 16 * u;
+                ssv[u] = j < vec_end ? *reinterpret_cast<const float4*>(sp + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+    }
+#define TFF_ROW_SCALE()                                                                            \
+    if constexpr (EPI == 1) {                                                                      \
+        if (scales && row_scale_pending) {                                                         \
+            row_scale_pending = false;                                                             \
+            const float* sp = fz.ss_in + (size_t)fr * fz.ss_stride;                                \
+            const int vec_end = fz.ss_count & ~3;                                                  \
+            float ssum = 0.f;                                                                      \
+            _Pragma("unroll") for (int u = 0; u < SSV; ++u)                                        \
+                if (fg * 4 + 16 * u < vec_end) ssum += (ssv[u].x + ssv[u].y) + (ssv[u].z + ssv[u].w); \
+            for (int j = fg * 4 + 16 * SSV; j < vec_end; j += 16) {   /* very long rows */           \
+                const float4 v = *reinterpret_cast<const float4*>(sp + j);                         \
+                ssum += (v.x + v.y) + (v.z + v.w);                                                 \
+            }                                                                                      \
+            if (fg == 0)                                                                           \
+                for (int j = vec_end; j < fz.ss_count; ++j) ssum += sp[j];                         \
+            ssum += __shfl_xor(ssum, 16, 64);                                                      \
+            ssum += __shfl_xor(ssum, 32, 64);                                                      \
+            row_scale = rsqrtf(ssum * fz.inv_dim + fz.eps);                                        \
+        }                                                                                          \
+    }
+    bool row_scale_pending = true;
+    if constexpr (EPI == 2) {
+        if (wave == 0) {
+            const int n = nb0 * 16 + fg * 4;
+            if (fr < M && n < N) {
+                resid_in = *reinterpret_cast<const float4*>(fz.resid + (size_t)fr * N + n);
+                normw_in = *reinterpret_cast<const float4*>(fz.norm_w + n);
+            }
+        }
+    }
+
     const int full_end = min(s_end, K / 32);   // steps below K / 32 have all their 32 k in A
     int s0 = s_begin;
     if constexpr (RING) {
@@ -342,6 +419,7 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
 #pragma unroll
                 for (int t = 0; t < MT; ++t) ra[u][t] = ld16(arow[t] + st * 32 + fg * 8);
             }
+            TFF_ROW_SCALE()
             for (; s0 < full_end; s0 += UNROLL) {
 #pragma unroll
                 for (int u = 0; u < UNROLL; ++u) {
@@ -372,6 +450,7 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
 #pragma unroll
             for (int t = 0; t < MT; ++t) ra[u][t] = ld16(arow[t] + (s0 + u) * 32 + fg * 8);
         }
+        TFF_ROW_SCALE()
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
@@ -399,6 +478,8 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
             for (int t = 0; t < MT; ++t)
                 acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(rw[r]), as_frag(ra[t]), acc[r][t], 0, 0, 0);
     }
+    TFF_ROW_SCALE()   // if no loop above came to it
+#undef TFF_ROW_SCALE
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -416,6 +497,10 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
                         const floatx4 pg = part[set * KSPLIT + w][t][lane], pu = part[(set + 1) * KSPLIT + w][t][lane];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) { g[e] += pg[e]; u[e] += pu[e]; }
+                    }
+                    if constexpr (EPI == 1) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) { g[e] *= row_scale; u[e] *= row_scale; }
                     }
                     const int n = (nb0 >> 1) * 16 + fg * 4;
                     const int m = t * 16 + fr;
@@ -436,24 +521,50 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
                     }
                     const int n = (nb0 + r) * 16 + fg * 4;
                     const int m = t * 16 + fr;
-                    if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, v, n, N, vec);
+                    if constexpr (EPI == 1) {
+                        v[0] *= row_scale; v[1] *= row_scale; v[2] *= row_scale; v[3] *= row_scale;
+                    }
+                    if constexpr (EPI == 2) {
+                        // N is a multiple of 4 here: four columns are in or out together
+                        float ss = 0.f;
+                        if (m < M && n < N) {
+                            const float4 sum = make_float4(resid_in.x + v[0], resid_in.y + v[1],
+                                                           resid_in.z + v[2], resid_in.w + v[3]);
+                            *reinterpret_cast<float4*>(fz.resid + (size_t)m * N + n) = sum;
+                            union { bf16_t h[4]; uint2 u; } pk;
+                            pk.h[0] = (bf16_t)(sum.x * normw_in.x);
+                            pk.h[1] = (bf16_t)(sum.y * normw_in.y);
+                            pk.h[2] = (bf16_t)(sum.z * normw_in.z);
+                            pk.h[3] = (bf16_t)(sum.w * normw_in.w);
+                            *reinterpret_cast<uint2*>(fz.x_out + (size_t)m * N + n) = pk.u;
+                            ss = fmaf(sum.x, sum.x, fmaf(sum.y, sum.y, fmaf(sum.z, sum.z, sum.w * sum.w)));
+                        }
+                        ss += __shfl_xor(ss, 16, 64);
+                        ss += __shfl_xor(ss, 32, 64);
+                        if (fg == 0 && nb0 + r < NB) fz.ss_out[(size_t)fr * fz.ss_out_stride + nb0 + r] = ss;
+                    } else if (m < M && n < N) {
+                        store4<TC>(C + (size_t)m * N + n, v, n, N, vec);
+                    }
                 }
         }
     }
 }
 
-template <int MT, int R, int UNROLL, int KSPLIT, int NSETS = 1, bool GLU = false, bool RING = false>
+template <int MT, int R, int UNROLL, int KSPLIT, int NSETS = 1, bool GLU = false, bool RING = false, int EPI = 0>
 static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
-                         int c_dtype, int n_out, hipStream_t s) {
+                         int c_dtype, int n_out, hipStream_t s, const SkinnyFuse* fuse = nullptr) {
     const int NB = (N + 15) / 16, KB = (K + 31) / 32;
     const int per_block = NSETS * R;
     const dim3 grid((NB + per_block - 1) / per_block);
+    const SkinnyFuse fz = fuse ? *fuse : SkinnyFuse{nullptr, 0, 0, 0.f, 0.f, nullptr, nullptr, nullptr, nullptr, 0};
     if (c_dtype == TFF_F32)
-        gemm_bf16_skinny_kernel<MT, R, UNROLL, KSPLIT, NSETS, GLU, float, RING>
-            <<<grid, 64 * KSPLIT * NSETS, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
+        gemm_bf16_skinny_kernel<MT, R, UNROLL, KSPLIT, NSETS, GLU, float, RING, EPI>
+            <<<grid, 64 * KSPLIT * NSETS, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out, fz);
+    else if constexpr (EPI != 2)
+        gemm_bf16_skinny_kernel<MT, R, UNROLL, KSPLIT, NSETS, GLU, bf16_t, RING, EPI>
+            <<<grid, 64 * KSPLIT * NSETS, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out, fz);
     else
-        gemm_bf16_skinny_kernel<MT, R, UNROLL, KSPLIT, NSETS, GLU, bf16_t, RING>
-            <<<grid, 64 * KSPLIT * NSETS, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
+        return tff_fail("gemm: the product before a norm has a float32 result");
     return tff_check_launch("gemm_bf16_skinny");
 }
 
@@ -514,6 +625,27 @@ TFF_API int tff_gemm_plan(int M, int N, int K, int glu, int keep_partials, int* 
     return 0;
 }
 
+// Up to 16 rows: which streaming kernel.  Gated: with a thousand row groups and more a wave takes
+// a group's whole K through a ring.  Plain: more waves per block where there are few blocks
+// (small N) or long rows (large K), fewer and deeper ones in between.
+template <int EPI>
+static int skinny_for(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda, int c_dtype,
+                      int glu_out, hipStream_t s, const SkinnyFuse* fuse) {
+    if (glu_out > 0) {
+        if constexpr (EPI != 2) {
+            if (N >= 16 * 1024)
+                return launch_skinny<1, 1, 8, 1, 2, true, true, EPI>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, fuse);
+            return launch_skinny<1, 1, 32, 4, 2, true, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, fuse);
+        } else {
+            return tff_fail("gemm: a gated product does not come before a norm");
+        }
+    }
+    if (N >= 32 * 1024) return launch_skinny<1, 1, 4, 8, 1, false, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, fuse);
+    if (K >= 8192 || N <= 4096)
+        return launch_skinny<1, 1, 4, 16, 1, false, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, fuse);
+    return launch_skinny<1, 1, 8, 4, 1, false, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, fuse);
+}
+
 // glu_out > 0: W holds gate and up groups in turn (N = 2 * ceil16(glu_out) rows) and C is
 // [M, glu_out] = silu(gate) * up.  workspace: room for partial sums (tff_gemm_workspace_bytes);
 // with less the blocks do not split K.
@@ -538,12 +670,7 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
     if (glu_out > 0) {
         TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
                     "gemm: a gated weight of %d rows does not fit %d output columns", N, glu_out);
-        if (M <= 16) {
-            // with a thousand row groups and more, a wave takes a group's whole K through a ring
-            if (N >= 16 * 1024)
-                return launch_skinny<1, 1, 8, 1, 2, true, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
-            return launch_skinny<1, 1, 32, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s);
-        }
+        if (M <= 16) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, nullptr);
         if (plan.tile == 64)
             return launch_async_g<2, 2, 2, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         if (plan.tile == 128 && plan.bn == 128)
@@ -552,13 +679,7 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
             return launch_async_g<2, 4, 4, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         return launch_async_g<4, 4, 4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
     }
-    if (M <= 16) {
-        // more waves per block where there are few blocks (small N) or long rows (large K),
-        // fewer and deeper ones in between
-        if (N >= 32 * 1024) return launch_skinny<1, 1, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
-        if (K >= 8192 || N <= 4096) return launch_skinny<1, 1, 4, 16>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
-        return launch_skinny<1, 1, 8, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
-    }
+    if (M <= 16) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, nullptr);
     if (plan.tile == 64) {
         // few columns and no room for partial sums: the streaming kernel, whose blocks split K
         // among their waves
@@ -573,6 +694,87 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
     if (plan.tile == 128)
         return launch_async_g<2, 4, 4, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     return launch_async_g<4, 4, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+}
+
+// ---- the norm between two products of up to 16 rows, taken into them ----
+static int check_fused_operands(const char* what, const void* A, const void* Wp, int M, int N, int K, int lda) {
+    TFF_REQUIRE(A && Wp, "%s: null pointer", what);
+    TFF_REQUIRE(M >= 1 && M <= 16 && N > 0 && K > 0 && lda >= K, "%s: bad sizes M=%d N=%d K=%d lda=%d (1 to 16 rows)",
+                what, M, N, K, lda);
+    TFF_REQUIRE(K % 8 == 0 && lda % 8 == 0, "%s: the inner size (K=%d, row stride %d) must be a multiple of 8", what,
+                K, lda);
+    TFF_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)Wp % 16) == 0, "%s: operands must be 16-byte aligned", what);
+    return 0;
+}
+
+// resid[M, N] += A . W^T (bfloat16 A and packed W, float32 sums); x_out[M, N] = bfloat16 of the new
+// resid times norm_w[N]; ss_out[m][g] (16 rows of ss_stride floats, ss_stride >= ceil(N / 16)) =
+// sum of squares of the new resid over columns 16 g .. 16 g + 15 of row m.  N a multiple of 8.
+TFF_API int tff_gemm_residual_prenorm(const void* A, const void* Wp, int M, int N, int K, int lda, float* resid,
+                                      const float* norm_w, void* x_out, float* ss_out, int ss_stride,
+                                      tff_stream_t stream) {
+    if (int rc = check_fused_operands("gemm_residual_prenorm", A, Wp, M, N, K, lda)) return rc;
+    TFF_REQUIRE(resid && norm_w && x_out && ss_out, "gemm_residual_prenorm: null pointer");
+    TFF_REQUIRE(N % 8 == 0 && ss_stride >= (N + 15) / 16, "gemm_residual_prenorm: N=%d must be a multiple of 8 and "
+                "ss_out needs %d floats a row, has %d", N, (N + 15) / 16, ss_stride);
+    TFF_REQUIRE(((uintptr_t)resid % 16) == 0 && ((uintptr_t)norm_w % 16) == 0 && ((uintptr_t)x_out % 8) == 0,
+                "gemm_residual_prenorm: operands must be 16-byte aligned");
+    SkinnyFuse fz{nullptr, 0, 0, 0.f, 0.f, resid, norm_w, (bf16_t*)x_out, ss_out, ss_stride};
+    return skinny_for<2>((const bf16_t*)A, (const bf16_t*)Wp, resid, M, N, K, lda, TFF_F32, 0, (hipStream_t)stream, &fz);
+}
+
+// C = rstd[m] * (A . W^T) with rstd[m] = rsqrt(sum_g ss[m][g] / dim + eps), g < ss_count: the product
+// after tff_gemm_residual_prenorm (A = its x_out, ss = its ss_out, dim = its N).  glu_out as in tff_gemm.
+TFF_API int tff_gemm_row_scaled(const void* A, const void* Wp, void* C, int M, int N, int K, int lda, int c_dtype,
+                                int glu_out, const float* ss, int ss_stride, int ss_count, int dim, float eps,
+                                tff_stream_t stream) {
+    if (int rc = check_fused_operands("gemm_row_scaled", A, Wp, M, N, K, lda)) return rc;
+    TFF_REQUIRE(C && ss && ((uintptr_t)C % 16) == 0 && ((uintptr_t)ss % 16) == 0, "gemm_row_scaled: null or unaligned pointer");
+    TFF_REQUIRE(c_dtype == TFF_F32 || c_dtype == TFF_BF16, "gemm_row_scaled: unknown output type %d", c_dtype);
+    TFF_REQUIRE(ss_count > 0 && ss_stride >= ss_count && ss_stride % 4 == 0 && dim > 0,
+                "gemm_row_scaled: %d sums of squares a row, %d apart (a multiple of 4), over %d elements", ss_count,
+                ss_stride, dim);
+    if (glu_out > 0)
+        TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
+                    "gemm_row_scaled: a gated weight of %d rows does not fit %d output columns", N, glu_out);
+    SkinnyFuse fz{ss, ss_stride, ss_count, 1.0f / (float)dim, eps, nullptr, nullptr, nullptr, nullptr, 0};
+    return skinny_for<1>((const bf16_t*)A, (const bf16_t*)Wp, C, M, N, K, lda, c_dtype, glu_out, (hipStream_t)stream, &fz);
+}
+
+// out[m, :] = bfloat16(x[m, :] * rstd[m]): what tff_gemm_row_scaled's A stands for, written out
+// (for a consumer that is no such product).
+__global__ __launch_bounds__(256) void scale_rows_kernel(const bf16_t* __restrict__ x, const float* __restrict__ ss,
+                                                         int ss_stride, int ss_count, float inv_dim, float eps,
+                                                         bf16_t* __restrict__ out, int N) {
+    __shared__ float red[8];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    // the same order of additions as in the product's prologue
+    float s4[4] = {0.f, 0.f, 0.f, 0.f};
+    if (tid < 4) {
+        const float* sp = ss + (size_t)m * ss_stride;
+        const int vec_end = ss_count & ~3;
+        for (int j = tid * 4; j < vec_end; j += 16) {
+            const float4 v = *reinterpret_cast<const float4*>(sp + j);
+            s4[0] += (v.x + v.y) + (v.z + v.w);
+        }
+        if (tid == 0)
+            for (int j = vec_end; j < ss_count; ++j) s4[0] += sp[j];
+        red[tid] = s4[0];
+    }
+    __syncthreads();
+    const float ssum = (red[0] + red[1]) + (red[2] + red[3]);
+    const float r = rsqrtf(ssum * inv_dim + eps);
+    for (int j = tid; j < N; j += blockDim.x) out[(size_t)m * N + j] = (bf16_t)((float)x[(size_t)m * N + j] * r);
+}
+
+TFF_API int tff_scale_rows(const void* x, const float* ss, int ss_stride, int ss_count, int dim, float eps, void* out,
+                           int M, int N, tff_stream_t stream) {
+    TFF_REQUIRE(x && ss && out && M >= 0 && M <= 16 && N > 0 && ss_count > 0 && ss_stride >= ss_count && dim > 0,
+                "scale_rows: bad operands (M=%d N=%d)", M, N);
+    if (M == 0) return 0;
+    scale_rows_kernel<<<M, 256, 0, (hipStream_t)stream>>>((const bf16_t*)x, ss, ss_stride, ss_count, 1.0f / (float)dim,
+                                                         eps, (bf16_t*)out, N);
+    return tff_check_launch("scale_rows");
 }
 
 int tff_gemm_f32(const float* A, const float* W, void* C, int M, int N, int K, int lda,

@@ -154,18 +154,93 @@ def embed(table, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Te
     return out
 
 
-def add_rmsnorm(resid: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, eps: float,
+class PendingProduct:
+    """A product ``x . weight^T`` of up to 16 bfloat16 rows that ``linear`` was
+    asked for with ``partials=True`` and has not run: ``add_rmsnorm`` runs it
+    with the residual sum and the norm's weight in its epilogue when the norm's
+    result goes to another such product, and plainly (:meth:`run`) otherwise."""
+
+    def __init__(self, x: torch.Tensor, weight: "PackedWeight"):
+        self.x, self.weight = x, weight
+        self.shape = (x.shape[0], weight.shape[0])
+        self.device = x.device
+
+    def run(self) -> torch.Tensor:
+        return linear(self.x, self.weight, out_dtype=torch.float32)
+
+
+class ScaledRows:
+    """The result of an RMS norm whose per-row factor has not been applied:
+    ``x`` [M, H] bfloat16 = (residual stream) * (norm weight), and the sums of
+    squares of every row's groups of 16 columns, ``ss`` [16, stride] float32
+    (``count`` of them a row).  ``linear`` applies rsqrt(sum / H + eps) to its
+    accumulators; :meth:`materialize` writes the normalised rows out."""
+
+    def __init__(self, x: torch.Tensor, ss: torch.Tensor, count: int, eps: float):
+        self.x, self.ss, self.count, self.eps = x, ss, int(count), float(eps)
+        self.shape, self.dtype, self.device = x.shape, x.dtype, x.device
+
+    def materialize(self) -> torch.Tensor:
+        M, H = self.x.shape
+        out = torch.empty_like(self.x)
+        L = _lib.load()
+        _lib.check(L.tff_scale_rows(self.x.data_ptr(), self.ss.data_ptr(), self.ss.stride(0), self.count, H,
+                                    self.eps, out.data_ptr(), M, H, _stream()))
+        return out
+
+
+def as_tensor(t) -> torch.Tensor:
+    """Whatever ``linear`` or ``add_rmsnorm`` returned, as a plain tensor: a
+    product that has not run is run, partial sums [S, T, H] are added up in
+    order, rows that lack their norm's factor get it."""
+    if isinstance(t, PendingProduct):
+        return t.run()
+    if isinstance(t, ScaledRows):
+        return t.materialize()
+    if isinstance(t, torch.Tensor) and t.dim() == 3:
+        acc = t[0].clone()
+        for part in t[1:]:
+            acc += part
+        return acc
+    return t
+
+
+def _fused_prenorm(p: PendingProduct, resid: torch.Tensor, weight: torch.Tensor, eps: float) -> ScaledRows:
+    x = p.x
+    M, K = x.shape
+    N = p.weight.shape[0]
+    lda = x.stride(0) if M > 1 else K
+    groups = -(-N // 16)
+    stride = -(-groups // 4) * 4
+    xs = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+    ss = torch.empty(16, stride, dtype=torch.float32, device=x.device)
+    L = _lib.load()
+    _lib.check(L.tff_gemm_residual_prenorm(x.data_ptr(), p.weight.data_ptr(), M, N, K, lda, resid.data_ptr(),
+                                           weight.data_ptr(), xs.data_ptr(), ss.data_ptr(), stride, _stream()))
+    return ScaledRows(xs, ss, groups, eps)
+
+
+def add_rmsnorm(resid: torch.Tensor, delta, weight: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: torch.Tensor | None = None,
-                out: torch.Tensor | None = None) -> torch.Tensor:
+                out: torch.Tensor | None = None, for_linear: bool = False):
     """``resid += delta`` (when given and ``rows`` is None) and the RMS norm of
     the sum; with ``rows`` the norm of those rows only, ``resid`` untouched.
-    ``delta`` may be a stack [S, T, H] of partial sums (``linear`` with
-    ``partials=True``): they are added up first, in order."""
+    ``delta`` may be what ``linear`` returns with ``partials=True``: a stack
+    [S, T, H] of partial sums, which are added up first, in order, or a
+    product that has not run.  ``for_linear``: the result goes to ``linear``
+    and nowhere else, so it may be a :class:`ScaledRows`."""
     _req(resid, "add_rmsnorm resid", torch.float32, 2)
     H = resid.shape[1]
     _req(weight, "add_rmsnorm weight", torch.float32, 1)
     if weight.numel() != H:
         raise _lib.KernelError(f"add_rmsnorm: weight has {weight.numel()} elements, rows have {H}")
+    if isinstance(delta, PendingProduct):
+        if tuple(delta.shape) != tuple(resid.shape):
+            raise _lib.KernelError(
+                f"add_rmsnorm: delta {tuple(delta.shape)} does not match resid {tuple(resid.shape)}")
+        if for_linear and rows is None and out is None and out_dtype == torch.bfloat16:
+            return _fused_prenorm(delta, resid, weight, eps)
+        delta = delta.run()
     planes, plane = 1, 0
     if delta is not None:
         _req(delta, "add_rmsnorm delta", torch.float32, 3 if delta.dim() == 3 else 2)
@@ -214,9 +289,13 @@ def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
     blocks, the partial sums are returned as they are, [S, M, N], for a
     consumer that adds them up anyway (``add_rmsnorm``); else the result is
     [M, N] as always."""
+    packed = isinstance(weight, PackedWeight)
+    if isinstance(x, ScaledRows):
+        if packed and out is None and not partials and x.shape[1] == weight.shape[1]:
+            return _linear_row_scaled(x, weight, out_dtype or x.dtype)
+        x = x.materialize()
     if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
         raise _lib.KernelError("linear x: expected a GPU matrix with unit inner stride")
-    packed = isinstance(weight, PackedWeight)
     if packed:
         _req(weight.data, "linear weight", x.dtype, 1)
     else:
@@ -236,6 +315,8 @@ def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
     L = _lib.load()
     # some shapes (few columns for the rows) split K over blocks and need room for partial sums
     want = bool(partials and packed and out is None and out_dtype == torch.float32 and not glu_out)
+    if want and M <= 16 and N % 8 == 0 and x.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0 and lda % 8 == 0:
+        return PendingProduct(x, weight)   # a few rows: the consumer runs it with its own work in the epilogue
     ws_bytes = (L.tff_gemm_workspace_bytes(M, N, K, dtype_code(x.dtype), 1 if glu_out else 0, 1 if want else 0)
                 if packed else 0)
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=x.device) if ws_bytes else None
@@ -251,6 +332,18 @@ def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
     _lib.check(L.tff_gemm(x.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K, lda,
                           dtype_code(x.dtype), dtype_code(out_dtype), 1 if packed else 0, glu_out,
                           _ptr(ws), ws_bytes, 1 if keep else 0, _stream()))
+    return out
+
+
+def _linear_row_scaled(x: ScaledRows, weight: "PackedWeight", out_dtype: torch.dtype) -> torch.Tensor:
+    M, K = x.shape
+    N = weight.shape[0]
+    glu_out = weight.glu_out
+    out = torch.empty(M, glu_out or N, dtype=out_dtype, device=x.device)
+    L = _lib.load()
+    _lib.check(L.tff_gemm_row_scaled(x.x.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K, K,
+                                     dtype_code(out_dtype), glu_out, x.ss.data_ptr(), x.ss.stride(0), x.count, K,
+                                     x.eps, _stream()))
     return out
 
 
@@ -707,6 +800,7 @@ OP_TABLE = {
     "add_rmsnorm": add_rmsnorm,
     "rmsnorm": rmsnorm,
     "linear": linear,
+    "as_tensor": as_tensor,
     "pack_weight": pack_weight,
     "qk_norm_rope_kv": qk_norm_rope_kv,
     "attention": paged_attention,

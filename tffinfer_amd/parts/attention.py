@@ -27,6 +27,8 @@ class GQAttention(Mixer):
     """
 
     graph_safe = True
+    #: the input is used by ``ops.linear`` and by nothing else
+    input_goes_to_linear = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position, qk_norm_eps: float | None = 1e-6, window: int = 0,

@@ -90,9 +90,14 @@ class Norm(Part):
         """Adds ``delta`` into the float32 residual stream ``resid`` (when
         ``rows`` is None) and returns the norm of the sum in the activation
         type; with ``rows`` returns the norm of those rows only.  ``delta`` is
-        what a mixer or feed-forward returned: [T, hidden], or a stack
-        [S, T, hidden] of partial sums to be added up (``ops.add_rmsnorm``
-        takes both)."""
+        what a mixer or feed-forward returned: [T, hidden], or what
+        ``ops.linear(..., partials=True)`` gave it: a stack [S, T, hidden] of
+        partial sums to be added up or a product that has not run yet
+        (``ops.add_rmsnorm`` takes all three; ``ops.as_tensor`` turns them into
+        a tensor for a norm of another kind).  A norm whose class says
+        ``for_linear_aware = True`` also takes ``for_linear``: the caller
+        promises that the result goes to ``ops.linear`` only, so it may be rows
+        that still lack the norm's per-row factor (``ops.ScaledRows``)."""
         raise NotImplementedError
 
 
@@ -107,15 +112,19 @@ class Mixer(Part):
 
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
         """x [T, hidden] in the activation type -> float32 [T, hidden] to be
-        added to the residual stream (or [S, T, hidden], whose sum over S is:
-        what ``ops.linear(..., partials=True)`` returns)."""
+        added to the residual stream, or what ``ops.linear(..., partials=True)``
+        returns in its place for the norm that follows (``ops.as_tensor`` makes
+        a tensor of it).  A mixer whose class says ``input_goes_to_linear =
+        True`` hands ``x`` to ``ops.linear`` and to nothing else; it may then
+        get rows that still lack their norm's factor."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
-        """x [T, hidden] in the activation type -> float32 [T, hidden] (or a
-        stack of partial sums [S, T, hidden], as for a mixer)."""
+        """x [T, hidden] in the activation type -> float32 [T, hidden] (or what
+        ``ops.linear(..., partials=True)`` returns, as for a mixer;
+        ``input_goes_to_linear`` as there)."""
         raise NotImplementedError
 
 

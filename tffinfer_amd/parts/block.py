@@ -27,8 +27,15 @@ class PreNormBlock(Block):
         return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2,
                 "feed_forward": self.feed_forward}
 
+    @staticmethod
+    def _norm(norm, consumer, ctx, resid, pending):
+        # a norm and a consumer that both say so may pass rows that still lack the norm's factor
+        if getattr(norm, "for_linear_aware", False) and getattr(consumer, "input_goes_to_linear", False):
+            return norm.forward(ctx, resid, pending, for_linear=True)
+        return norm.forward(ctx, resid, pending)
+
     def forward(self, ctx, resid, pending):
-        h = self.norm1.forward(ctx, resid, pending)
+        h = self._norm(self.norm1, self.mixer, ctx, resid, pending)
         a = self.mixer.forward(ctx, h)
-        z = self.norm2.forward(ctx, resid, a)
+        z = self._norm(self.norm2, self.feed_forward, ctx, resid, a)
         return self.feed_forward.forward(ctx, z)

@@ -16,6 +16,8 @@ class SwiGLU(FeedForward):
     """
 
     graph_safe = True
+    #: the input is used by ``ops.linear`` and by nothing else
+    input_goes_to_linear = True
 
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size = int(hidden_size)

@@ -27,5 +27,10 @@ class RMSNorm(Norm):
         # norm weights stay in float32 whatever the activation type is
         self.weight = weights["weight"].to(torch.float32).contiguous().to(device)
 
-    def forward(self, ctx, resid, delta, rows=None):
-        return ctx.ops.add_rmsnorm(resid, delta, self.weight, self.eps, ctx.act_dtype, rows=rows)
+    #: ``forward`` takes ``for_linear``: its result may then be rows that lack the norm's factor,
+    #: which only ``ops.linear`` understands
+    for_linear_aware = True
+
+    def forward(self, ctx, resid, delta, rows=None, for_linear=False):
+        return ctx.ops.add_rmsnorm(resid, delta, self.weight, self.eps, ctx.act_dtype, rows=rows,
+                                   for_linear=for_linear)
