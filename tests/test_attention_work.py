@@ -25,7 +25,8 @@ def test_every_item_once_and_even_loads(bins, window):
     entries = [(0, 2048), (333, 200), (5, 1), (1000, 130), (0, 37)]
     G, cols = 4, 128
     batch = _batch(entries)
-    items, starts, blocks = _attention_block_work(batch, G, 8, window, "cpu", cols, bins=bins)
+    items, starts, blocks, groups = _attention_block_work(batch, G, 8, window, "cpu", cols, bins=bins)
+    assert groups in (1, 2)
     items, starts = items.tolist(), starts.tolist()
     want = sorted((r, c0) for r, (P, n) in enumerate(entries) for c0 in range(0, n * G, cols))
     assert sorted(map(tuple, items)) == want                      # no item lost, none twice
@@ -45,7 +46,25 @@ def test_entry_filters():
     from tffinfer_amd.kernels.ops import _attention_block_work, _attention_work, _entries
     batch = _batch([(900, 1), (0, 300), (40, 1), (333, 150)])
     assert _entries(batch, "single") == [0, 2] and _entries(batch, "multi") == [1, 3]
-    items, starts, blocks = _attention_block_work(batch, 4, 2, 0, "cpu", 128, bins=64, which="multi")
+    items, starts, blocks, _ = _attention_block_work(batch, 4, 2, 0, "cpu", 128, bins=64, which="multi")
     assert {r for r, _ in items.tolist()} == {1, 3}
     single = _attention_work(batch, 20, 16, "cpu", "single").tolist()     # 20 heads to a kv head: two tiles
     assert single == [[0, 0], [0, 16], [2, 0], [2, 16]]
+
+
+def test_key_groups_and_blocks_follow_the_amount_of_work():
+    """Little work: one block a CU, two groups of waves in it that share an item's slices; plenty:
+    two blocks of one group a CU; large heads always one group, one block a CU."""
+    from tffinfer_amd.kernels.ops import _attention_block_work
+    short, long_ = _batch([(0, 2048)]), _batch([(0, 8192)])
+    _, _, blocks, groups = _attention_block_work(short, 4, 8, 0, "cpu", num_cus=256)
+    assert (blocks, groups) == (32, 2)
+    _, _, blocks, groups = _attention_block_work(long_, 4, 8, 0, "cpu", num_cus=256)
+    assert (blocks, groups) == (64, 1)
+    _, _, blocks, groups = _attention_block_work(long_, 4, 8, 0, "cpu", num_cus=256, head_dim=256)
+    assert (blocks, groups) == (32, 1)
+    _, _, blocks, groups = _attention_block_work(long_, 4, 8, 0, "cpu", num_cus=256, key_groups=2)
+    assert (blocks, groups) == (32, 2)
+    # a portion of 2,048 tokens late in a long context is plenty of work as well
+    _, _, blocks, groups = _attention_block_work(_batch([(6144, 2048)]), 4, 8, 0, "cpu", num_cus=256)
+    assert (blocks, groups) == (64, 1)

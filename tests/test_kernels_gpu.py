@@ -536,11 +536,11 @@ def test_attention_mfma_prompt_portions_and_mixed(nq, nkv, d, ps, window):
     _close(gen.reshape(T, nq, d), ref, 1.5e-2, "generic attention on the same step")
 
 
-@pytest.mark.parametrize("bins", [None, 3, 1])
+@pytest.mark.parametrize("bins,groups", [(None, None), (3, 2), (1, 2), (None, 1), (3, 1), (1, 1)])
 @pytest.mark.parametrize("nq,nkv,d,ps,window", [
     (32, 8, 128, 16, 0), (8, 2, 32, 8, 300), (6, 3, 48, 8, 0), (5, 1, 128, 32, 0), (40, 2, 96, 8, 77),
     (4, 2, 16, 16, 0), (3, 1, 256, 64, 0)])
-def test_attention_mfma_long_portions(nq, nkv, d, ps, window, bins):
+def test_attention_mfma_long_portions(nq, nkv, d, ps, window, bins, groups):
     """Portions long enough for the kernel whose blocks share keys through LDS:
     several blocks per request, a cached prefix, windows that start mid-page."""
     ops = _ops()
@@ -551,7 +551,9 @@ def test_attention_mfma_long_portions(nq, nkv, d, ps, window, bins):
     q = torch.randn(T, nq, d, generator=g).to(torch.bfloat16)
     scale = 1 / math.sqrt(d)
     # bins: with fewer blocks than runs of 128 columns a block works through several runs in turn
-    out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale, block_bins=bins)
+    # groups: a block of two groups of waves that take every other slice, or of one
+    out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale, block_bins=bins,
+                             key_groups=groups)
     # the general kernel is the yardstick here (it is checked against float64 above)
     gen = ops.attention_generic(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv.k_cache, kv.v_cache, kv.block_tables,
                                 batch.token_req, batch.positions, window, scale)

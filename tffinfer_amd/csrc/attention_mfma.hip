@@ -953,17 +953,25 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
                        const int32_t* work, int num_work, const int32_t* block_items, int num_blocks,
                        int tiles_per_entry, int cols_per_wave,
                        int splits, int nq, int nkv, int page_size, int window, float scale,
-                       int T_total, hipStream_t s, const AttnFuse* fuse = nullptr) {
+                       int T_total, hipStream_t s, const AttnFuse* fuse = nullptr, int key_groups = 2) {
     int page_shift = -1;
     if ((page_size & (page_size - 1)) == 0)
         for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
     if (cols_per_wave == 128) {   // blocks of eight waves that share their keys through LDS
-        // two groups of eight waves that take every other slice, where LDS holds their stages
-        if constexpr (DT <= 8)
-            attn_mfma_block_kernel<DT, 1, 8, 2><<<dim3(num_blocks, nkv), 1024, 0, s>>>(
-                q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
-                block_items, nq, nkv, page_size, page_shift, window, scale);
-        else
+        // Two groups of eight waves that take every other slice, where LDS holds their stages:
+        // half as many slices one after the other for a block, which is what counts when there
+        // is little work for the machine; with plenty of it, blocks of one group, two to a CU,
+        // spend less on merging and waiting for each other.
+        if constexpr (DT <= 8) {
+            if (key_groups == 2)
+                attn_mfma_block_kernel<DT, 1, 8, 2><<<dim3(num_blocks, nkv), 1024, 0, s>>>(
+                    q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
+                    block_items, nq, nkv, page_size, page_shift, window, scale);
+            else
+                attn_mfma_block_kernel<DT, 1, 8, 1><<<dim3(num_blocks, nkv), 512, 0, s>>>(
+                    q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
+                    block_items, nq, nkv, page_size, page_shift, window, scale);
+        } else
             attn_mfma_block_kernel<DT, 1, 8, 1><<<dim3(num_blocks, nkv), 512, 0, s>>>(
                 q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
                 block_items, nq, nkv, page_size, page_shift, window, scale);
@@ -1006,11 +1014,12 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                const int32_t* block_tables, int bt_stride, const int32_t* cu_tokens,
                                const int32_t* start_pos, const int32_t* work, int num_work,
                                const int32_t* block_items, int num_blocks,
-                               int tiles_per_entry, int cols_per_wave, int splits, int T_total,
+                               int tiles_per_entry, int cols_per_wave, int key_groups, int splits, int T_total,
                                int nq, int nkv, int d, int page_size, int num_pages, int window,
                                float scale, tff_stream_t stream) {
     TFF_REQUIRE(q && out && k_cache && v_cache && block_tables && cu_tokens && start_pos,
                 "attention_mfma: null pointer");
+    TFF_REQUIRE(key_groups == 1 || key_groups == 2, "attention_mfma: %d key groups (1 or 2)", key_groups);
     TFF_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0,
                 "attention_mfma: %d query heads are not a multiple of %d key heads", nq, nkv);
     TFF_REQUIRE(tff_attention_mfma_supported(d, page_size),
@@ -1042,7 +1051,8 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                 (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,       \
                                 bt_stride, cu_tokens, start_pos, work, num_work, block_items,       \
                                 num_blocks, tiles_per_entry,                                        \
-                                cols_per_wave, splits, nq, nkv, page_size, window, scale, T_total, s);
+                                cols_per_wave, splits, nq, nkv, page_size, window, scale, T_total, s, \
+                                nullptr, key_groups);
     switch (d) {
         TFF_ATTN_CASE(1) TFF_ATTN_CASE(2) TFF_ATTN_CASE(3) TFF_ATTN_CASE(4) TFF_ATTN_CASE(5)
         TFF_ATTN_CASE(6) TFF_ATTN_CASE(7) TFF_ATTN_CASE(8) TFF_ATTN_CASE(12) TFF_ATTN_CASE(16)

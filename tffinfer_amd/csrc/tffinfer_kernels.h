@@ -119,7 +119,8 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out,
 // number of entries) tff_attention_split_reduce merges.  cols_per_wave 128: work items
 // are runs of 128 columns for a block of eight waves that stages keys and
 // values in LDS; block b works through items block_items[b] ..
-// block_items[b + 1] of the work table (block_items null: item b).  Head sizes 16..128 in steps of
+// block_items[b + 1] of the work table (block_items null: item b); key_groups 2 (head sizes
+// up to 128): a block is two groups of eight waves that take every other slice, 1: one group.  Head sizes 16..128 in steps of
 // 16, 192 and 256; pages a multiple of 8; values transposed in their pages.
 TFF_API int tff_attention_mfma_supported(int d, int page_size);
 TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* part_o, float* part_ml,
@@ -127,7 +128,7 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                const int32_t* block_tables, int bt_stride, const int32_t* cu_tokens,
                                const int32_t* start_pos, const int32_t* work, int num_work,
                                const int32_t* block_items, int num_blocks,
-                               int tiles_per_entry, int cols_per_wave, int splits, int T_total,
+                               int tiles_per_entry, int cols_per_wave, int key_groups, int splits, int T_total,
                                int nq, int nkv, int d, int page_size, int num_pages, int window,
                                float scale, tff_stream_t stream);
 // Decoding steps (every entry brings one token), bfloat16, from the fused projection's output:

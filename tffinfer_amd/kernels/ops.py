@@ -459,19 +459,20 @@ def _num_cus(device) -> int:
 
 
 def _attention_block_work(batch, G: int, nkv: int, window: int, device, cols: int = 128,
-                          bins: int | None = None, which: str = "all"):
+                          bins: int | None = None, which: str = "all", key_groups: int | None = None,
+                          head_dim: int = 128, num_cus: int | None = None):
     """Work table of the block kernel: items (entry, first column) of ``cols``
     columns, dealt to blocks so that every block goes through about the same
     number of 32-key slices (an item late in a long prompt sees many times the
     keys of an early one).  There are at most as many blocks as the device
-    can hold at once, so none waits for another to end.  Returns (items
-    [n, 2], block_items [blocks + 1], blocks)."""
+    can hold at once, so none waits for another to end: with little work one
+    block a CU whose two groups of waves share an item's slices, with plenty
+    (some 96 slices a block and more) two blocks of one group a CU.  Returns
+    (items [n, 2], block_items [blocks + 1], blocks, key groups)."""
     cache = getattr(batch, "_attn_work", None)
     if cache is None:
         cache = batch._attn_work = {}
-    if bins is None:
-        bins = max(1, _num_cus(device) // max(1, nkv))
-    key = ("blocks", G, nkv, cols, window, bins, which)
+    key = ("blocks", G, nkv, cols, window, bins, which, key_groups, head_dim, num_cus)
     if key not in cache:
         cu, P = batch.host_cu_tokens, batch.host_start_pos
         items = []                       # (slices, entry, first column)
@@ -482,15 +483,26 @@ def _attention_block_work(batch, G: int, nkv: int, window: int, device, cols: in
                 last = P[r] + (min(c0 + cols, ncols) - 1) // G
                 lo = max(0, first - window + 1) if window > 0 else 0
                 items.append((last // 32 - lo // 32 + 1, r, c0))
-        if len(items) <= bins:
+        if num_cus is None:
+            num_cus = _num_cus(device) if torch.device(device).type == "cuda" else 256
+        per_cu = max(1, num_cus // max(1, nkv))
+        groups = key_groups
+        if groups is None:
+            groups = 2
+            if head_dim <= 128 and sum(it[0] for it in items) >= 96 * 2 * per_cu:
+                groups = 1
+        if head_dim > 128:
+            groups = 1                   # LDS holds one group's stages there
+        nbins = bins if bins is not None else (per_cu if groups == 2 or head_dim > 128 else 2 * per_cu)
+        if len(items) <= nbins:
             order = sorted(items, reverse=True)        # the longest start first
             starts = list(range(len(order) + 1))
         else:
             # longest first, each to the block with the least to do so far
             import heapq
-            loads = [(0, b) for b in range(bins)]
+            loads = [(0, b) for b in range(nbins)]
             heapq.heapify(loads)
-            per_bin = [[] for _ in range(bins)]
+            per_bin = [[] for _ in range(nbins)]
             for it in sorted(items, reverse=True):
                 load, b = heapq.heappop(loads)
                 per_bin[b].append(it)
@@ -501,7 +513,7 @@ def _attention_block_work(batch, G: int, nkv: int, window: int, device, cols: in
                 starts.append(len(order))
         flat = [x for it in order for x in it[1:]]
         cache[key] = (torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(device),
-                      torch.tensor(starts, dtype=torch.int32).to(device), len(starts) - 1)
+                      torch.tensor(starts, dtype=torch.int32).to(device), len(starts) - 1, groups)
     return cache[key]
 
 
@@ -514,11 +526,12 @@ def pick_splits(waves: int, max_context: int) -> int:
 
 def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,
                    scale: float | None = None, splits: int | None = None,
-                   block_bins: int | None = None) -> torch.Tensor:
+                   block_bins: int | None = None, key_groups: int | None = None) -> torch.Tensor:
     """bfloat16 attention of the step's tokens on the matrix cores; decode-only
     steps split each request's keys over several waves and merge them.
-    ``splits`` and ``block_bins`` (blocks per kv head that share the work of
-    long portions) override the choices made from the step's sizes."""
+    ``splits``, ``block_bins`` (blocks per kv head that share the work of
+    long portions) and ``key_groups`` (groups of waves in such a block)
+    override the choices made from the step's sizes."""
     _req(q, "attention q", torch.bfloat16, 2)
     T = q.shape[0]
     if q.shape[1] < nq * d:
@@ -542,7 +555,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
     L = _lib.load()
     stream = _stream()
 
-    def launch(work, num_work, block_items, num_blocks, tiles, cols, splits, rows=None):
+    def launch(work, num_work, block_items, num_blocks, tiles, cols, splits, rows=None, groups=2):
         # partial results of split keys are kept by entry (split entries bring one token each)
         part_o = part_ml = None
         if splits > 1:
@@ -552,7 +565,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
             q.data_ptr(), q.stride(0), out.data_ptr(), _ptr(part_o), _ptr(part_ml), k_cache.data_ptr(),
             v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(),
             batch.start_pos.data_ptr(), _ptr(work), num_work, _ptr(block_items), num_blocks, tiles, cols,
-            splits, R if splits > 1 else T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window),
+            groups, splits, R if splits > 1 else T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window),
             float(scale), stream))
         if splits > 1:
             _lib.check(L.tff_attention_split_reduce(
@@ -583,9 +596,9 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
         sp = splits if splits is not None else pick_splits(work.shape[0] * nkv, batch.max_context)
         launch(work, work.shape[0], None, 0, 1, 16, sp, cache["single_rows"])
     if cols == 128:
-        work, block_items, num_blocks = _attention_block_work(batch, G, nkv, int(window), q.device,
-                                                              bins=block_bins, which=which)
-        launch(work, work.shape[0], block_items, num_blocks, 1, 128, 1)
+        work, block_items, num_blocks, groups = _attention_block_work(
+            batch, G, nkv, int(window), q.device, bins=block_bins, which=which, key_groups=key_groups, head_dim=d)
+        launch(work, work.shape[0], block_items, num_blocks, 1, 128, 1, groups=groups)
     else:
         work = _attention_work(batch, G, cols, q.device)
         launch(work, work.shape[0], None, 0, 1, cols, 1)
