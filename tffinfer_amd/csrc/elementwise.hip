@@ -110,17 +110,24 @@ __device__ __forceinline__ void store_out4<bf16_t>(bf16_t* o, float4 v) {
     *reinterpret_cast<uint2*>(o) = pk.u;
 }
 
+// planes are added in their order; four loads are in flight at a time
 __device__ __forceinline__ float4 delta_sum4(const float4* d4, int j, int planes, size_t plane4) {
     float4 d = d4[j];
-    for (int p = 1; p < planes; ++p) {
-        const float4 e = d4[p * plane4 + j];
-        d.x += e.x; d.y += e.y; d.z += e.z; d.w += e.w;
+    for (int p = 1; p < planes; p += 4) {
+        float4 e[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            e[u] = p + u < planes ? d4[(size_t)(p + u) * plane4 + j] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (p + u < planes) { d.x += e[u].x; d.y += e[u].y; d.z += e[u].z; d.w += e[u].w; }
     }
     return d;
 }
 
-template <typename TO>
-__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid,
+// NT threads a row: 256, or 1024 where there are few rows (more loads in flight for each)
+template <typename TO, int NT>
+__global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__ resid,
                                                                const float* __restrict__ delta,
                                                                int planes, size_t plane,
                                                                const float* __restrict__ w, float eps,
@@ -135,11 +142,12 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     const float4* d4 = delta ? reinterpret_cast<const float4*>(delta + (size_t)r * H) : nullptr;
     const float4* w4 = reinterpret_cast<const float4*>(w);
     const bool store = rows == nullptr && d4 != nullptr;
-    float4 cache[4];
+    constexpr int ITS = 1024 / NT;
+    float4 cache[ITS];
     float ss = 0.f;
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
-        const int j = tid + it * 256;
+    for (int it = 0; it < ITS; ++it) {
+        const int j = tid + it * NT;
         if (j < H4) {
             float4 v = x4[j];
             if (d4) { const float4 dv = delta_sum4(d4, j, planes, plane4); v.x += dv.x; v.y += dv.y; v.z += dv.z; v.w += dv.w; }
@@ -148,7 +156,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
             ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
         }
     }
-    for (int j = tid + 1024; j < H4; j += 256) {
+    for (int j = tid + 1024; j < H4; j += NT) {
         float4 v = x4[j];
         if (d4) { const float4 dv = delta_sum4(d4, j, planes, plane4); v.x += dv.x; v.y += dv.y; v.z += dv.z; v.w += dv.w; }
         if (store) x4[j] = v;
@@ -158,14 +166,14 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     const float rr = rsqrtf(ss / (float)H + eps);
     TO* o = out + (size_t)i * H;
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
-        const int j = tid + it * 256;
+    for (int it = 0; it < ITS; ++it) {
+        const int j = tid + it * NT;
         if (j < H4) {
             const float4 v = cache[it], wv = w4[j];
             store_out4<TO>(o + 4 * j, make_float4(v.x * rr * wv.x, v.y * rr * wv.y, v.z * rr * wv.z, v.w * rr * wv.w));
         }
     }
-    for (int j = tid + 1024; j < H4; j += 256) {
+    for (int j = tid + 1024; j < H4; j += NT) {
         float4 v = x4[j];
         if (d4 && !store) { const float4 dv = delta_sum4(d4, j, planes, plane4); v.x += dv.x; v.y += dv.y; v.z += dv.z; v.w += dv.w; }
         const float4 wv = w4[j];
@@ -188,10 +196,14 @@ TFF_API int tff_add_rmsnorm(float* resid, const float* delta, int delta_planes, 
     const bool vec = H % 4 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)weight % 16) == 0 &&
                      ((uintptr_t)out % 16) == 0 && (!delta || ((uintptr_t)delta % 16) == 0);
     if (vec) {
-        if (out_dtype == TFF_F32)
-            add_rmsnorm_vec_kernel<float><<<n, 256, 0, s>>>(resid, delta, planes, plane, weight, eps, (float*)out, rows, H);
-        else
-            add_rmsnorm_vec_kernel<bf16_t><<<n, 256, 0, s>>>(resid, delta, planes, plane, weight, eps, (bf16_t*)out, rows, H);
+        const bool wide = n <= 128 && H >= 2048;
+        if (out_dtype == TFF_F32) {
+            if (wide) add_rmsnorm_vec_kernel<float, 1024><<<n, 1024, 0, s>>>(resid, delta, planes, plane, weight, eps, (float*)out, rows, H);
+            else add_rmsnorm_vec_kernel<float, 256><<<n, 256, 0, s>>>(resid, delta, planes, plane, weight, eps, (float*)out, rows, H);
+        } else {
+            if (wide) add_rmsnorm_vec_kernel<bf16_t, 1024><<<n, 1024, 0, s>>>(resid, delta, planes, plane, weight, eps, (bf16_t*)out, rows, H);
+            else add_rmsnorm_vec_kernel<bf16_t, 256><<<n, 256, 0, s>>>(resid, delta, planes, plane, weight, eps, (bf16_t*)out, rows, H);
+        }
         return tff_check_launch("add_rmsnorm");
     }
     const int threads = H >= 2048 ? 1024 : 256;
