@@ -187,6 +187,46 @@ def test_norm_taken_into_the_products_on_either_side(M, H, K, N2, glu):
     assert isinstance(z3, torch.Tensor) and torch.equal(z3, z) and torch.equal(r3, r2)
 
 
+@pytest.mark.parametrize("M,N,K,glu", [(2000, 8100, 328, False), (1500, 8000, 1096, False), (2048, 4096, 12288, False),
+                                         (2000, 16160, 328, True), (1024, 16000, 328, False)])
+def test_linear_on_the_largest_tile(M, N, K, glu):
+    """Shapes for which the plan takes 256 x 256 tiles: an odd number of
+    32-k steps, a last step that is not whole, rows and columns that do not fill the tiles, K
+    split over blocks with the partial sums added or handed on.  The float32 product of the
+    same (bfloat16) numbers is the yardstick."""
+    import ctypes
+    from tffinfer_amd.kernels import lib
+    ops = _ops()
+    L = lib.load()
+    g = torch.Generator().manual_seed(N)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    r, c, sp = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    if glu:
+        I = N // 2
+        gate = (torch.randn(I, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+        up = (torch.randn(I, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+        assert L.tff_gemm_plan(M, 2 * I, K, 1, 0, ctypes.byref(r), ctypes.byref(c), ctypes.byref(sp)) == 0
+        assert (r.value, c.value) == (256, 256)
+        y = ops.linear(x, ops.pack_gate_up(gate, up), out_dtype=torch.float32)
+        a, b = ops.linear(x.float(), gate.float()), ops.linear(x.float(), up.float())
+        ref = a / (1 + torch.exp(-a)) * b
+        _close(y, ref, 3e-5, "gated product")
+        return
+    w = (torch.randn(N, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+    pw = ops.pack_weight(w)
+    ref = ops.linear(x.float(), w.float())
+    for keep in (0, 1):
+        assert L.tff_gemm_plan(M, N, K, 0, keep, ctypes.byref(r), ctypes.byref(c), ctypes.byref(sp)) == 0
+        if K < 12288 or keep:       # (the long K runs on this tile when its two halves are handed on)
+            assert (r.value, c.value) == (256, 256), (r.value, c.value, sp.value)
+        y = ops.linear(x, pw, out_dtype=torch.float32, partials=bool(keep))
+        if keep and sp.value > 1:
+            assert y.dim() == 3 and y.shape[0] == sp.value
+        _close(ops.as_tensor(y), ref, 3e-5, f"product (keep={keep}, {sp.value} parts)")
+    yb = ops.linear(x, pw)       # bfloat16 result
+    _close(yb, ref, 8e-3, "bfloat16 result")
+
+
 def test_gemm_plan():
     """The plan of the tiled product: large tiles where they fill the machine, smaller ones or K
     split over blocks where they would not; never more parts than K has tiles for."""
