@@ -76,10 +76,10 @@ def sync():
     torch.cuda.synchronize()
 
 
-def measure_prefill(engine, gen, T, vocab, reps=3):
+def measure_prefill(engine, gen, T, vocab, reps=5, warm=2):
     from tffinfer_amd.engine.batch import StepEntry
     times = []
-    for i in range(reps + 1):
+    for i in range(reps + warm):
         rid = f"prefill{i}"
         toks = random_prompt(gen, T, vocab)
         engine.runner.add_request(rid)
@@ -90,7 +90,7 @@ def measure_prefill(engine, gen, T, vocab, reps=3):
         dt = time.perf_counter() - t0
         assert logits.shape[0] == 1
         engine.runner.free_request(rid)
-        if i > 0:   # the first run warms up
+        if i >= warm:   # the first runs warm up (allocator, work tables, clocks)
             times.append(dt)
     return statistics.median(times)
 

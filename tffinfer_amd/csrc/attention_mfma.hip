@@ -198,8 +198,7 @@ __global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
                     sv[kt * 4 + i] = x;
                     mt = fmaxf(mt, x);
                 }
-            mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            mt = rows_max(mt);
             const float m_new = fmaxf(m_run[t], mt);
             const float alpha = m_new == -INFINITY ? 1.f : __expf(m_run[t] - m_new);
             float ps = 0.f;
@@ -238,8 +237,7 @@ __global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
 #pragma unroll
     for (int t = 0; t < NQT; ++t) {
         float l = l_run[t];
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
+        l = rows_sum(l);
         if (!c_ok[t]) continue;
         {
             const float inv = 1.0f / l;
@@ -303,8 +301,7 @@ __device__ __forceinline__ void norm_rope_fragments(bf16x8 (&f)[(DT * 16 + 31) /
             x[ks][j] = (float)f[ks][j];
             ss = fmaf(x[ks][j], x[ks][j], ss);
         }
-    ss += __shfl_xor(ss, 16, 64);
-    ss += __shfl_xor(ss, 32, 64);
+    ss = rows_sum(ss);
     if (has_norm) {
         const float rr = rsqrtf(ss / (float)D + eps);
 #pragma unroll
@@ -530,8 +527,7 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
                 sv_[kt * 4 + i] = x;                                                                \
                 mt_ = fmaxf(mt_, x);                                                                \
             }                                                                                       \
-        mt_ = fmaxf(mt_, __shfl_xor(mt_, 16, 64));                                                  \
-        mt_ = fmaxf(mt_, __shfl_xor(mt_, 32, 64));                                                  \
+        mt_ = rows_max(mt_);                                                                        \
         const float m_new_ = fmaxf(m_run, mt_);                                                     \
         const float alpha_ = m_new_ == -INFINITY ? 1.f : __expf(m_run - m_new_);                    \
         float ps_ = 0.f;                                                                            \
@@ -601,8 +597,7 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
 #undef TFF_WAVE_COMPUTE
 
     float l = l_run;
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
+    l = rows_sum(l);
     if (!c_ok) return;
     if (SPLIT) {
         // keys are split for entries of one token only: partial results are kept by entry
@@ -860,8 +855,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
             }
             float mt = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
                              fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-            mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            mt = rows_max(mt);
             const float m_new = fmaxf(m_run[t], mt);          // maxima are kept in raw score units
             const float mb = m_new == -INFINITY ? 0.f : m_new * sl2;
             const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((m_run[t] - m_new) * sl2);
@@ -930,8 +924,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
 #pragma unroll
     for (int t = 0; t < NQT; ++t) {
         float l = l_run[t];
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
+        l = rows_sum(l);
         if (!c_ok[t]) continue;
         const float inv = 1.0f / l;
         bf16_t* op = out + ((size_t)c_tok[t] * nq + c_head[t]) * D;

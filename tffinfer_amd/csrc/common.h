@@ -71,6 +71,26 @@ int tff_check_launch(const char* what);
         if (!(cond)) return tff_fail(__VA_ARGS__); \
     } while (0)
 
+// Maximum / sum over the four lanes i, i ^ 16, i ^ 32, i ^ 48 (the four 16-lane rows of a wave),
+// the result in all four.  v_permlane16_swap exchanges the odd rows of one register with the
+// even rows of another and v_permlane32_swap the upper half of one with the lower half of the
+// other: applied to two copies of a value, the two results hold, lane by lane, the two values
+// to combine.  No trip through LDS, unlike a shuffle across rows.  The sum adds in the order
+// (row 0 + row 1) + (row 2 + row 3), as two shuffle steps would.
+typedef unsigned tff_uint2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float rows_max(float v) {
+    tff_uint2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    const float m = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(m), __float_as_uint(m), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float rows_sum(float v) {
+    tff_uint2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    const float m = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(m), __float_as_uint(m), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Copies 16 bytes a lane from global memory straight into LDS: lane i's bytes land at
 // lds_wave_base + 16 i (global_load_lds_dwordx4; the LDS base travels in M0 and is the same for
 // the whole wave).  It is written as inline assembly on purpose: the compiler's own builtin
