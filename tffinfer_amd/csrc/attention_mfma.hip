@@ -657,6 +657,51 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __r
     }
 }
 
+// The same for a few splits (many requests): one wave per (row, head), four to a block, and no
+// exchange between lanes: every lane goes
+// through the splits' maxima and sums itself (the loads are the same for the whole wave) and
+// adds up its own elements of the head, in the order of the splits.
+__global__ __launch_bounds__(256) void attn_split_reduce_few_kernel(const float* __restrict__ part_o,
+                                                                 const float* __restrict__ part_ml,
+                                                                 bf16_t* __restrict__ out, int splits,
+                                                                 int R_total, int nq, int d,
+                                                                 const int32_t* __restrict__ rows, int n) {
+    const int lane = threadIdx.x & 63;
+    const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);     // (row, head), heads fastest
+    if (pair >= n * nq) return;
+    const int i = pair / nq, h = pair - i * nq;
+    // rows: (entry, token) pairs; without them entry i is token i
+    const int r = rows ? rows[2 * i] : i;
+    const int t = rows ? rows[2 * i + 1] : i;
+    const size_t stride_ml = (size_t)R_total * nq * 2, stride_o = (size_t)R_total * nq * d;
+    const float* ml = part_ml + ((size_t)r * nq + h) * 2;
+    const float* po = part_o + ((size_t)r * nq + h) * d;
+    float m = -INFINITY;
+    for (int s = 0; s < splits; ++s) m = fmaxf(m, ml[s * stride_ml]);
+    float l = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};              // d <= 256: up to four elements a lane
+    for (int s0 = 0; s0 < splits; s0 += 4) {
+        float w[4], v[4][4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {                            // four splits' loads in flight
+            const int s = min(s0 + u, splits - 1);
+            const float ms = ml[s * stride_ml];
+            w[u] = (s0 + u < splits && ms != -INFINITY) ? __expf(ms - m) : 0.f;
+            l = fmaf(ml[s * stride_ml + 1], w[u], l);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[u][e] = lane + 64 * e < d ? po[s * stride_o + lane + 64 * e] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = fmaf(v[u][e], w[u], acc[e]);
+    }
+    const float inv = 1.0f / l;
+    bf16_t* o = out + ((size_t)t * nq + h) * d;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        if (lane + 64 * e < d) o[lane + 64 * e] = (bf16_t)(acc[e] * inv);
+}
+
 // ------------------------------------------------- prompt portions, by block ---
 // For portions of many tokens a block of NW waves shares its keys and values:
 // every 32-key slice is copied once from the pages into LDS (by the load unit,
@@ -1117,7 +1162,11 @@ TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml
     TFF_REQUIRE(n >= 0 && n <= R_total, "attention_split_reduce: %d rows of %d entries", n, R_total);
     if (n == 0) return 0;
     TFF_REQUIRE(splits <= 256, "attention_split_reduce: at most 256 splits, got %d", splits);
-    attn_split_reduce_kernel<<<dim3(n, nq), 256, 0, (hipStream_t)stream>>>(
-        part_o, part_ml, (bf16_t*)out, splits, R_total, nq, d, rows);
+    if (splits <= 4 && d <= 256)
+        attn_split_reduce_few_kernel<<<(n * nq + 3) / 4, 256, 0, (hipStream_t)stream>>>(
+            part_o, part_ml, (bf16_t*)out, splits, R_total, nq, d, rows, n);
+    else
+        attn_split_reduce_kernel<<<dim3(n, nq), 256, 0, (hipStream_t)stream>>>(
+            part_o, part_ml, (bf16_t*)out, splits, R_total, nq, d, rows);
     return tff_check_launch("attention_split_reduce");
 }

@@ -358,7 +358,8 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
     // here and added up (TFF_ROW_SCALE) after the first loads of W are on their way.
     constexpr int SSV = 16;   // 16-byte loads a lane keeps: rows of up to 64 * SSV sums
     float4 ssv[EPI == 1 ? SSV : 1];
-    const bool scales = EPI == 1 && wave == 0;
+    // (the waves that write results: the first of a set, of the gate's set with GLU; rows that exist)
+    const bool scales = EPI == 1 && wave == 0 && (!GLU || (set & 1) == 0) && fr < M;
     if constexpr (EPI == 1) {
         if (scales) {
             const float* sp = fz.ss_in + (size_t)fr * fz.ss_stride;
