@@ -633,11 +633,14 @@ def test_attention_decode_fused(nq, nkv, d, ps, window, splits, pairing, with_no
     """Decode steps from the raw projection output: q/k norm, rotation, the token's key and value
     into its page and attention in one kernel, against each part's formula; the slot of the new
     token holds large numbers beforehand, which must not reach the result; nothing else in the
-    cache changes; with write_kv off the cache is read only."""
+    cache changes.  One entry has a negative slot (a padding row of a captured step, a call that
+    reads another call's cache): nothing of it is written and its key and value come from its
+    page.  Without a slot mapping the cache is read only."""
     ops = _ops()
     from tffinfer_amd.parts.position import RotaryEmbedding
     eps, theta = 1e-5, 5000.0
     entries = [(0, 1), (1, 1), (31, 1), (32, 1), (700, 1), (255, 1), (64, 1), (7, 1), (8, 1)]
+    unwritten = 2
     batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=d + ps)
     R = batch.num_tokens
     g = torch.Generator().manual_seed(5)
@@ -673,41 +676,50 @@ def test_attention_decode_fused(nq, nkv, d, ps, window, splits, pairing, with_no
     scale = 1 / math.sqrt(d)
     refs = []
     for r, (P, _) in enumerate(entries):
-        k = torch.cat([ks[r][:P], k_new[r:r + 1]])
-        v = torch.cat([vs[r][:P], v_new[r:r + 1]])
+        if r == unwritten:          # its key and value are the page's
+            k, v = ks[r][:P + 1], vs[r][:P + 1]
+        else:
+            k = torch.cat([ks[r][:P], k_new[r:r + 1]])
+            v = torch.cat([vs[r][:P], v_new[r:r + 1]])
         refs.append(_attn_ref(q[r:r + 1], k, v, positions[r:r + 1], window, scale)[0])
     ref = torch.stack(refs)
     # the slots of the new tokens hold numbers that would wreck the result if they were read
     bt = kv.block_tables.cpu()
     kc0, vc0 = kv.k_cache.cpu().clone(), kv.v_cache.cpu().clone()
+    slots = []
     for r, (P, _) in enumerate(entries):
+        if r == unwritten:
+            slots.append(-1)
+            continue
         kc0[bt[r, P // ps], :, P % ps] = 300.0
         vc0[bt[r, P // ps], :, :, P % ps] = -300.0
+        slots.append(int(bt[r, P // ps]) * ps + P % ps)
+    slots = torch.tensor(slots, dtype=torch.int32, device=DEV)
     kv.k_cache, kv.v_cache = kc0.to(DEV), vc0.to(DEV)
     w = (None if qw is None else qw.to(DEV), None if kw is None else kw.to(DEV))
     assert ops.decode_fused_supported(qkv.to(DEV), d, ps, table, pr, batch)
     out = ops.attention_decode_fused(qkv.to(DEV), nq, nkv, d, w[0], w[1], eps, table, pr, kv, batch, window, scale,
-                                     write_kv=True, splits=splits)
+                                     slot_mapping=slots, splits=splits)
     _close(out.reshape(R, nq, d), ref, 1.5e-2, "fused decode attention")
     kc1, vc1 = kv.k_cache.cpu(), kv.v_cache.cpu()
     expect_k, expect_v = kc0.clone(), vc0.clone()
     for r, (P, _) in enumerate(entries):
+        if r == unwritten:
+            continue
         _close(kc1[bt[r, P // ps], :, P % ps], k_new[r].double(), 8e-3, f"key of entry {r} in its page")
         assert torch.equal(vc1[bt[r, P // ps], :, :, P % ps], v_new[r]), f"value of entry {r} in its page"
         expect_k[bt[r, P // ps], :, P % ps] = kc1[bt[r, P // ps], :, P % ps]
         expect_v[bt[r, P // ps], :, :, P % ps] = vc1[bt[r, P // ps], :, :, P % ps]
     assert torch.equal(kc1, expect_k) and torch.equal(vc1, expect_v), "a slot of another token was written"
-    # a call that only reads: the pages hold the token already
+    # a call that only reads: the pages hold the tokens already
     out2 = ops.attention_decode_fused(qkv.to(DEV), nq, nkv, d, w[0], w[1], eps, table, pr, kv, batch, window, scale,
-                                      write_kv=False, splits=splits)
+                                      slot_mapping=None, splits=splits)
     assert torch.equal(kv.k_cache.cpu(), kc1) and torch.equal(kv.v_cache.cpu(), vc1)
     _close(out2.reshape(R, nq, d), ref, 1.5e-2, "fused decode attention, cache read only")
     # the two-kernel path gives the same to rounding
     kv.k_cache, kv.v_cache = kc0.to(DEV), vc0.to(DEV)
-    slots = torch.tensor([int(bt[r, P // ps]) * ps + P % ps for r, (P, _) in enumerate(entries)], dtype=torch.int32)
     dq = qkv.to(DEV).clone()
-    ops.qk_norm_rope_kv(dq, nq, nkv, d, w[0], w[1], eps, table, pr, batch.positions, slots.to(DEV),
-                        kv.k_cache, kv.v_cache)
+    ops.qk_norm_rope_kv(dq, nq, nkv, d, w[0], w[1], eps, table, pr, batch.positions, slots, kv.k_cache, kv.v_cache)
     out3 = ops.attention_mfma(dq, nq, nkv, d, kv, batch, window, scale, splits=splits)
     _close(out.reshape(R, nq, d), out3.reshape(R, nq, d).double().cpu(), 1.5e-2, "fused against two kernels")
 

@@ -57,7 +57,7 @@ def test_trace_run_program(model_dirs, tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 @pytest.mark.parametrize("mode", ["tail", "mixed"])
 def test_replay_with_decode_graphs(model_dirs, name, dtype, mode):
     """Decode-only steps run as replays of a captured HIP graph: every replay,
@@ -81,7 +81,45 @@ def test_replay_with_decode_graphs(model_dirs, name, dtype, mode):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,n", [("A", 128), ("B", 256)])
+@pytest.mark.parametrize("name", ["A", "B", "C"])     # (C's head size takes the decode kernel that writes keys itself)
+def test_padding_rows_of_a_graph_write_nothing(model_dirs, name, dtype):
+    """Three requests decode through the graph of four rows: the fourth row is padding (token 0
+    at position 0 with a block table of zeros).  After every step the caches must hold, bit for
+    bit, what the same steps leave without graphs: nothing of the padding row may reach page 0
+    or any other page."""
+    from tffinfer_amd.engine.batch import StepEntry
+    from tffinfer_amd.engine.runner import ModelRunner
+    from tffinfer_amd.models import load_model
+    model_dir = model_dirs[name]
+    V = read_config(model_dir)["vocab_size"]
+    ps = PAGE_SIZE[name]
+    prompts = {f"r{i}": random_tokens(5 + 7 * i, V, 300 + i) for i in range(3)}
+    runners = [ModelRunner(load_model(model_dir, DTYPES[dtype], "cuda:0"), page_size=ps, num_pages=24, max_seqs=4,
+                           use_graphs=g) for g in (False, True)]
+    for rn in runners:
+        for rid, toks in prompts.items():
+            rn.add_request(rid)
+        rn.step([StepEntry(rid, toks, []) for rid, toks in prompts.items()])
+    for step in range(6):
+        toks = {rid: (step * 13 + i * 5 + 1) % V for i, rid in enumerate(prompts)}
+        logits = [rn.step([StepEntry(rid, [toks[rid]], [0]) for rid in prompts]).clone() for rn in runners]
+        assert torch.equal(logits[0], logits[1]), f"logits differ at decode step {step}"
+        for (k0, v0), (k1, v1) in zip(_all_caches(runners[0]), _all_caches(runners[1])):
+            assert torch.equal(k0, k1) and torch.equal(v0, v1), f"caches differ after decode step {step}"
+    assert runners[1]._graphs and not runners[0]._graphs
+
+
+def _all_caches(runner):
+    out, seen = [], set()
+    for cache_id, _, kvspec, _ in runner.model.call_requirements():
+        if kvspec is not None and cache_id not in seen:
+            seen.add(cache_id)
+            out.append(runner.cache.kv_tensors(cache_id))
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,n", [("A", 128), ("B", 256), ("C", 300)])
 @pytest.mark.parametrize("graphs", [False, True])
 def test_long_decoding(model_dirs, name, dtype, n, graphs):
     """A few prompt tokens, then one token a step up to the model's longest

@@ -270,13 +270,15 @@ __global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
 // the token: the weights of the per-head RMS norms of q and k (null: no norm), the table of
 // rotation angles [position][pair][cos, sin] (null: no rotation; else the whole head is
 // rotated), the pairing (0: (i, i + d/2), 1: (2i, 2i+1)) and the caches to write the token's
-// key and value into (null: the cache holds them already and is only read).
+// key and value into (null: the cache holds them already and is only read; so it is for a
+// token whose slot_mapping entry is negative: a padding row of a captured step, say).
 struct AttnFuse {
     const float* q_weight;
     const float* k_weight;
     const float* cos_sin;
     bf16_t* k_write;
     bf16_t* v_write;
+    const int32_t* slot_mapping;   // per token; a negative entry: this token's key and value are not written
     float eps;
     int pairing;
 };
@@ -406,7 +408,7 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
     // The norm weights and the position's angles go to LDS beside the page numbers; the raw q, k
     // and v are loaded after the barrier and worked on once the first keys and values are on
     // their way, so that they delay nothing.
-    const bool owns_new = FUSED && fz.k_write != nullptr && s_begin < s_end && s_end == nsteps;
+    const bool owns_new = FUSED && fz.k_write != nullptr && s_begin < s_end && s_end == nsteps && fz.slot_mapping[tok0] >= 0;
     const bool has_norm = FUSED && fz.q_weight != nullptr, has_rope = FUSED && fz.cos_sin != nullptr;
 
     if constexpr (FUSED) {
@@ -1016,7 +1018,7 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
         return tff_check_launch("attention_mfma_block");
     }
     const dim3 grid(num_work, nkv, splits);
-    const AttnFuse fz = fuse ? *fuse : AttnFuse{nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
+    const AttnFuse fz = fuse ? *fuse : AttnFuse{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
 #define TFF_ATTN_ARGS                                                                              \
     q, q_stride, out, part_o, part_ml, k_cache, v_cache, block_tables, bt_stride, cu_tokens,       \
         start_pos, work, tiles_per_entry, nq, nkv, page_size, page_shift, window, scale, T_total
@@ -1104,15 +1106,18 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
 // of token r are row r of qkv ([R, (nq + 2 nkv) d]).  Per head, q and k get their RMS norm
 // (weights [d]; both null: none) and the rotation by the angles of the token's position
 // start_pos[r] (cos_sin [max_pos, d/2, 2]; null: none; the whole head is rotated; pairing 0:
-// (i, i + d/2), which needs d to be a multiple of 64, 1: (2i, 2i+1)); with write_kv the token's
-// key and value go to position start_pos[r] of the entry's pages, else the pages hold them
-// already.  Then attention as tff_attention_mfma does it for such a step.
+// (i, i + d/2), which needs d to be a multiple of 64, 1: (2i, 2i+1)).  Where slot_mapping[r] >= 0
+// the token's key and value go to position start_pos[r] of the entry's pages (the slot that
+// the entry's block table gives for it); where it is negative, and everywhere if slot_mapping
+// is null, the pages hold them already and are only read.  Then attention as
+// tff_attention_mfma does it for such a step.
 TFF_API int tff_attention_decode_fused(const void* qkv, int qkv_stride, void* out, float* part_o,
                                        float* part_ml, void* k_cache, void* v_cache,
                                        const int32_t* block_tables, int bt_stride,
                                        const int32_t* cu_tokens, const int32_t* start_pos,
+                                       const int32_t* slot_mapping,
                                        const float* q_weight, const float* k_weight, float eps,
-                                       const float* cos_sin, int max_pos, int pairing, int write_kv,
+                                       const float* cos_sin, int max_pos, int pairing,
                                        int splits, int R, int nq, int nkv, int d, int page_size,
                                        int num_pages, int window, float scale, tff_stream_t stream) {
     TFF_REQUIRE(qkv && out && k_cache && v_cache && block_tables && cu_tokens && start_pos,
@@ -1134,8 +1139,8 @@ TFF_API int tff_attention_decode_fused(const void* qkv, int qkv_stride, void* ou
     TFF_REQUIRE(bt_stride > 0 && num_pages > 0 && window >= 0 && R >= 0, "attention_decode_fused: bad geometry");
     if (R == 0) return 0;
     const int tiles = (nq / nkv + 15) / 16;
-    AttnFuse fz{q_weight, k_weight, cos_sin, write_kv ? (bf16_t*)k_cache : nullptr,
-                write_kv ? (bf16_t*)v_cache : nullptr, eps, pairing};
+    AttnFuse fz{q_weight, k_weight, cos_sin, slot_mapping ? (bf16_t*)k_cache : nullptr,
+                slot_mapping ? (bf16_t*)v_cache : nullptr, slot_mapping, eps, pairing};
     hipStream_t s = (hipStream_t)stream;
 #define TFF_ATTN_CASE(DTV)                                                                          \
     case DTV * 16:                                                                                  \

@@ -137,14 +137,16 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
 // per-head RMS norm of q and k (weights [d]; both null: none), rotation by the angles of the
 // token's position start_pos[r] (cos_sin [max_pos, d/2, 2]; null: none; the whole head is
 // rotated; pairing 0 needs d to be a multiple of 64), the token's key and value written to
-// their page (write_kv = 0: the pages hold them already), attention over the pages.  With
+// position start_pos[r] of the entry's pages where slot_mapping[r] >= 0 (negative, or
+// slot_mapping null: the pages hold them already), attention over the pages.  With
 // splits > 1 the partial results need tff_attention_split_reduce as there.
 TFF_API int tff_attention_decode_fused(const void* qkv, int qkv_stride, void* out, float* part_o,
                                        float* part_ml, void* k_cache, void* v_cache,
                                        const int32_t* block_tables, int bt_stride,
                                        const int32_t* cu_tokens, const int32_t* start_pos,
+                                       const int32_t* slot_mapping,
                                        const float* q_weight, const float* k_weight, float eps,
-                                       const float* cos_sin, int max_pos, int pairing, int write_kv,
+                                       const float* cos_sin, int max_pos, int pairing,
                                        int splits, int R, int nq, int nkv, int d, int page_size,
                                        int num_pages, int window, float scale, tff_stream_t stream);
 // Merges partial results kept by entry (part_o [splits, R_total, nq, d]) into out rows:

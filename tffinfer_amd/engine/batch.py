@@ -25,16 +25,15 @@ class StepEntry:
 
 class KVView:
     """What a mixer sees of the cache in one layer call."""
-    __slots__ = ("k_cache", "v_cache", "block_tables", "slot_mapping", "page_size", "group", "writes")
+    __slots__ = ("k_cache", "v_cache", "block_tables", "slot_mapping", "page_size", "group")
 
-    def __init__(self, k_cache, v_cache, block_tables, slot_mapping, page_size, group, writes=True):
+    def __init__(self, k_cache, v_cache, block_tables, slot_mapping, page_size, group):
         self.k_cache = k_cache
         self.v_cache = v_cache
         self.block_tables = block_tables
-        self.slot_mapping = slot_mapping     # of -1 where the call only reads the cache
+        self.slot_mapping = slot_mapping     # per token; -1: not written (a call that only reads, padding)
         self.page_size = page_size
         self.group = group
-        self.writes = writes                 # whether the call puts the step's keys and values in
 
 
 class GroupTables:

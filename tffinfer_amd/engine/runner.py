@@ -51,7 +51,7 @@ class StepContext(LayerContext):
         if group is not None:
             gt = self.batch.groups[group]
             c.kv = KVView(k, v, gt.block_tables, gt.slot_mapping if writes else gt.no_slot_mapping,
-                          self._cache.page_size, group, bool(writes))
+                          self._cache.page_size, group)
         c.state = state
         return c
 

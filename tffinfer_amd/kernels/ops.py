@@ -618,10 +618,13 @@ def decode_fused_supported(qkv: torch.Tensor, d: int, page_size: int, cos_sin, p
 
 def attention_decode_fused(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, eps: float,
                            cos_sin, pairing: int, kv, batch, window: int = 0, scale: float | None = None,
-                           write_kv: bool = True, splits: int | None = None) -> torch.Tensor:
+                           slot_mapping: torch.Tensor | None = None, splits: int | None = None) -> torch.Tensor:
     """A decode-only step from the fused projection's output ``qkv`` [R, (nq +
     2 nkv) d]: q/k norm, rotation, the new keys and values into their pages and
-    the attention over the pages, in one kernel (plus the merge of split keys)."""
+    the attention over the pages, in one kernel (plus the merge of split keys).
+    ``slot_mapping`` (int32 [R]) says which tokens' keys and values are written
+    (entries >= 0; the place is the one the block table gives for the token's
+    position); None: no token's, the pages hold them already."""
     _req(qkv, "attention_decode_fused qkv", torch.bfloat16, 2)
     R = batch.num_reqs
     if qkv.shape[0] != R or batch.num_tokens != R or batch.max_new_tokens != 1:
@@ -650,6 +653,10 @@ def attention_decode_fused(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weigh
         if 2 * cos_sin.shape[1] != d or cos_sin.shape[2] != 2:
             raise _lib.KernelError(f"attention_decode_fused: a rotation table of shape {tuple(cos_sin.shape)} "
                                    f"does not rotate whole heads of {d}")
+    if slot_mapping is not None:
+        _req(slot_mapping, "slot_mapping", torch.int32, 1)
+        if slot_mapping.numel() != R:
+            raise _lib.KernelError("attention_decode_fused: slot_mapping needs one entry per token")
     G = nq // nkv
     tiles = -(-G // 16)
     if scale is None:
@@ -666,7 +673,7 @@ def attention_decode_fused(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weigh
     _lib.check(L.tff_attention_decode_fused(
         qkv.data_ptr(), qkv.stride(0), out.data_ptr(), _ptr(part_o), _ptr(part_ml), k_cache.data_ptr(),
         v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(), batch.start_pos.data_ptr(),
-        _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin), max_pos, int(pairing), 1 if write_kv else 0,
+        _ptr(slot_mapping), _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin), max_pos, int(pairing),
         splits, R, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale), stream))
     if splits > 1:
         _lib.check(L.tff_attention_split_reduce(part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), splits, R,
@@ -677,13 +684,13 @@ def attention_decode_fused(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weigh
 def qkv_attention(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, eps: float, cos_sin,
                   pairing: int, kv, batch, window: int = 0, scale: float | None = None) -> torch.Tensor:
     """From the fused projection's output to the attention's output [T, nq d]:
-    q/k norm and rotation, the step's keys and values into the cache (unless
-    ``kv.writes`` is false: the call reads a cache that another call fills),
-    attention over the cache.  Decode-only steps in bfloat16 are one kernel."""
-    writes = getattr(kv, "writes", True)
+    q/k norm and rotation, the step's keys and values into the cache at
+    ``kv.slot_mapping`` (negative entries: not written; the call reads a cache
+    that another call fills, or the row is padding), attention over the cache.  Decode-only steps in bfloat16 are one kernel."""
     if decode_fused_supported(qkv, d, kv.k_cache.shape[2], cos_sin, pairing, batch):
+        # (a call that only reads its cache, or a padding row, has negative slots)
         return attention_decode_fused(qkv, nq, nkv, d, q_weight, k_weight, eps, cos_sin, pairing, kv, batch,
-                                      window, scale, write_kv=writes)
+                                      window, scale, slot_mapping=kv.slot_mapping)
     qk_norm_rope_kv(qkv, nq, nkv, d, q_weight, k_weight, eps, cos_sin, pairing, batch.positions,
                     kv.slot_mapping, kv.k_cache, kv.v_cache)
     return paged_attention(qkv, nq, nkv, d, kv, batch, window, scale)
