@@ -55,10 +55,11 @@ def test_greedy_through_the_reference_style_entry_point_fp32(model_dirs):
     assert out == [plain_generate_greedy(d, p, 16) for p in prompts]
 
 
+@pytest.mark.parametrize("name", ["A", "C"])    # (C: the head size of the large models and its decode kernels)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_greedy_engine(model_dirs, dtype):
+def test_greedy_engine(model_dirs, dtype, name):
     from tffinfer_amd import EngineOptions, LLMEngine
-    d = model_dirs["A"]
+    d = model_dirs[name]
     V = read_config(d)["vocab_size"]
     prompts = [random_tokens(n, V, 60 + n) for n in (1, 9, 40)]
     eng = LLMEngine.from_model_dir(d, EngineOptions(dtype=dtype, page_size=16, kv_tokens=256, max_num_seqs=4))
@@ -134,7 +135,11 @@ def test_steps_launched_ahead_give_the_same_tokens(model_dirs, dtype, use_graphs
     """Decode steps launched before the tokens of the step in flight are read: the same
     outputs as with one step at a time, with requests that end at different lengths, one
     that ends on a token of its own choosing, more requests than slots and a pool that
-    runs out."""
+    runs out.  (A request that ends is noticed a step later when steps are launched ahead, so
+    the next one is admitted a step later and some tokens are computed in other batches, by
+    other kernels, than with one step at a time: equal to rounding, which with this model and
+    these seeds flips no choice.  What the engine computes is checked against the plain
+    implementation, with tolerances, by the tests above.)"""
     from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
     d = model_dirs["B"]
     V = read_config(d)["vocab_size"]
@@ -150,7 +155,7 @@ def test_steps_launched_ahead_give_the_same_tokens(model_dirs, dtype, use_graphs
         if ahead:   # request 2 stops at the token it chose as its 12th
             eos = outs[False][2][11]
         for i, (p, s, n) in enumerate(zip(prompts, sc, lens)):
-            eng.add_request(p, s, max_new_tokens=n, ignore_eos=not (ahead and i == 2),
+            eng.add_request(p, s, max_new_tokens=n, ignore_eos=not (eos is not None and i == 2),
                             eos_token_id=eos if i == 2 else None, request_id=i)
         got = {i: [] for i in range(6)}
         fin = {}
