@@ -355,7 +355,7 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
     float4 resid_in = make_float4(0.f, 0.f, 0.f, 0.f), normw_in = resid_in;
     // EPI 1: lane (fr, fg) of a set's first wave adds every fourth group of four sums of row fr,
     // then the four lanes of a row meet: the same order in every block.  The loads are issued
-    // here and added up (TFF_ROW_SCALE) after the first loads of W are on their way.
+    // here, ahead of the stream of W, and added up (TFF_ROW_SCALE) when that stream has ended.
     constexpr int SSV = 16;   // 16-byte loads a lane keeps: rows of up to 64 * SSV sums
     float4 ssv[EPI == 1 ? SSV : 1];
     // (the waves that write results: the first of a set, of the gate's set with GLU; rows that exist)
@@ -373,8 +373,7 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
     }
 #define TFF_ROW_SCALE()                                                                            \
     if constexpr (EPI == 1) {                                                                      \
-        if (scales && row_scale_pending) {                                                         \
-            row_scale_pending = false;                                                             \
+        if (scales) {                                                                              \
             const float* sp = fz.ss_in + (size_t)fr * fz.ss_stride;                                \
             const int vec_end = fz.ss_count & ~3;                                                  \
             float ssum = 0.f;                                                                      \
@@ -391,7 +390,6 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
             row_scale = rsqrtf(ssum * fz.inv_dim + fz.eps);                                        \
         }                                                                                          \
     }
-    bool row_scale_pending = true;
     if constexpr (EPI == 2) {
         if (wave == 0) {
             const int n = nb0 * 16 + fg * 4;
@@ -420,7 +418,6 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
 #pragma unroll
                 for (int t = 0; t < MT; ++t) ra[u][t] = ld16(arow[t] + st * 32 + fg * 8);
             }
-            TFF_ROW_SCALE()
             for (; s0 < full_end; s0 += UNROLL) {
 #pragma unroll
                 for (int u = 0; u < UNROLL; ++u) {
@@ -451,7 +448,6 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
 #pragma unroll
             for (int t = 0; t < MT; ++t) ra[u][t] = ld16(arow[t] + (s0 + u) * 32 + fg * 8);
         }
-        TFF_ROW_SCALE()
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
@@ -479,7 +475,7 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
             for (int t = 0; t < MT; ++t)
                 acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(rw[r]), as_frag(ra[t]), acc[r][t], 0, 0, 0);
     }
-    TFF_ROW_SCALE()   // if no loop above came to it
+    TFF_ROW_SCALE()
 #undef TFF_ROW_SCALE
 #pragma unroll
     for (int r = 0; r < R; ++r)
