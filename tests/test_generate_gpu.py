@@ -70,13 +70,14 @@ def test_greedy_engine(model_dirs, dtype, name):
         check_choices(d, r, dtype)
 
 
+@pytest.mark.parametrize("name", ["B", "C"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_chunked_prefill_mixed_with_decode_temperature_small_pool(model_dirs, dtype):
-    """Tiny B's workload: 5 requests, portions of 24 tokens beside decoding,
-    24 tokens at temperature 0.8 with a fixed seed, on a pool so small that
+def test_chunked_prefill_mixed_with_decode_temperature_small_pool(model_dirs, dtype, name):
+    """Tiny B's workload (and with C's head size): 5 requests, portions of 24 tokens beside
+    decoding, 24 tokens at temperature 0.8 with a fixed seed, on a pool so small that
     requests are preempted and computed again."""
     from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
-    d = model_dirs["B"]
+    d = model_dirs[name]
     V = read_config(d)["vocab_size"]
     prompts = [random_tokens(n, V, 70 + n) for n in (3, 17, 31, 64, 100)]
     sc = [SamplingConfig("random", temperature=0.8, seed=100 + i) for i in range(5)]
