@@ -28,8 +28,16 @@ TINY_C = dict(
     vocab_size=1000, max_position_embeddings=512, rms_norm_eps=3e-6, rope_theta=500000.0,
     tie_word_embeddings=False,
 )
-TINY_CONFIGS = {"A": (TINY_A, 11), "B": (TINY_B, 23), "C": (TINY_C, 31)}
-PAGE_SIZE = {"A": 16, "B": 8, "C": 32}
+# The same head size with a sliding window on every other layer (the decode kernel that writes
+# keys itself, on pages that a window has passed and given back), four heads to a kv head.
+TINY_D = dict(
+    architectures=["Qwen3ForCausalLM"], hidden_size=104, num_hidden_layers=4,
+    num_attention_heads=4, num_key_value_heads=1, head_dim=64, intermediate_size=72,
+    vocab_size=777, max_position_embeddings=320, rms_norm_eps=2e-6, rope_theta=20000.0,
+    tie_word_embeddings=True, use_sliding_window=True, sliding_window=40, max_window_layers=2,
+)
+TINY_CONFIGS = {"A": (TINY_A, 11), "B": (TINY_B, 23), "C": (TINY_C, 31), "D": (TINY_D, 47)}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 32, "D": 16}
 
 
 def make_model_dir(path: str, cfg: dict, seed: int, dtype: str = "bfloat16") -> str:

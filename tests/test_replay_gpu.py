@@ -10,7 +10,7 @@ from helpers import PAGE_SIZE, TOL, random_tokens, read_config, rel_err
 pytestmark = pytest.mark.gpu
 
 DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
-LENGTHS = {"A": [1, 9, 40, 100], "B": [3, 17, 31, 64, 100, 150], "C": [2, 33, 70, 129, 200]}
+LENGTHS = {"A": [1, 9, 40, 100], "B": [3, 17, 31, 64, 100, 150], "C": [2, 33, 70, 129, 200], "D": [5, 41, 90, 160]}
 
 
 def requests_for(name, model_dir):
@@ -26,7 +26,7 @@ def make_runner(model_dir, dtype, page_size, num_pages, max_seqs=8):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("mode", ["whole", "tail", "chunks", "mixed"])
 def test_replay_modes(model_dirs, name, dtype, mode):
     model_dir = model_dirs[name]
@@ -57,7 +57,7 @@ def test_trace_run_program(model_dirs, tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("mode", ["tail", "mixed"])
 def test_replay_with_decode_graphs(model_dirs, name, dtype, mode):
     """Decode-only steps run as replays of a captured HIP graph: every replay,
@@ -81,7 +81,7 @@ def test_replay_with_decode_graphs(model_dirs, name, dtype, mode):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])     # (C's head size takes the decode kernel that writes keys itself)
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])     # (C's and D's head sizes take the decode kernel that writes keys itself)
 def test_padding_rows_of_a_graph_write_nothing(model_dirs, name, dtype):
     """Three requests decode through the graph of four rows: the fourth row is padding (token 0
     at position 0 with a block table of zeros).  After every step the caches must hold, bit for
@@ -119,7 +119,7 @@ def _all_caches(runner):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,n", [("A", 128), ("B", 256), ("C", 300)])
+@pytest.mark.parametrize("name,n", [("A", 128), ("B", 256), ("C", 300), ("D", 320)])
 @pytest.mark.parametrize("graphs", [False, True])
 def test_long_decoding(model_dirs, name, dtype, n, graphs):
     """A few prompt tokens, then one token a step up to the model's longest
@@ -136,7 +136,7 @@ def test_long_decoding(model_dirs, name, dtype, n, graphs):
                          num_pages=-(-n // ps), max_seqs=2, use_graphs=graphs)
     results = rl.run_steps_in_process(runner, steps)
     rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
-    if name == "B":   # the window groups gave pages back on the way
+    if name in ("B", "D"):   # the window groups gave pages back on the way
         assert any(g.spec.window > 0 for g in runner.cache.groups)
 
 
