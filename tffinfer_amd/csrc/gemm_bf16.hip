@@ -65,7 +65,7 @@ typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 
 constexpr int vmcnt_imm(int v) { return (v & 15) | (7 << 4) | (15 << 8) | ((v >> 4) << 14); }
 
-template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU, typename TC, int KPS = 2>
+template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU, typename TC, int KPS = 2, bool EARLY = false>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
     int K, int lda, int KB, int n_out, float* __restrict__ part) {
@@ -74,8 +74,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
     constexpr int AF = BM / 16 * KPS, WF = BN / 16 * KPS;   // fragments per operand tile (KPS k-steps of 32)
     constexpr int FR = AF + WF;                          // fragments per stage, 1 KB each
-    constexpr int LPW = FR / NW;                         // copies a wave issues per tile
-    static_assert(FR % NW == 0, "fragments are dealt to the waves evenly");
+    // copies a wave issues per tile: fragment wave + NW j is copy j of a wave; where the fragments
+    // do not go round evenly the last waves copy the last fragment once more (same bytes to the
+    // same place), so that every wave has the same number of copies in flight
+    constexpr int LPW = (FR + NW - 1) / NW;
     static_assert((STAGES - 2) * LPW < 64, "vmcnt has 6 bits");
     __shared__ __attribute__((aligned(1024))) bf16_t smem[STAGES * FR * 512];
     const int tid = threadIdx.x;
@@ -87,9 +89,14 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     // XCD t % 8), and the blocks an XCD runs one after the other walk the row tiles of one
     // column tile before the next: a tile of W is fetched into one L2 only, and the (smaller) A
     // is what every L2 holds.
+    // Row tiles are walked in groups of eight: with 32 blocks of an XCD in flight, four column
+    // tiles by eight row tiles share their fetches better than one column tile by 32 row tiles.
     const int TM = (M + BM - 1) / BM;
     const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
-    const int tn = (seq / TM) * 8 + xcd, tm = seq % TM;
+    const int per_group = (int)(gridDim.x >> 3) / TM * 8;   // blocks of an XCD per group of eight row tiles
+    const int grp = seq / per_group, in_grp = seq - grp * per_group;
+    const int grp_rows = min(8, TM - grp * 8);
+    const int tn = (in_grp / grp_rows) * 8 + xcd, tm = grp * 8 + in_grp % grp_rows;
     if (tn * BN >= N) return;   // the launch is padded to whole groups of eight column tiles
     const int m0 = tm * BM, n0 = tn * BN;
     const int NB = (N + 15) / 16;
@@ -110,7 +117,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     const bf16_t* src[LPW];
 #pragma unroll
     for (int j = 0; j < LPW; ++j) {
-        const int f = wave + NW * j;
+        const int f = min(wave + NW * j, FR - 1);
         if (f < AF) {
             const int row = min(m0 + (f / KPS) * 16 + fr, M - 1);   // rows past the end repeat the last
             src[j] = A + (size_t)row * lda;
@@ -127,7 +134,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
         const int kt_ = min((tile), nk - 1);                                                       \
         const int st_ = ((tile) - kt0) % STAGES;                                                   \
         _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                          \
-            const int f = wave + NW * j;                                                            \
+            const int f = min(wave + NW * j, FR - 1);                                               \
             const bf16_t* g_;                                                                      \
             if (f < AF) g_ = src[j] + min((kt_ * KPS + f % KPS) * 32 + fg * 8, K - 8);                 \
             else g_ = src[j] + (size_t)min(KPS * kt_ + (f - AF) % KPS, KB - 1) * 512;                  \
@@ -137,6 +144,36 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
 
 #pragma unroll
     for (int t = 0; t < STAGES - 1; ++t) TFF_ISSUE_TILE(kt0 + t)
+    if constexpr (EARLY) {
+        // The barrier stands between a tile's LDS reads and its MFMAs: a wave arrives with its
+        // operands on the way, and when the barrier opens every wave can start its MFMAs at once
+        // (with the barrier before the reads, all waves read at the same time and the matrix
+        // cores wait for the first operands after every barrier).  The barrier of tile kt makes
+        // tile kt + 1 visible, so the copies have to be one tile further ahead.
+        static_assert(KPS == 1 && STAGES >= 3, "one k-step a tile, three stages or more");
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * LPW));
+        __syncthreads();
+        for (int kt = kt0; kt < kt1; ++kt) {
+            const bf16_t* st = smem + ((kt - kt0) % STAGES) * FR * 512;
+            bf16x8 fw[WTN], fa[WTM];
+#pragma unroll
+            for (int i = 0; i < WTN; ++i)
+                fw[i] = *reinterpret_cast<const bf16x8*>(st + (AF + wn * WTN + i) * 512 + lane * 8);
+#pragma unroll
+            for (int j = 0; j < WTM; ++j)
+                fa[j] = *reinterpret_cast<const bf16x8*>(st + (wm * WTM + j) * 512 + lane * 8);
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * LPW));   // this wave's part of tile kt + 1 is in
+            asm volatile("s_barrier" ::: "memory");
+            TFF_ISSUE_TILE(kt + STAGES - 1)                              // into the stage of tile kt - 1
+            if (kt < KB) {
+#pragma unroll
+                for (int i = 0; i < WTN; ++i)
+#pragma unroll
+                    for (int j = 0; j < WTM; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[i], fa[j], acc[i][j], 0, 0, 0);
+            }
+        }
+    } else
     for (int kt = kt0; kt < kt1; ++kt) {
         __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * LPW));   // this wave's part of tile kt is in
         __syncthreads();                                             // ... and everybody else's
@@ -245,7 +282,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
 }
 
 // splits > 1: the blocks of a tile split K among them; part holds splits * M * N floats
-template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU = false, int KPS = 2>
+template <int WGM, int WGN, int WTM, int WTN, int STAGES, bool GLU = false, int KPS = 2, bool EARLY = false>
 static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda,
                           int c_dtype, int n_out, hipStream_t s, int splits = 1, float* part = nullptr,
                           bool reduce = true) {
@@ -256,10 +293,10 @@ static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int
     TFF_REQUIRE(tiles < (1L << 31), "gemm: too many tiles for M=%d N=%d", M, N);
     const dim3 grid((unsigned)tiles, 1, splits);
     if (c_dtype == TFF_F32)
-        gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, float, KPS>
+        gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, float, KPS, EARLY>
             <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out, part);
     else
-        gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, bf16_t, KPS>
+        gemm_bf16_async_kernel<WGM, WGN, WTM, WTN, STAGES, GLU, bf16_t, KPS, EARLY>
             <<<grid, 64 * WGM * WGN, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out, part);
     if (int rc = tff_check_launch("gemm_bf16_async")) return rc;
     if (splits > 1 && reduce) {
@@ -586,11 +623,13 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
     }
     // rate: flops a microsecond that a CU sustains on blocks of this tile; slots: blocks a CU holds
     struct Cand { int bm, bn, slots; double rate; };
-    static const Cand cands[4] = {{256, 256, 1, 4.2e6}, {128, 256, 1, 3.8e6}, {128, 128, 1, 2.6e6}, {64, 128, 2, 2.6e6}};
+    static const Cand cands[5] = {{256, 256, 1, 4.8e6}, {256, 192, 1, 4.5e6}, {128, 256, 1, 3.8e6},
+                                  {128, 128, 1, 2.6e6}, {64, 128, 2, 2.6e6}};
     GemmPlan best = {256, 256, 1};
     double best_t = 1e30;
     for (const Cand& c : cands)
         for (int S = 1; S <= (glu ? 2 : 8); S *= 2) {
+            if (glu && c.bn == 192) break;   // gate and up groups come in pairs: an even number a wave
             if (S > 1 && nk / S < 8) break;
             const double blocks = (double)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * S;
             const double cap = 256.0 * c.slots;
@@ -674,7 +713,7 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
             return launch_async_g<2, 2, 4, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         if (plan.tile == 128)
             return launch_async_g<2, 4, 4, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
-        return launch_async_g<4, 4, 4, 4, 2, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+        return launch_async_g<4, 4, 4, 4, 5, true, 1, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
     }
     if (M <= 16) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, nullptr);
     if (plan.tile == 64) {
@@ -690,7 +729,9 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
         return launch_async_g<2, 2, 4, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     if (plan.tile == 128)
         return launch_async_g<2, 4, 4, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
-    return launch_async_g<4, 4, 4, 4, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+    if (plan.bn == 192)
+        return launch_async_g<4, 4, 4, 3, 5, false, 1, true>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+    return launch_async_g<4, 4, 4, 4, 5, false, 1, true>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
 }
 
 // ---- the norm between two products of up to 16 rows, taken into them ----
