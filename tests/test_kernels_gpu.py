@@ -834,3 +834,5 @@ def test_measured_ceilings_are_plausible():
     assert 1000 < c["stream_read_GBps"] <= 8000
     assert 300 < c["mfma_bf16_TFLOPs_1_waves_per_simd"] <= c["mfma_bf16_TFLOPs_4_waves_per_simd"] * 1.1 <= 2500 * 1.1
 
+    # operands that change cost power, never gain speed (a tenth of slack for the clock's wander)
+    assert 300 < c["mfma_bf16_TFLOPs_varied_operands"] <= c["mfma_bf16_TFLOPs_4_waves_per_simd"] * 1.1

@@ -1,6 +1,7 @@
 // Two measuring kernels for the ceilings the other kernels are judged by on the
 // machine at hand: how fast memory can be streamed into registers, and how
-// fast the matrix cores run 16x16x32 bfloat16 MFMAs back to back.  They compute
+// fast the matrix cores run 16x16x32 bfloat16 MFMAs back to back (with operands
+// that never change, and with operands that change as those of a real product do).  They compute
 // nothing of use; the callers time them.
 #include "common.h"
 #include "tffinfer_kernels.h"
@@ -25,16 +26,38 @@ __global__ __launch_bounds__(256) void probe_stream_kernel(const uint4* __restri
     if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[0] = acc.x;   // keeps the loads alive
 }
 
+// VARIED = false: every MFMA multiplies the same two registers of small integers (few bits change
+// from one instruction to the next, the lowest power the matrix cores can draw); true: eight
+// registers of pseudo-random values on either side, taken in turn, as the operands of a real
+// product change.  The difference between the two rates is what the power limit costs.
+__device__ __forceinline__ uint32_t probe_hash(uint32_t x) {
+    x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+    return x;
+}
+template <bool VARIED>
 __global__ __launch_bounds__(256) void probe_mfma_kernel(float* __restrict__ sink, int iters) {
     floatx4 acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
-    bf16x8 a, b;
+    constexpr int R = VARIED ? 8 : 1;
+    bf16x8 a[R], b[R];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) { a[e] = (bf16_t)(float)((threadIdx.x + e) & 7); b[e] = (bf16_t)(float)(e + 1); }
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if constexpr (VARIED) {
+                const uint32_t h1 = probe_hash(threadIdx.x * 977u + r * 131u + e * 7u + 1u), h2 = probe_hash(h1 + 12345u);
+                a[r][e] = (bf16_t)(((int)(h1 & 0xffff) - 32768) * (0.05f / 32768.f));
+                b[r][e] = (bf16_t)(((int)(h2 & 0xffff) - 32768) * (1.0f / 32768.f));
+            } else {
+                a[r][e] = (bf16_t)(float)((threadIdx.x + e) & 7);
+                b[r][e] = (bf16_t)(float)(e + 1);
+            }
+        }
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
+        for (int i = 0; i < 16; ++i)
+            acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i % R], b[(i * 3 + 1) % R], acc[i], 0, 0, 0);
     }
     float s = 0.f;
 #pragma unroll
@@ -51,8 +74,9 @@ TFF_API int tff_probe_stream_read(const void* src, size_t bytes, void* sink, int
 }
 
 // blocks x 4 waves, each issuing iters x 16 independent MFMAs: blocks * 4 * iters * 16 * 16384 flops.
-TFF_API int tff_probe_mfma(void* sink, int blocks, int iters, tff_stream_t stream) {
+TFF_API int tff_probe_mfma(void* sink, int blocks, int iters, int varied_operands, tff_stream_t stream) {
     TFF_REQUIRE(sink && blocks > 0 && iters > 0, "probe_mfma: bad arguments");
-    probe_mfma_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((float*)sink, iters);
+    if (varied_operands) probe_mfma_kernel<true><<<blocks, 256, 0, (hipStream_t)stream>>>((float*)sink, iters);
+    else probe_mfma_kernel<false><<<blocks, 256, 0, (hipStream_t)stream>>>((float*)sink, iters);
     return tff_check_launch("probe_mfma");
 }

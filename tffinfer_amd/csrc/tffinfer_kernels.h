@@ -180,6 +180,7 @@ TFF_API int tff_sample(const float* logits, int32_t* out, int rows, int V,
                        tff_stream_t stream);
 
 // Measuring kernels (csrc/probes.hip): stream `bytes` from src once; run blocks x 4 waves of
-// iters x 16 back-to-back 16x16x32 bfloat16 MFMAs.  The caller times them.
+// iters x 16 back-to-back 16x16x32 bfloat16 MFMAs, on operands that never change or
+// (varied_operands) that change from one instruction to the next.  The caller times them.
 TFF_API int tff_probe_stream_read(const void* src, size_t bytes, void* sink, int blocks, tff_stream_t stream);
-TFF_API int tff_probe_mfma(void* sink, int blocks, int iters, tff_stream_t stream);
+TFF_API int tff_probe_mfma(void* sink, int blocks, int iters, int varied_operands, tff_stream_t stream);

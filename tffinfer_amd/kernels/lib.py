@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 
 class KernelLibraryError(RuntimeError):
@@ -47,7 +47,7 @@ _SIGNATURES = {
     "tff_repetition_penalty": [_P, _I, _I, _P, _P, _P, _P],
     "tff_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
     "tff_probe_stream_read": [_P, _Z, _P, _I, _P],
-    "tff_probe_mfma": [_P, _I, _I, _P],
+    "tff_probe_mfma": [_P, _I, _I, _I, _P],
 }
 
 _lib = None
