@@ -18,13 +18,20 @@ import time
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense, published
 
-# layer sizes of the benchmark configuration (Qwen3-8B shape)
+# layer sizes of the benchmark configuration (Qwen3-8B shape) and of the two larger shapes
 QWEN3_8B = dict(
     architectures=["Qwen3ForCausalLM"], hidden_size=4096, num_hidden_layers=36,
     num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288,
     vocab_size=151936, max_position_embeddings=8192, rms_norm_eps=1e-6, rope_theta=1000000.0,
     tie_word_embeddings=False,
 )
+SHAPES = {
+    "8b": ("Qwen3-8B shape", QWEN3_8B),
+    "14b": ("Qwen3-14B shape", dict(QWEN3_8B, hidden_size=5120, num_hidden_layers=40, num_attention_heads=40,
+                                    intermediate_size=17408)),
+    "32b": ("Qwen3-32B shape", dict(QWEN3_8B, hidden_size=5120, num_hidden_layers=64, num_attention_heads=64,
+                                    intermediate_size=25600, max_position_embeddings=16384)),
+}
 
 
 def parse_args():
@@ -34,6 +41,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048)
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="8b",
+                    help="layer sizes: the benchmark configuration (8b) or one of the larger shapes")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
@@ -95,13 +104,18 @@ def measure_prefill(engine, gen, T, vocab, reps=5, warm=2):
     return statistics.median(times)
 
 
+def decode_slack(batch, context, chunk=2048):
+    """Steps the first request may decode while the last one still reads its prompt."""
+    return batch * (-(-context // chunk) + 1)
+
+
 def measure_decode(engine, gen, batch, context, steps, warmup, vocab):
     """Fills ``batch`` requests with ``context`` tokens each (untimed prefill),
     then times ``steps`` decode steps of the engine."""
     for _ in range(batch):
         # requests that finish their prompt early decode while the others still prefill
-        engine.add_request(random_prompt(gen, context, vocab), max_new_tokens=warmup + steps + batch + 8,
-                           ignore_eos=True)
+        engine.add_request(random_prompt(gen, context, vocab),
+                           max_new_tokens=warmup + steps + decode_slack(batch, context) + 8, ignore_eos=True)
     # untimed: prompts, up to the first decode-only step
     while any(r.num_pending > 1 for r in engine.scheduler.running) or engine.scheduler.waiting:
         engine.step()
@@ -136,7 +150,8 @@ def main():
         print(json.dumps({"ceilings": ops.measure_ceilings("cuda:0"),
                           "published": {"hbm_GBps": HBM_PEAK_GBS, "bf16_TFLOPs": MFMA_PEAK["bf16"] / 1e12}}))
         return
-    cfg = dict(QWEN3_8B)
+    shape_name, shape = SHAPES[args.shape]
+    cfg = dict(shape)
     L_full = cfg["num_hidden_layers"]
     L = args.layers or L_full
     cfg["num_hidden_layers"] = L
@@ -146,7 +161,7 @@ def main():
     model.init_random(args.seed, torch.bfloat16, "cuda:0", on_device=True)
     sync()
     max_batch = args.batch if args.no_points else max(args.batch, 64)
-    total_steps = args.steps + args.warmup + max_batch + 16
+    total_steps = args.steps + args.warmup + decode_slack(max_batch, args.context) + 16
     kv_tokens = max_batch * (args.context + total_steps + args.page_size) + args.prefill_tokens
     opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=kv_tokens, max_num_seqs=max_batch,
                         max_num_batched_tokens=max(4096, max_batch), prefill_chunk=2048,
@@ -182,7 +197,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic (seeded random weights and token ids)",
         "config": {
-            "model": "Qwen3-8B shape", "layers": L_full, "layers_run": L, "hidden": cfg["hidden_size"],
+            "model": shape_name, "layers": L_full, "layers_run": L, "hidden": cfg["hidden_size"],
             "q_heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": vocab,
             "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],

@@ -603,23 +603,36 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
 }
 
 // The tiled product's plan for M > 16: which tile, and into how many parts the blocks of a
-// tile split K.  Up to 64 rows: 64 x 128 tiles (two blocks to a CU), split so that the launch
-// has some 256 blocks.  Beyond: the cheapest of 256 x 256, 128 x 256, 128 x 128 and 64 x 128
-// tiles with 1 .. 8 parts by a small cost model: rounds of blocks over the CUs times a
-// block's work at the tile's measured rate (large tiles read fewer bytes of LDS per flop; a
-// last round that fills part of the machine costs between half and all of a full one), plus
-// the traffic of the partial sums (less where the caller takes them as they are).  Its constants were fitted to measurements of the four
-// products of an 8B model at 128 .. 2,048 rows on an MI355X, where it picks within a tenth of
-// the best of these candidates everywhere.
+// tile split K.  Up to 64 rows: 64 x 128 tiles (two blocks to a CU), K split so that the most
+// loaded CU has the least to stream.  Beyond: the cheapest of 256 x 256, 256 x 192, 128 x 256,
+// 128 x 128 and 64 x 128 tiles with 1 .. 8 parts by a small cost model: rounds of blocks over
+// the CUs times a block's work at the tile's measured rate (large tiles read fewer bytes of
+// LDS per flop; a last round that fills part of the machine costs between half and all of a
+// full one), plus the traffic of the partial sums (less where the caller takes them as they
+// are).  Its constants were fitted to measurements of the four products of an 8B model at
+// 128 .. 2,048 rows on an MI355X, where it picks within a tenth of the best of these
+// candidates everywhere.
 struct GemmPlan { int tile; int bn; int splits; };   // tile = rows of a block tile
 static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
     if (M <= 16) return {0, 0, 1};
     const int nk = (K + 63) / 64;
     if (M <= 64) {
+        // A stream of W: a CU pulls a block's k-tile of 64 (16 KB) in some 0.63 us whatever else
+        // runs, blocks go round the 256 CUs, and the most loaded CU sets the time.  Splitting K
+        // evens the load out (272 blocks are two rounds for 16 CUs and one for the rest; 1,088
+        // quarters are five rounds against 4.25) at the price of the partial sums' traffic and
+        // of some 4 us that a block spends before its first and after its last k-tile (two
+        // blocks of a CU overlap theirs).
         const long blocks = (N + 127) / 128;
-        int S = 1;
-        while (S < 8 && blocks * S * 2 <= 256 && nk / (S * 2) >= 4) S *= 2;
-        return {64, 128, S};
+        int best_s = 1;
+        double best_t = 1e30;
+        for (int S = 1; S <= 8; S *= 2) {
+            if (S > 1 && nk / S < 4) break;
+            double t = ceil(blocks * S / 256.0) * ceil((double)nk / S) * 0.63 + ceil(blocks * S / 512.0) * 4.0 + 1.0;
+            if (S > 1) t += keep ? (S - 1.0) * M * N * 4.0 / 4e6 : (double)S * M * N * 8.0 / 4e6 + 3.0;
+            if (t < best_t) { best_t = t; best_s = S; }
+        }
+        return {64, 128, best_s};
     }
     // rate: flops a microsecond that a CU sustains on blocks of this tile; slots: blocks a CU holds
     struct Cand { int bm, bn, slots; double rate; };
