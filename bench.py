@@ -50,6 +50,10 @@ def parse_args():
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="measure one phase only (for profiling); the JSON line then lacks the other")
+    ap.add_argument("--mixed", type=int, default=0, metavar="R",
+                    help="instead of the decode steps: R requests with prompt lengths uniform in [128, 4096], "
+                         "prompt portions of --chunk tokens beside decoding requests, 256 tokens generated each")
+    ap.add_argument("--chunk", type=int, default=512, help="prompt portion of the --mixed workload")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--ceilings", action="store_true",
                     help="measure streaming-read bandwidth and back-to-back MFMA rate on this machine and stop")
@@ -134,6 +138,28 @@ def measure_decode(engine, gen, batch, context, steps, warmup, vocab):
     return dt
 
 
+def measure_mixed(engine, gen, requests, vocab, new_tokens=256, lo=128, hi=4096):
+    """Continuous batching: all requests arrive at once, the scheduler admits them as
+    slots and pages allow, cuts prompts into portions and decodes the others beside them."""
+    import torch
+    lens = torch.randint(lo, hi + 1, (requests,), generator=gen).tolist()
+    for n in lens:
+        engine.add_request(random_prompt(gen, n, vocab), max_new_tokens=new_tokens, ignore_eos=True)
+    sync()
+    t0 = time.perf_counter()
+    steps = 0
+    while engine.has_work:
+        engine.step()
+        steps += 1
+    sync()
+    dt = time.perf_counter() - t0
+    st = engine.scheduler.stats
+    return {"requests": requests, "prompt_tokens": sum(lens), "generated_tokens": requests * new_tokens,
+            "seconds": round(dt, 3), "engine_steps": steps, "preemptions": st.preemptions,
+            "total_tokens_per_s": round((sum(lens) + requests * new_tokens) / dt, 1),
+            "generated_tokens_per_s": round(requests * new_tokens / dt, 1)}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -160,6 +186,16 @@ def main():
     model = build_model_skeleton(config_from_dict(cfg))
     model.init_random(args.seed, torch.bfloat16, "cuda:0", on_device=True)
     sync()
+    if args.mixed:
+        kv_tokens = args.mixed * (4096 + 256 + args.page_size)
+        opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=kv_tokens,
+                            max_num_seqs=args.mixed, max_num_batched_tokens=max(args.chunk + args.mixed, 1024),
+                            prefill_chunk=args.chunk, max_model_len=cfg["max_position_embeddings"],
+                            use_graphs=not args.no_graphs)
+        engine = LLMEngine(model, opt)
+        res = measure_mixed(engine, gen, args.mixed, vocab)
+        print(json.dumps({"workload": "mixed", "model": shape_name, "layers_run": L, "chunk": args.chunk, **res}))
+        return
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     total_steps = args.steps + args.warmup + decode_slack(max_batch, args.context) + 16
     kv_tokens = max_batch * (args.context + total_steps + args.page_size) + args.prefill_tokens
