@@ -85,19 +85,28 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     const int wm = wave / WGN, wn = wave % WGN;
     const int fr = lane & 15, fg = lane >> 4;
     // Blocks are handed to the eight XCDs in turn, and each XCD has an L2 of its own: block b
-    // of the launch runs on XCD b % 8.  Column tiles are therefore dealt to the XCDs (tile t to
-    // XCD t % 8), and the blocks an XCD runs one after the other walk the row tiles of one
-    // column tile before the next: a tile of W is fetched into one L2 only, and the (smaller) A
-    // is what every L2 holds.
-    // Row tiles are walked in groups of eight: with 32 blocks of an XCD in flight, four column
-    // tiles by eight row tiles share their fetches better than one column tile by 32 row tiles.
-    const int TM = (M + BM - 1) / BM;
+    // of the launch runs on XCD b % 8.  Row tiles are taken in groups of eight; within a group
+    // the tiles are numbered column tile by column tile, and XCD x works through the x-th
+    // eighth of that sequence one after the other: with 32 blocks of an XCD in flight these are
+    // four column tiles by eight row tiles, a tile of W is fetched into one L2 only (two at the
+    // seam of two eighths) and the (smaller) A is what every L2 holds.  A full group gives
+    // every XCD exactly TN tiles whatever TN is; only the last, smaller group pads the launch.
+    const int TM = (M + BM - 1) / BM, TN = (N + BN - 1) / BN;
     const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
-    const int per_group = (int)(gridDim.x >> 3) / TM * 8;   // blocks of an XCD per group of eight row tiles
-    const int grp = seq / per_group, in_grp = seq - grp * per_group;
-    const int grp_rows = min(8, TM - grp * 8);
-    const int tn = (in_grp / grp_rows) * 8 + xcd, tm = grp * 8 + in_grp % grp_rows;
-    if (tn * BN >= N) return;   // the launch is padded to whole groups of eight column tiles
+    const int full = (TM >> 3) * TN;           // blocks an XCD runs for the full groups
+    int grp, grp_rows, j;
+    if (seq < full) {
+        grp = seq / TN;
+        grp_rows = 8;
+        j = xcd * TN + (seq - grp * TN);
+    } else {
+        grp = TM >> 3;
+        grp_rows = TM & 7;
+        const int per = (grp_rows * TN + 7) >> 3;
+        j = xcd * per + (seq - full);
+        if (seq - full >= per || j >= grp_rows * TN) return;   // the launch is padded to eight equal shares
+    }
+    const int tn = j / grp_rows, tm = grp * 8 + j % grp_rows;
     const int m0 = tm * BM, n0 = tn * BN;
     const int NB = (N + 15) / 16;
     const int nk = (K + 32 * KPS - 1) / (32 * KPS);
@@ -289,7 +298,8 @@ static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int
     const int KB = (K + 31) / 32;
     constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
     if (splits <= 1 || !part) { splits = 1; part = nullptr; }
-    const long tiles = (long)((M + BM - 1) / BM) * (((N + BN - 1) / BN + 7) / 8 * 8);
+    const long TM = (M + BM - 1) / BM, TN = (N + BN - 1) / BN;
+    const long tiles = 8 * ((TM / 8) * TN + ((TM % 8) * TN + 7) / 8);   // eight equal shares, see the kernel
     TFF_REQUIRE(tiles < (1L << 31), "gemm: too many tiles for M=%d N=%d", M, N);
     const dim3 grid((unsigned)tiles, 1, splits);
     if (c_dtype == TFF_F32)
@@ -607,11 +617,10 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
 // loaded CU has the least to stream.  Beyond: the cheapest of 256 x 256, 256 x 192, 128 x 256,
 // 128 x 128 and 64 x 128 tiles with 1 .. 8 parts by a small cost model: rounds of blocks over
 // the CUs times a block's work at the tile's measured rate (large tiles read fewer bytes of
-// LDS per flop; a last round that fills part of the machine costs between half and all of a
-// full one), plus the traffic of the partial sums (less where the caller takes them as they
-// are).  Its constants were fitted to measurements of the four products of an 8B model at
-// 128 .. 2,048 rows on an MI355X, where it picks within a tenth of the best of these
-// candidates everywhere.
+// LDS per flop), plus the traffic of the partial sums (less where the caller takes them as
+// they are).  Its constants were fitted to measurements of the four products of the 8B, 14B
+// and 32B shapes at 96 .. 4,096 rows on an MI355X (156 cases, every tile with 1 .. 8 parts),
+// where its pick is within 7 % of the best candidate everywhere and 0.3 % from it on average.
 struct GemmPlan { int tile; int bn; int splits; };   // tile = rows of a block tile
 static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
     if (M <= 16) return {0, 0, 1};
@@ -636,8 +645,8 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
     }
     // rate: flops a microsecond that a CU sustains on blocks of this tile; slots: blocks a CU holds
     struct Cand { int bm, bn, slots; double rate; };
-    static const Cand cands[5] = {{256, 256, 1, 4.8e6}, {256, 192, 1, 4.5e6}, {128, 256, 1, 3.8e6},
-                                  {128, 128, 1, 2.6e6}, {64, 128, 2, 2.6e6}};
+    static const Cand cands[5] = {{256, 256, 1, 5.2e6}, {256, 192, 1, 4.4e6}, {128, 256, 1, 3.6e6},
+                                  {128, 128, 1, 2.6e6}, {64, 128, 2, 2.2e6}};
     GemmPlan best = {256, 256, 1};
     double best_t = 1e30;
     for (const Cand& c : cands)
@@ -645,14 +654,14 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
             if (glu && c.bn == 192) break;   // gate and up groups come in pairs: an even number a wave
             if (S > 1 && nk / S < 8) break;
             const double blocks = (double)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * S;
-            const double cap = 256.0 * c.slots;
-            const double rounds = ceil(blocks / cap);
-            const double last = (blocks - (rounds - 1.0) * cap) / cap;
-            const double round_us = 2.0 * c.bm * c.bn * ((double)K / S) * c.slots / c.rate;
-            double t = round_us * (rounds - 1.0 + 0.5 + 0.5 * last) + 3.0;
+            const double rounds = ceil(blocks / (256.0 * c.slots));
+            // a round: the blocks' work at the tile's rate plus some 3 us to fill the pipeline and
+            // store the tile; a last round that fills part of the machine takes as long as a full one
+            const double round_us = 2.0 * c.bm * c.bn * ((double)K / S) * c.slots / c.rate + 3.0;
+            double t = round_us * rounds + 3.0;
             // the partial sums: written, read and added by a second kernel, or (kept) read by the
             // consumer in place of one plane
-            if (S > 1) t += keep ? (S - 1.0) * M * N * 4.0 / 4e6 : (double)S * M * N * 4.0 / 2e6 + 3.0;
+            if (S > 1) t += keep ? (S - 1.0) * M * N * 4.0 / 4e6 : (double)S * M * N * 4.0 / 3e6 + 3.0;
             if (t < best_t) { best_t = t; best = {c.bm, c.bn, S}; }
         }
     return best;
