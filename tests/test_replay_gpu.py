@@ -44,6 +44,21 @@ def test_replay_modes(model_dirs, name, dtype, mode):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,ps", [("B", 24), ("C", 40)])
+def test_replay_with_pages_that_are_no_power_of_two(model_dirs, name, ps, dtype):
+    """The matrix-core attention takes pages of a power of two of tokens; with other page sizes
+    the bfloat16 engine runs the general attention kernel, and nothing else changes."""
+    from tffinfer_amd.kernels import ops
+    assert not ops.mfma_attention_supported(torch.bfloat16, 128, ps)
+    model_dir = model_dirs[name]
+    reqs = requests_for(name, model_dir)
+    steps = rl.trace_mixed(reqs)
+    runner = make_runner(model_dir, dtype, ps, rl.max_live_tokens(steps, unit=ps) // ps)
+    results = rl.run_steps_in_process(runner, steps)
+    rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(model_dirs, tmp_path, dtype):
     """The program itself, as a user calls it: mixed trace, files and 'done' lines."""
     model_dir = model_dirs["B"]

@@ -32,13 +32,15 @@ typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 // s_waitcnt immediate: vmcnt = 0, the other counters untouched
 constexpr int vmcnt_imm0() { return (7 << 4) | (15 << 8); }
 
-// Page and slot of a key; a shift and a mask when the page size is a power of two
-// (page_shift >= 0), a division otherwise (the GPU has no integer divider).
+// Page and slot of a key: a shift and a mask.  These kernels take pages of a power of two of
+// tokens only (the GPU has no integer divider); other page sizes run on the general kernel.
 __device__ __forceinline__ int page_index(int j, int page_size, int page_shift) {
-    return page_shift >= 0 ? (j >> page_shift) : j / page_size;
+    (void)page_size;
+    return j >> page_shift;
 }
 __device__ __forceinline__ int page_slot(int j, int page_size, int page_shift) {
-    return page_shift >= 0 ? (j & (page_size - 1)) : j % page_size;
+    (void)page_shift;
+    return j & (page_size - 1);
 }
 
 template <int DT, int NQT>
@@ -421,16 +423,24 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
         }
     }
 
-    // the page numbers of this wave's keys
+    // The page numbers of this wave's keys come from LDS, always: a lookup in the table itself
+    // is a memory load, and to wait for it is to wait for every key and value load issued
+    // before it, one round trip to HBM after the other.  Keys beyond what ATTN_WAVE_BT pages
+    // hold are worked through in segments, each with its own page numbers in LDS.
+    const int seg_steps = max(1, ((ATTN_WAVE_BT - 1) * page_size) >> 5);
     int pi0 = 0;
-    bool bt_in_lds = false;
-    if (s_begin < s_end) {
-        pi0 = page_index(kb0 + s_begin * 32, page_size, page_shift);
-        const int pi1 = page_index(min(kmax, kb0 + s_end * 32 - 1), page_size, page_shift);
-        bt_in_lds = pi1 - pi0 < ATTN_WAVE_BT;
-        if (bt_in_lds)
-            for (int i = lane; i <= pi1 - pi0; i += 64) bt_lds[i] = bt[pi0 + i];
+    // the page the token's own key and value go to, read now: later it would be waited for
+    // behind the first keys and values
+    int new_page = 0;
+    if constexpr (FUSED) {
+        if (owns_new) new_page = bt[page_index(P, page_size, page_shift)];
     }
+    auto fill_pages = [&](int seg0, int seg1) {
+        pi0 = page_index(kb0 + seg0 * 32, page_size, page_shift);
+        const int pi1 = page_index(min(kmax, kb0 + seg1 * 32 - 1), page_size, page_shift);
+        for (int i = lane; i <= pi1 - pi0; i += 64) bt_lds[i] = bt[pi0 + i];
+    };
+    if (s_begin < s_end) fill_pages(s_begin, min(s_end, s_begin + seg_steps));
     __syncthreads();
 
     bf16x8 qf[KS];
@@ -470,8 +480,7 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
     bf16x8 kf[RING][2][KS];   // [ring slot][key tile][k-step]
     bf16x8 vf[RING][DT];
 
-#define TFF_WAVE_PAGE(j) (bt_in_lds ? bt_lds[page_index((j), page_size, page_shift) - pi0]          \
-                                    : bt[page_index((j), page_size, page_shift)])
+#define TFF_WAVE_PAGE(j) bt_lds[page_index((j), page_size, page_shift) - pi0]
 #define TFF_WAVE_LOAD(buf, step)                                                                    \
     {                                                                                               \
         const int kb_ = kb0 + (step) * 32;                                                          \
@@ -549,44 +558,52 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
             oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[buf][dt], pv_, oacc[dt], 0, 0, 0); \
     }
 
-    if (s_begin < s_end) {
+    for (int seg0 = s_begin; seg0 < s_end; seg0 += seg_steps) {
+        const int seg1 = min(s_end, seg0 + seg_steps);
+        if (seg0 > s_begin) {
+            __syncthreads();            // the segment before is read
+            fill_pages(seg0, seg1);
+            __syncthreads();
+        }
         // steps past the end load the last step again and are not used
 #pragma unroll
-        for (int u = 0; u < RING; ++u) TFF_WAVE_LOAD(u, min(s_begin + u, s_end - 1))
+        for (int u = 0; u < RING; ++u) TFF_WAVE_LOAD(u, min(seg0 + u, seg1 - 1))
         if constexpr (FUSED) {   // while the first keys and values travel
-            if (has_norm || has_rope) norm_rope_fragments<DT>(qf, has_norm, fz_lds, fz.eps, has_rope, fz_lds + 2 * D, fz.pairing, kg);
-            if (owns_new) {
-                norm_rope_fragments<DT>(knew, has_norm, fz_lds + D, fz.eps, has_rope, fz_lds + 2 * D, fz.pairing, kg);
-                if (col0 == 0) {
-                    const int page = TFF_WAVE_PAGE(P);
-                    const int slot = page_slot(P, page_size, page_shift);
-                    if (qc == 0) {
-                        bf16_t* kd = fz.k_write + (((size_t)page * nkv + g) * page_size + slot) * D;
+            if (seg0 == s_begin) {
+                if (has_norm || has_rope) norm_rope_fragments<DT>(qf, has_norm, fz_lds, fz.eps, has_rope, fz_lds + 2 * D, fz.pairing, kg);
+                if (owns_new) {
+                    norm_rope_fragments<DT>(knew, has_norm, fz_lds + D, fz.eps, has_rope, fz_lds + 2 * D, fz.pairing, kg);
+                    if (col0 == 0) {
+                        const int page = new_page;
+                        const int slot = page_slot(P, page_size, page_shift);
+                        if (qc == 0) {
+                            bf16_t* kd = fz.k_write + (((size_t)page * nkv + g) * page_size + slot) * D;
 #pragma unroll
-                        for (int ks = 0; ks < KS; ++ks) {
-                            const int e = ks * 32 + kg * 8;
-                            if (e < D) *reinterpret_cast<uint4*>(kd + e) = *reinterpret_cast<const uint4*>(&knew[ks]);
+                            for (int ks = 0; ks < KS; ++ks) {
+                                const int e = ks * 32 + kg * 8;
+                                if (e < D) *reinterpret_cast<uint4*>(kd + e) = *reinterpret_cast<const uint4*>(&knew[ks]);
+                            }
                         }
-                    }
-                    if (kg == 0) {
-                        bf16_t* vd = fz.v_write + ((size_t)page * nkv + g) * D * page_size + slot;
+                        if (kg == 0) {
+                            bf16_t* vd = fz.v_write + ((size_t)page * nkv + g) * D * page_size + slot;
 #pragma unroll
-                        for (int dt = 0; dt < DT; ++dt) vd[(size_t)(dt * 16 + qc) * page_size] = vnew[dt];
+                            for (int dt = 0; dt < DT; ++dt) vd[(size_t)(dt * 16 + qc) * page_size] = vnew[dt];
+                        }
                     }
                 }
             }
         }
-        int s = s_begin;
-        for (; s_end - s > RING; s += RING) {
+        int s = seg0;
+        for (; seg1 - s > RING; s += RING) {
 #pragma unroll
             for (int u = 0; u < RING; ++u) {
                 TFF_WAVE_COMPUTE(u, s + u)
-                TFF_WAVE_LOAD(u, min(s + u + RING, s_end - 1))
+                TFF_WAVE_LOAD(u, min(s + u + RING, seg1 - 1))
             }
         }
 #pragma unroll
         for (int u = 0; u < RING; ++u)
-            if (s + u < s_end) {
+            if (s + u < seg1) {
                 if constexpr (FUSED) {
                     if (owns_new && s + u == s_end - 1) TFF_WAVE_PATCH(u, s + u)
                 }
@@ -784,12 +801,12 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
     const int kmax = P + tl_last;
     const int kb0 = (kmin / 32) * 32;
     const int nsteps = (kmax - kb0) / 32 + 1;
-    // the block's part of the block table, once
-    const int pg0 = page_index(kb0, page_size, page_shift);
-    const int npg = page_index(kmax, page_size, page_shift) - pg0 + 1;
-    const bool bt_in_lds = npg <= ATTN_BT_LDS;
-    if (bt_in_lds)
-        for (int i = tid; i < npg; i += 64 * NWT) pages[i] = bt[pg0 + i];
+    // The page numbers of the block's keys come from LDS, always (a lookup in the table itself
+    // is a memory load, and to wait for it is to wait for every copy in flight).  Keys beyond
+    // what ATTN_BT_LDS pages hold are worked through in segments, each with its own page numbers
+    // in LDS and a pipeline of copies of its own.
+    const int seg_steps = max(KGRP, ((((ATTN_BT_LDS - 1) * page_size) >> 5) / KGRP) * KGRP);
+    int pg0 = 0;
 
     bf16x8 qf[NQT][KS];
 #pragma unroll
@@ -812,10 +829,12 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) oacc[t][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
-    __syncthreads();   // pages[] is written
+    // q is waited for here, once: the compiler does not see the copies below (they are inline
+    // assembly), so a wait for q that it placed inside the loop would be a wait for all copies
+    // in flight, in every iteration.
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm0());
 
-#define ATTN_PAGE(j) (bt_in_lds ? pages[page_index((j), page_size, page_shift) - pg0] \
-                                : bt[page_index((j), page_size, page_shift)])
+#define ATTN_PAGE(j) pages[page_index((j), page_size, page_shift) - pg0]
     // fragment f of a slice: f < KFR is key tile f / KS, k-step f % KS; else value tile f - KFR
     // Every wave issues LPW copies per slice, also past the last slice (clamped to it) and past
     // the last fragment (a second copy of it): the count in flight is then the same for every
@@ -826,7 +845,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
         _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                           \
             const int F = min(wave_all + NWT * j, FRT - 1);                                         \
             const int f = F % FR;                                                                   \
-            const int kb_ = kb0 + min((step) * KGRP + F / FR, nsteps - 1) * 32;                     \
+            const int kb_ = kb0 + min(seg0 + (step) * KGRP + F / FR, seg1 - 1) * 32;                \
             {                                                                                       \
                 const bf16_t* g_;                                                                   \
                 if (f < KFR) {                                                                      \
@@ -864,15 +883,27 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
         t_max_lo[t] = mx;
     }
 
+    for (int seg0 = 0; seg0 < nsteps; seg0 += seg_steps) {
+    const int seg1 = min(nsteps, seg0 + seg_steps);
+    if (seg0 > 0) {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm0());   // the segment before: its copies past the end have landed,
+        __syncthreads();                            // its slices and page numbers are read
+    }
+    pg0 = page_index(kb0 + seg0 * 32, page_size, page_shift);
+    {
+        const int npg = page_index(min(kmax, kb0 + seg1 * 32 - 1), page_size, page_shift) - pg0 + 1;
+        for (int i = tid; i < npg; i += 64 * NWT) pages[i] = bt[pg0 + i];
+    }
+    __syncthreads();   // pages[] is written
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) ATTN_ISSUE(s)
-    const int nsup = (nsteps + KGRP - 1) / KGRP;
+    const int nsup = (seg1 - seg0 + KGRP - 1) / KGRP;
     for (int s = 0; s < nsup; ++s) {
         __builtin_amdgcn_s_waitcnt(attn_vmcnt_imm((STAGES - 2) * LPW));   // this wave's copies of stage s are in
         __syncthreads();                            // ... and the other waves'; stage s - 1 is read
         ATTN_ISSUE(s + STAGES - 1)                  // into the stage of step s - 1
-        if (KGRP > 1 && s * KGRP + kgi >= nsteps) continue;   // past the last slice: nothing for this group
-        const int kb = kb0 + (s * KGRP + kgi) * 32;
+        if (KGRP > 1 && seg0 + s * KGRP + kgi >= seg1) continue;   // past the last slice: nothing for this group
+        const int kb = kb0 + (seg0 + s * KGRP + kgi) * 32;
         const bf16_t* st = smem + ((s % STAGES) * FRT + kgi * FR) * 512;
         floatx4 sacc[NQT][2];
 #pragma unroll
@@ -933,6 +964,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
                 oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfr, pf[t], oacc[t][dt], 0, 0, 0);
         }
     }
+    }   // segments
 #undef ATTN_ISSUE
 #undef ATTN_PAGE
     __builtin_amdgcn_s_waitcnt(vmcnt_imm0());   // the copies past the end must not outlive the block
@@ -994,9 +1026,8 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
                        int tiles_per_entry, int cols_per_wave,
                        int splits, int nq, int nkv, int page_size, int window, float scale,
                        int T_total, hipStream_t s, const AttnFuse* fuse = nullptr, int key_groups = 2) {
-    int page_shift = -1;
-    if ((page_size & (page_size - 1)) == 0)
-        for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
+    int page_shift = 0;   // the page size is a power of two (tff_attention_mfma_supported)
+    while ((1 << page_shift) < page_size) ++page_shift;
     if (cols_per_wave == 128) {   // blocks of eight waves that share their keys through LDS
         // Two groups of eight waves that take every other slice, where LDS holds their stages:
         // half as many slices one after the other for a block, which is what counts when there
@@ -1040,7 +1071,7 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
 }
 
 TFF_API int tff_attention_mfma_supported(int d, int page_size) {
-    if (page_size <= 0 || page_size % 8) return 0;
+    if (page_size < 8 || (page_size & (page_size - 1))) return 0;   // a power of two, at least 8
     switch (d) {
         case 16: case 32: case 48: case 64: case 80: case 96: case 112: case 128: case 192: case 256:
             return 1;

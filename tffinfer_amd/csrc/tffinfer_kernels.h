@@ -121,7 +121,7 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out,
 // values in LDS; block b works through items block_items[b] ..
 // block_items[b + 1] of the work table (block_items null: item b); key_groups 2 (head sizes
 // up to 128): a block is two groups of eight waves that take every other slice, 1: one group.  Head sizes 16..128 in steps of
-// 16, 192 and 256; pages a multiple of 8; values transposed in their pages.
+// 16, 192 and 256; pages of a power of two of tokens, at least 8; values transposed in their pages.
 TFF_API int tff_attention_mfma_supported(int d, int page_size);
 TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* part_o, float* part_ml,
                                const void* k_cache, const void* v_cache,
