@@ -413,35 +413,47 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
     const bool owns_new = FUSED && fz.k_write != nullptr && s_begin < s_end && s_end == nsteps && fz.slot_mapping[tok0] >= 0;
     const bool has_norm = FUSED && fz.q_weight != nullptr, has_rope = FUSED && fz.cos_sin != nullptr;
 
-    if constexpr (FUSED) {
-        for (int i = lane; i < D; i += 64) {
-            if (has_norm) {
-                fz_lds[i] = fz.q_weight[i];
-                fz_lds[D + i] = fz.k_weight[i];
-            }
-            if (has_rope) fz_lds[2 * D + i] = fz.cos_sin[(size_t)P * D + i];
-        }
-    }
-
     // The page numbers of this wave's keys come from LDS, always: a lookup in the table itself
     // is a memory load, and to wait for it is to wait for every key and value load issued
     // before it, one round trip to HBM after the other.  Keys beyond what ATTN_WAVE_BT pages
     // hold are worked through in segments, each with its own page numbers in LDS.
     const int seg_steps = max(1, ((ATTN_WAVE_BT - 1) * page_size) >> 5);
     int pi0 = 0;
-    // the page the token's own key and value go to, read now: later it would be waited for
-    // behind the first keys and values
-    int new_page = 0;
+    auto fill_pages = [&](int seg0, int seg1, int from) {
+        pi0 = page_index(kb0 + seg0 * 32, page_size, page_shift);
+        const int pi1 = page_index(min(kmax, kb0 + seg1 * 32 - 1), page_size, page_shift);
+        for (int i = from + lane; i <= pi1 - pi0; i += 64) bt_lds[i] = bt[pi0 + i];
+    };
+    // Everything the wave needs before its first keys is asked for at once, the page numbers
+    // first (loads come back in the order they were issued, so the wait for the page numbers
+    // is a wait for nothing else): one round trip instead of one per table.  What is not needed
+    // for the addresses of the keys (norm weights, angles, the raw q, k and v) is put to use
+    // after the first keys and values are on their way.
+    int new_page = 0, first_page = 0, first_count = 0;
+    if (s_begin < s_end) {
+        pi0 = page_index(kb0 + s_begin * 32, page_size, page_shift);
+        first_count = page_index(min(kmax, kb0 + min(s_end, s_begin + seg_steps) * 32 - 1), page_size, page_shift) - pi0 + 1;
+        if (lane < first_count) first_page = bt[pi0 + lane];
+    }
     if constexpr (FUSED) {
         if (owns_new) new_page = bt[page_index(P, page_size, page_shift)];
     }
-    auto fill_pages = [&](int seg0, int seg1) {
-        pi0 = page_index(kb0 + seg0 * 32, page_size, page_shift);
-        const int pi1 = page_index(min(kmax, kb0 + seg1 * 32 - 1), page_size, page_shift);
-        for (int i = lane; i <= pi1 - pi0; i += 64) bt_lds[i] = bt[pi0 + i];
-    };
-    if (s_begin < s_end) fill_pages(s_begin, min(s_end, s_begin + seg_steps));
-    __syncthreads();
+    constexpr int FZN = FUSED ? (D + 63) / 64 : 1;
+    float fz_q[FZN], fz_k[FZN], fz_cs[FZN];
+    if constexpr (FUSED) {
+#pragma unroll
+        for (int u = 0; u < FZN; ++u) {
+            const int i = lane + 64 * u;
+            fz_q[u] = fz_k[u] = fz_cs[u] = 0.f;
+            if (i < D) {
+                if (has_norm) {
+                    fz_q[u] = fz.q_weight[i];
+                    fz_k[u] = fz.k_weight[i];
+                }
+                if (has_rope) fz_cs[u] = fz.cos_sin[(size_t)P * D + i];
+            }
+        }
+    }
 
     bf16x8 qf[KS];
     {
@@ -471,6 +483,11 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
             for (int dt = 0; dt < DT; ++dt) vnew[dt] = vraw[dt * 16 + qc];
         }
     }
+
+    // the page numbers of the first segment: the first 64 came with the loads above
+    if (lane < first_count) bt_lds[lane] = first_page;
+    if (first_count > 64) fill_pages(s_begin, min(s_end, s_begin + seg_steps), 64);
+    __syncthreads();
 
     floatx4 oacc[DT];
 #pragma unroll
@@ -562,7 +579,7 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
         const int seg1 = min(s_end, seg0 + seg_steps);
         if (seg0 > s_begin) {
             __syncthreads();            // the segment before is read
-            fill_pages(seg0, seg1);
+            fill_pages(seg0, seg1, 0);
             __syncthreads();
         }
         // steps past the end load the last step again and are not used
@@ -570,6 +587,16 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
         for (int u = 0; u < RING; ++u) TFF_WAVE_LOAD(u, min(seg0 + u, seg1 - 1))
         if constexpr (FUSED) {   // while the first keys and values travel
             if (seg0 == s_begin) {
+#pragma unroll
+                for (int u = 0; u < FZN; ++u) {
+                    const int i = lane + 64 * u;
+                    if (i < D) {
+                        fz_lds[i] = fz_q[u];
+                        fz_lds[D + i] = fz_k[u];
+                        fz_lds[2 * D + i] = fz_cs[u];
+                    }
+                }
+                __syncthreads();
                 if (has_norm || has_rope) norm_rope_fragments<DT>(qf, has_norm, fz_lds, fz.eps, has_rope, fz_lds + 2 * D, fz.pairing, kg);
                 if (owns_new) {
                     norm_rope_fragments<DT>(knew, has_norm, fz_lds + D, fz.eps, has_rope, fz_lds + 2 * D, fz.pairing, kg);
