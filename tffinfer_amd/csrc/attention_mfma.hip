@@ -689,6 +689,13 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __r
         ms = ml[0];
         ls = ml[1];
     }
+    // the first splits' elements are asked for together with the maxima and sums, not after the
+    // reductions that need those: one trip to memory instead of two
+    constexpr int AHEAD = 16;
+    float po[AHEAD];
+#pragma unroll
+    for (int s = 0; s < AHEAD; ++s)
+        po[s] = (tid < d && s < splits) ? part_o[(((size_t)s * R_total + r) * nq + h) * d + tid] : 0.f;
     const float m = block_max(ms, red);
     const float ws = ms == -INFINITY ? 0.f : __expf(ms - m);
     w[tid] = ws;
@@ -696,8 +703,15 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __r
     const float inv = 1.0f / l;
     for (int e = tid; e < d; e += blockDim.x) {
         float acc = 0.f;
+        int s0 = 0;
+        if (e == tid) {   // (the thread's first element) splits in their order, as below
+#pragma unroll
+            for (int s = 0; s < AHEAD; ++s)
+                if (s < splits) acc = fmaf(po[s], w[s], acc);
+            s0 = AHEAD;
+        }
 #pragma unroll 8
-        for (int s = 0; s < splits; ++s)
+        for (int s = s0; s < splits; ++s)
             acc = fmaf(part_o[(((size_t)s * R_total + r) * nq + h) * d + e], w[s], acc);
         out[((size_t)t * nq + h) * d + e] = (bf16_t)(acc * inv);
     }
