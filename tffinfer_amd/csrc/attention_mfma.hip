@@ -880,28 +880,50 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
     // Every wave issues LPW copies per slice, also past the last slice (clamped to it) and past
     // the last fragment (a second copy of it): the count in flight is then the same for every
     // wave and iteration, and one constant wait covers the slice about to be read.
+    // What does not change from slice to slice is worked out once per copy: which fragment
+    // (the wave's index is made a scalar, so that the choice between a key and a value
+    // fragment is a branch of the whole wave and not two masked halves), the lane's key within
+    // the slice and its offset within a page; a slice then costs a page lookup and one
+    // multiply-add per copy.
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave_all);
+    const uint32_t page_stride = (uint32_t)nkv * page_size * D;      // elements of a page, K or V (the host checks that it fits)
+    const bf16_t* kbase = k_cache + (size_t)g * page_size * D;
+    const bf16_t* vbase = v_cache + (size_t)g * D * page_size;
+    const int vkmax = (kmax >> 3) << 3;
+    int cp_F[LPW], cp_sub[LPW], cp_key[LPW], cp_off[LPW];
+    bool cp_is_k[LPW];
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) {
+        const int F = min(wave_u + NWT * j, FRT - 1);
+        const int f = F % FR;
+        cp_F[j] = F;
+        cp_sub[j] = F / FR;
+        cp_is_k[j] = f < KFR;
+        if (f < KFR) {
+            const int kt = f / KS, ks = f - kt * KS;
+            cp_key[j] = (qc >> 2) * 8 + kt * 4 + (qc & 3);
+            cp_off[j] = min(ks * 32 + kg * 8, D - 8);
+        } else {
+            cp_key[j] = kg * 8;
+            cp_off[j] = ((f - KFR) * 16 + qc) * page_size;
+        }
+    }
 #define ATTN_ISSUE(step)                                                                            \
     {                                                                                               \
         const int st_ = (step) % STAGES;                                                            \
         _Pragma("unroll") for (int j = 0; j < LPW; ++j) {                                           \
-            const int F = min(wave_all + NWT * j, FRT - 1);                                         \
-            const int f = F % FR;                                                                   \
-            const int kb_ = kb0 + min(seg0 + (step) * KGRP + F / FR, seg1 - 1) * 32;                \
-            {                                                                                       \
-                const bf16_t* g_;                                                                   \
-                if (f < KFR) {                                                                      \
-                    const int kt = f / KS, ks = f - kt * KS;                                        \
-                    const int key = min(kb_ + (qc >> 2) * 8 + kt * 4 + (qc & 3), kmax);             \
-                    g_ = k_cache + (((size_t)ATTN_PAGE(key) * nkv + g) * page_size +                 \
-                                    page_slot(key, page_size, page_shift)) * D +                      \
-                         min(ks * 32 + kg * 8, D - 8);                                              \
-                } else {                                                                            \
-                    const int j0 = min(kb_ + kg * 8, (kmax / 8) * 8);                               \
-                    g_ = v_cache + (((size_t)ATTN_PAGE(j0) * nkv + g) * D + (f - KFR) * 16 + qc) * page_size + \
-                         page_slot(j0, page_size, page_shift);                                      \
-                }                                                                                   \
-                copy16_to_lds(g_, smem + (st_ * FRT + F) * 512);                                    \
+            const int kb_ = kb0 + min(seg0 + (step) * KGRP + cp_sub[j], seg1 - 1) * 32;             \
+            const bf16_t* g_;                                                                       \
+            if (cp_is_k[j]) {                                                                       \
+                const int key = min(kb_ + cp_key[j], kmax);                                         \
+                g_ = kbase + ((uint64_t)(uint32_t)ATTN_PAGE(key) * page_stride +                    \
+                              (uint32_t)(page_slot(key, page_size, page_shift) * D + cp_off[j]));   \
+            } else {                                                                                \
+                const int j0 = min(kb_ + cp_key[j], vkmax);                                         \
+                g_ = vbase + ((uint64_t)(uint32_t)ATTN_PAGE(j0) * page_stride +                     \
+                              (uint32_t)(cp_off[j] + page_slot(j0, page_size, page_shift)));        \
             }                                                                                       \
+            copy16_to_lds(g_, smem + (st_ * FRT + cp_F[j]) * 512);                                  \
         }                                                                                           \
     }
 
@@ -1136,7 +1158,8 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                 "attention_mfma: %d query heads are not a multiple of %d key heads", nq, nkv);
     TFF_REQUIRE(tff_attention_mfma_supported(d, page_size),
                 "attention_mfma: head size %d with pages of %d is not supported by the matrix-core "
-                "kernel (head sizes 16..128 in steps of 16, 192, 256; pages a multiple of 8)", d, page_size);
+                "kernel (head sizes 16..128 in steps of 16, 192, 256; pages of a power of two, at least 8)", d, page_size);
+    TFF_REQUIRE((long)nkv * page_size * d < (1L << 31), "attention_mfma: a page of %d x %d x %d elements is too large", nkv, page_size, d);
     TFF_REQUIRE(q_stride >= nq * d && q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0,
                 "attention_mfma: query rows must be 16-byte aligned (stride %d)", q_stride);
     TFF_REQUIRE(cols_per_wave == 16 || cols_per_wave == 32 || cols_per_wave == 128,
