@@ -763,8 +763,8 @@ def test_attention_mfma_portions_beside_decoding_requests(nq, nkv, d, ps, window
 
 @pytest.mark.parametrize("splits", [1, 2, 5])
 def test_attention_mfma_decode_more_pages_than_the_wave_keeps(splits):
-    """A wave keeps 1024 page numbers at hand; with more pages in its run of keys it reads
-    them from the table in memory.  One key far back is made to dominate."""
+    """A wave keeps 1024 page numbers at hand; with more pages in its run of keys it works
+    through them in segments.  One key far back is made to dominate."""
     ops = _ops()
     nq, nkv, d, ps = 4, 2, 32, 8
     P, far = 8300, 77
@@ -780,6 +780,32 @@ def test_attention_mfma_decode_more_pages_than_the_wave_keeps(splits):
     out = ops.attention_mfma(q.reshape(2, nq * d).to(DEV), nq, nkv, d, kv, batch, 0, scale, splits=splits)
     _close(out.reshape(2, nq, d), ref, 1.5e-2, "decode attention over 1038 pages")
     assert torch.allclose(out.reshape(2, nq, d)[0, 0].float().cpu(), vs[0][far, 0].float(), atol=5e-2)
+
+
+@pytest.mark.parametrize("window", [0, 9000])
+def test_attention_mfma_portion_over_more_pages_than_a_block_keeps(window):
+    """A block keeps 2048 page numbers at hand; a portion late in a long prompt goes through
+    its keys in segments, each with page numbers and a pipeline of copies of its own.  One
+    key in the first segment and one in the last are made to stand out for two of the heads."""
+    ops = _ops()
+    nq, nkv, d, ps = 4, 2, 32, 8
+    P, n, far1, far2 = 17300, 40, 131, 16900
+    batch, kv, ks, vs, positions, token_req = _fake_step([(P, n)], ps, nkv, d, torch.bfloat16, seed=33)
+    assert (P + n) // ps > 2048
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(n, nq, d, generator=g).to(torch.bfloat16)
+    for far, (t, h) in ((far1, (3, 0)), (far2, (20, 3))):
+        kfar = (30 * q[t, h].float() / q[t, h].float().norm()).to(torch.bfloat16)
+        kv.k_cache[int(kv.block_tables[0, far // ps]), h // 2, far % ps] = kfar.to(DEV)
+        ks[0][far, h // 2] = kfar
+    scale = 1 / math.sqrt(d)
+    ref = _attn_ref(q, ks[0], vs[0], positions, window, scale)
+    out = ops.attention_mfma(q.reshape(n, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale)
+    _close(out.reshape(n, nq, d), ref, 1.5e-2, "portion over 2,167 pages")
+    got = out.reshape(n, nq, d).float().cpu()
+    if window == 0:      # (with the window the first of the two keys is out of sight)
+        assert torch.allclose(got[3, 0], vs[0][far1, 0].float(), atol=5e-2)
+    assert torch.allclose(got[20, 3], vs[0][far2, 1].float(), atol=5e-2)
 
 
 def test_attention_mfma_far_key_and_window_edge():
