@@ -54,6 +54,8 @@ def parse_args():
                     help="instead of the decode steps: R requests with prompt lengths uniform in [128, 4096], "
                          "prompt portions of --chunk tokens beside decoding requests, 256 tokens generated each")
     ap.add_argument("--chunk", type=int, default=512, help="prompt portion of the --mixed workload")
+    ap.add_argument("--budget", type=int, default=0,
+                    help="tokens of a step of the --mixed workload (default: a portion beside every decoding request, at least 1,024)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--ceilings", action="store_true",
                     help="measure streaming-read bandwidth and back-to-back MFMA rate on this machine and stop")
@@ -189,7 +191,7 @@ def main():
     if args.mixed:
         kv_tokens = args.mixed * (4096 + 256 + args.page_size)
         opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=kv_tokens,
-                            max_num_seqs=args.mixed, max_num_batched_tokens=max(args.chunk + args.mixed, 1024),
+                            max_num_seqs=args.mixed, max_num_batched_tokens=args.budget or max(args.chunk + args.mixed, 1024),
                             prefill_chunk=args.chunk, max_model_len=cfg["max_position_embeddings"],
                             use_graphs=not args.no_graphs)
         engine = LLMEngine(model, opt)
