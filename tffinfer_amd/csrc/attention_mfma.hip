@@ -798,6 +798,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
     constexpr int STAGES = ATTN_STAGES;                      // stages in LDS: one in use, the rest in flight
     __shared__ __attribute__((aligned(1024))) bf16_t smem[STAGES * FRT * 512];
     __shared__ int32_t pages[ATTN_BT_LDS];
+    static_assert(ATTN_STAGES >= 3, "the barrier between reads and MFMAs needs the copies one slice further ahead");
     static_assert(KGRP == 1 || (size_t)STAGES * FRT * 1024 >= (size_t)NW * (DT * 1024 + 512),
                   "the merge of the key groups borrows the stages");
     const int tid = threadIdx.x, lane = tid & 63, wave_all = tid >> 6;
@@ -886,6 +887,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
     // the slice and its offset within a page; a slice then costs a page lookup and one
     // multiply-add per copy.
     const int wave_u = __builtin_amdgcn_readfirstlane(wave_all);
+    const unsigned smem_addr = (unsigned)(size_t)(lds_ptr_t)smem;    // where the stages begin in LDS
     const uint32_t page_stride = (uint32_t)nkv * page_size * D;      // elements of a page, K or V (the host checks that it fits)
     const bf16_t* kbase = k_cache + (size_t)g * page_size * D;
     const bf16_t* vbase = v_cache + (size_t)g * D * page_size;
@@ -923,7 +925,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
                 g_ = vbase + ((uint64_t)(uint32_t)ATTN_PAGE(j0) * page_stride +                     \
                               (uint32_t)(cp_off[j] + page_slot(j0, page_size, page_shift)));        \
             }                                                                                       \
-            copy16_to_lds(g_, smem + (st_ * FRT + cp_F[j]) * 512);                                  \
+            copy16_to_lds_at(g_, smem_addr + (unsigned)(st_ * FRT + cp_F[j]) * 1024u);              \
         }                                                                                           \
     }
 
@@ -961,13 +963,25 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) ATTN_ISSUE(s)
     const int nsup = (seg1 - seg0 + KGRP - 1) / KGRP;
+    // The barrier of a slice stands between the reads of its key fragments and their MFMAs: a
+    // wave arrives with its keys on the way and starts its MFMAs when the barrier opens.  The
+    // barrier of slice s makes slice s + 1 visible, so the copies are one slice further ahead.
+    __builtin_amdgcn_s_waitcnt(attn_vmcnt_imm((STAGES - 2) * LPW));   // this wave's copies of the first stage are in
+    __syncthreads();
     for (int s = 0; s < nsup; ++s) {
-        __builtin_amdgcn_s_waitcnt(attn_vmcnt_imm((STAGES - 2) * LPW));   // this wave's copies of stage s are in
-        __syncthreads();                            // ... and the other waves'; stage s - 1 is read
-        ATTN_ISSUE(s + STAGES - 1)                  // into the stage of step s - 1
-        if (KGRP > 1 && seg0 + s * KGRP + kgi >= seg1) continue;   // past the last slice: nothing for this group
-        const int kb = kb0 + (seg0 + s * KGRP + kgi) * 32;
+        const bool mine = !(KGRP > 1 && seg0 + s * KGRP + kgi >= seg1);   // past the last slice: nothing for this group
         const bf16_t* st = smem + ((s % STAGES) * FRT + kgi * FR) * 512;
+        bf16x8 kfr[2][KS];   // (read also where there is no slice for this group: the stage is there)
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                kfr[kt][ks] = *reinterpret_cast<const bf16x8*>(st + (kt * KS + ks) * 512 + lane * 8);
+        __builtin_amdgcn_s_waitcnt(attn_vmcnt_imm((STAGES - 3) * LPW));   // this wave's copies of stage s + 1 are in
+        asm volatile("s_barrier" ::: "memory");     // ... and the other waves'; stage s - 1 is read
+        ATTN_ISSUE(s + STAGES - 1)                  // into the stage of step s - 1
+        if (!mine) continue;
+        const int kb = kb0 + (seg0 + s * KGRP + kgi) * 32;
         floatx4 sacc[NQT][2];
 #pragma unroll
         for (int t = 0; t < NQT; ++t) sacc[t][0] = sacc[t][1] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -975,10 +989,9 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8 kf = *reinterpret_cast<const bf16x8*>(st + (kt * KS + ks) * 512 + lane * 8);
 #pragma unroll
                 for (int t = 0; t < NQT; ++t)
-                    sacc[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[t][ks], sacc[t][kt], 0, 0, 0);
+                    sacc[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kfr[kt][ks], qf[t][ks], sacc[t][kt], 0, 0, 0);
             }
         bf16x8 pf[NQT];
 #pragma unroll

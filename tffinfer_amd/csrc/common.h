@@ -99,6 +99,13 @@ __device__ __forceinline__ float rows_sum(float v) {
 // the compiler knows nothing of the copy; the kernels wait for their copies themselves
 // (s_waitcnt vmcnt(n), copies complete in the order they were issued) before the barrier that
 // lets other waves read them.
+// The same with the LDS address (bytes from the start of LDS) worked out by the caller.
+__device__ __forceinline__ void copy16_to_lds_at(const void* gptr, unsigned lds_wave_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_wave_addr)), "v"(gptr)
+                 : "memory", "m0");
+}
 __device__ __forceinline__ void copy16_to_lds(const void* gptr, void* lds_wave_base) {
     const unsigned base = (unsigned)(size_t)(__attribute__((address_space(3))) void*)lds_wave_base;
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off"
