@@ -985,6 +985,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
         floatx4 sacc[NQT][2];
 #pragma unroll
         for (int t = 0; t < NQT; ++t) sacc[t][0] = sacc[t][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+        __builtin_amdgcn_s_setprio(1);   // a wave with its keys in registers goes before the softmax of the others
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -993,6 +994,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
                 for (int t = 0; t < NQT; ++t)
                     sacc[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kfr[kt][ks], qf[t][ks], sacc[t][kt], 0, 0, 0);
             }
+        __builtin_amdgcn_s_setprio(0);
         bf16x8 pf[NQT];
 #pragma unroll
         for (int t = 0; t < NQT; ++t) {
