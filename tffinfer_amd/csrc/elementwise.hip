@@ -402,8 +402,29 @@ __global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(
     const int h = valid ? hh : 0;
     const bool is_k = h >= nq;
     bf16_t* x = qkv + (size_t)t * (nq + 2 * nkv) * D + (size_t)h * D + l * 8;
+    // everything that does not depend on something loaded is asked for at once, the position
+    // (which the angles' address waits for) first
+    const int pos = cos_sin ? positions[t] : 0;
+    const int slot = is_k ? slot_mapping[t] : 0;
+    const float* w = is_k ? kw : qw;
+    float4 w0 = make_float4(1.f, 1.f, 1.f, 1.f), w1 = w0;
+    if (w) {
+        w0 = *reinterpret_cast<const float4*>(w + l * 8);
+        w1 = *reinterpret_cast<const float4*>(w + l * 8 + 4);
+    }
     union { uint4 u; bf16_t e[8]; } in, outv;
     in.u = *reinterpret_cast<const uint4*>(x);
+    float4 q0 = make_float4(0.f, 0.f, 0.f, 0.f), q1 = q0, q2 = q0, q3 = q0;
+    if (cos_sin) {
+        const float* cs = cos_sin + (size_t)pos * D;   // [pos][pair][cos, sin]
+        if (pairing == 0) {
+            const float4* c4 = reinterpret_cast<const float4*>(cs + (l % (LPH / 2)) * 16);
+            q0 = c4[0]; q1 = c4[1]; q2 = c4[2]; q3 = c4[3];
+        } else {
+            const float4* c4 = reinterpret_cast<const float4*>(cs + l * 8);
+            q0 = c4[0]; q1 = c4[1];
+        }
+    }
     float v[8];
     float ss = 0.f;
 #pragma unroll
@@ -413,20 +434,14 @@ __global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(
     }
 #pragma unroll
     for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-    const float* w = is_k ? kw : qw;
     if (w) {
         const float rr = rsqrtf(ss / (float)D + eps);
-        const float4 w0 = *reinterpret_cast<const float4*>(w + l * 8);
-        const float4 w1 = *reinterpret_cast<const float4*>(w + l * 8 + 4);
         v[0] = v[0] * rr * w0.x; v[1] = v[1] * rr * w0.y; v[2] = v[2] * rr * w0.z; v[3] = v[3] * rr * w0.w;
         v[4] = v[4] * rr * w1.x; v[5] = v[5] * rr * w1.y; v[6] = v[6] * rr * w1.z; v[7] = v[7] * rr * w1.w;
     }
     if (cos_sin) {
-        const float* cs = cos_sin + (size_t)positions[t] * D;   // [pos][pair][cos, sin]
         if (pairing == 0) {
             constexpr int HL = LPH / 2;
-            const float4* c4 = reinterpret_cast<const float4*>(cs + (l % HL) * 16);
-            const float4 q0 = c4[0], q1 = c4[1], q2 = c4[2], q3 = c4[3];
             const float c[8] = {q0.x, q0.z, q1.x, q1.z, q2.x, q2.z, q3.x, q3.z};
             const float sn[8] = {q0.y, q0.w, q1.y, q1.w, q2.y, q2.w, q3.y, q3.w};
             const bool first = l < HL;
@@ -437,8 +452,6 @@ __global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(
                 v[e] = first ? v[e] * c[e] - pv * sn[e] : pv * sn[e] + v[e] * c[e];
             }
         } else {
-            const float4* c4 = reinterpret_cast<const float4*>(cs + l * 8);
-            const float4 q0 = c4[0], q1 = c4[1];
             const float c[4] = {q0.x, q0.z, q1.x, q1.z};
             const float sn[4] = {q0.y, q0.w, q1.y, q1.w};
 #pragma unroll
@@ -455,7 +468,6 @@ __global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(
     if (!is_k) {
         *reinterpret_cast<uint4*>(x) = outv.u;
     } else {
-        const int slot = slot_mapping[t];
         if (slot < 0) return;
         const int page = slot / page_size, off = slot % page_size;
         bf16_t* kdst = k_cache + (((size_t)page * nkv + (h - nq)) * page_size + off) * D + l * 8;
