@@ -399,8 +399,13 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
     const int nsteps = (kmax - kb0) / 32 + 1;
     int s_begin = 0, s_end = nsteps;
     if (SPLIT) {
-        const int per = (nsteps + (int)gridDim.z - 1) / (int)gridDim.z;
-        s_begin = (int)blockIdx.z * per;
+        // The launch is sized for the longest context the engine allows; with shorter ones a run
+        // of keys is not made shorter than 256 keys as long as some 512 waves are left with
+        // work (the other waves of the launch end at once; their partial results are empty):
+        // runs of 128 keys were 7 % slower at 8 requests of 2,048 tokens.
+        const int busy = (512 + (int)(gridDim.x * gridDim.y) - 1) / (int)(gridDim.x * gridDim.y);
+        const int per = max((nsteps + (int)gridDim.z - 1) / (int)gridDim.z, min(8, (nsteps + busy - 1) / busy));
+        s_begin = min(nsteps, (int)blockIdx.z * per);
         s_end = min(nsteps, s_begin + per);
     }
 
