@@ -404,7 +404,8 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
         // work (the other waves of the launch end at once; their partial results are empty):
         // runs of 128 keys were 7 % slower at 8 requests of 2,048 tokens.
         const int busy = (512 + (int)(gridDim.x * gridDim.y) - 1) / (int)(gridDim.x * gridDim.y);
-        const int per = max((nsteps + (int)gridDim.z - 1) / (int)gridDim.z, min(8, (nsteps + busy - 1) / busy));
+        const int per = max(max((nsteps + (int)gridDim.z - 1) / (int)gridDim.z, min(8, (nsteps + busy - 1) / busy)),
+                            min(3, nsteps));   // (and never under 96 keys: more partial results cost more than they gain)
         s_begin = min(nsteps, (int)blockIdx.z * per);
         s_end = min(nsteps, s_begin + per);
     }
