@@ -43,218 +43,6 @@ __device__ __forceinline__ int page_slot(int j, int page_size, int page_shift) {
     return j & (page_size - 1);
 }
 
-template <int DT, int NQT>
-__global__ __launch_bounds__(64, (NQT == 2 ? 2 : 1)) void attn_mfma_kernel(
-    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, const bf16_t* __restrict__ k_cache,
-    const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int bt_stride,
-    const int32_t* __restrict__ cu_tokens, const int32_t* __restrict__ start_pos,
-    const int32_t* __restrict__ work, int tiles_per_entry, int nq, int nkv, int page_size,
-    int page_shift, int window, float scale, int T_total) {
-    constexpr int D = DT * 16;
-    constexpr int KS = (D + 31) / 32;
-    const int lane = threadIdx.x, qc = lane & 15, kg = lane >> 4;
-    int r, col0;
-    if (work) {
-        r = work[2 * blockIdx.x];
-        col0 = work[2 * blockIdx.x + 1];
-    } else {
-        r = blockIdx.x / tiles_per_entry;
-        col0 = (blockIdx.x % tiles_per_entry) * (16 * NQT);
-    }
-    const int g = blockIdx.y;
-    const int G = nq / nkv;
-    const int tok0 = cu_tokens[r];
-    const int n = cu_tokens[r + 1] - tok0;
-    const int P = start_pos[r];
-    const int ncols = n * G;
-    const int32_t* bt = block_tables + (size_t)r * bt_stride;
-
-    // this lane's column in each tile
-    int c_tok[NQT], c_head[NQT], c_pos[NQT], c_lo[NQT];
-    bool c_ok[NQT];
-#pragma unroll
-    for (int t = 0; t < NQT; ++t) {
-        const int c = col0 + t * 16 + qc;
-        c_ok[t] = c < ncols;
-        const int cc = c_ok[t] ? c : ncols - 1;
-        const int tl = cc / G;
-        c_tok[t] = tok0 + tl;
-        c_head[t] = g * G + (cc - tl * G);
-        c_pos[t] = c_ok[t] ? P + tl : -1;   // a missing column sees no key
-        c_lo[t] = window > 0 ? max(0, P + tl - window + 1) : 0;
-    }
-    // keys any column of this wave can see
-    const int tl_first = col0 / G;
-    const int tl_last = (min(col0 + NQT * 16, ncols) - 1) / G;
-    const int kmin = window > 0 ? max(0, P + tl_first - window + 1) : 0;
-    const int kmax = P + tl_last;
-    const int kb0 = (kmin / 32) * 32;
-    const int nsteps = (kmax - kb0) / 32 + 1;
-    const int s_begin = 0, s_end = nsteps;
-
-    // Q as second operand: lane (col, g) holds elements ks*32 + g*8 .. +8 of its column
-    bf16x8 qf[NQT][KS];
-#pragma unroll
-    for (int t = 0; t < NQT; ++t) {
-        const bf16_t* qp = q + (size_t)c_tok[t] * q_stride + (size_t)c_head[t] * D;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const int e = ks * 32 + kg * 8;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (c_ok[t] && e < D) v = *reinterpret_cast<const uint4*>(qp + e);
-            qf[t][ks] = *reinterpret_cast<bf16x8*>(&v);
-        }
-    }
-
-    floatx4 oacc[NQT][DT];
-    float m_run[NQT], l_run[NQT];
-#pragma unroll
-    for (int t = 0; t < NQT; ++t) {
-        m_run[t] = -INFINITY;
-        l_run[t] = 0.f;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) oacc[t][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
-    }
-
-    union VF { uint2 u[2]; bf16x8 v; };
-    bf16x8 kf[2][2][KS];   // [buffer][key tile][k-step]
-    VF vf[2][DT];
-
-#define TFF_ATTN_LOAD(buf, step)                                                                    \
-    {                                                                                               \
-        const int kb_ = kb0 + (step) * 32;                                                          \
-        _Pragma("unroll") for (int kt = 0; kt < 2; ++kt) {                                          \
-            /* rows past the last key repeat it; they are masked */                                 \
-            const int j_ = min(kb_ + kt * 16 + qc, kmax);                                           \
-            const int page_ = bt[page_index(j_, page_size, page_shift)];                            \
-            const bf16_t* kp_ = k_cache + (((size_t)page_ * nkv + g) * page_size + page_slot(j_, page_size, page_shift)) * D; \
-            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                     \
-                const int e_ = ks * 32 + kg * 8;                                                    \
-                uint4 v_ = make_uint4(0, 0, 0, 0);                                                  \
-                if (e_ < D) v_ = *reinterpret_cast<const uint4*>(kp_ + e_);                         \
-                kf[buf][kt][ks] = *reinterpret_cast<bf16x8*>(&v_);                                  \
-            }                                                                                       \
-        }                                                                                           \
-        /* value runs of this lane group: keys kb + g*4 .. +3 and kb + 16 + g*4 .. +3 */            \
-        const bf16_t* vrun_[2];                                                                     \
-        _Pragma("unroll") for (int kt = 0; kt < 2; ++kt) {                                          \
-            const int j0_ = min(kb_ + kt * 16 + kg * 4, (kmax / 4) * 4);                            \
-            const int page_ = bt[page_index(j0_, page_size, page_shift)];                           \
-            vrun_[kt] = v_cache + ((size_t)page_ * nkv + g) * D * page_size + page_slot(j0_, page_size, page_shift); \
-        }                                                                                           \
-        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                         \
-            const size_t eoff_ = (size_t)(dt * 16 + qc) * page_size;                                \
-            vf[buf][dt].u[0] = *reinterpret_cast<const uint2*>(vrun_[0] + eoff_);                   \
-            vf[buf][dt].u[1] = *reinterpret_cast<const uint2*>(vrun_[1] + eoff_);                   \
-        }                                                                                           \
-    }
-
-    // One column tile per wave (decoding, short portions): the loads of step s + 1 are issued
-    // before the arithmetic of step s.  Two tiles per wave need the registers for accumulators
-    // and rely on other waves of the SIMD to cover the latency instead.
-    constexpr bool PIPE = NQT == 1;
-    if (PIPE && s_begin < s_end) TFF_ATTN_LOAD(0, s_begin)
-    for (int s = s_begin; s < s_end; ++s) {
-        const int kb = kb0 + s * 32;
-        const int cur = PIPE ? ((s - s_begin) & 1) : 0;
-        if constexpr (PIPE) {
-            if (s + 1 < s_end) {
-                if (cur == 0) TFF_ATTN_LOAD(1, s + 1) else TFF_ATTN_LOAD(0, s + 1)
-            }
-        } else {
-            TFF_ATTN_LOAD(0, s)
-        }
-        floatx4 sacc[NQT][2];
-#pragma unroll
-        for (int t = 0; t < NQT; ++t) sacc[t][0] = sacc[t][1] = floatx4{0.f, 0.f, 0.f, 0.f};
-        if (cur == 0) {
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-                    for (int t = 0; t < NQT; ++t)
-                        sacc[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][kt][ks], qf[t][ks], sacc[t][kt], 0, 0, 0);
-        } else {
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-                    for (int t = 0; t < NQT; ++t)
-                        sacc[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][kt][ks], qf[t][ks], sacc[t][kt], 0, 0, 0);
-        }
-        bf16x8 pf[NQT];
-#pragma unroll
-        for (int t = 0; t < NQT; ++t) {
-            float sv[8];
-            float mt = -INFINITY;
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int j = kb + kt * 16 + kg * 4 + i;
-                    const bool vis = j >= c_lo[t] && j <= c_pos[t];
-                    const float x = vis ? sacc[t][kt][i] * scale : -INFINITY;
-                    sv[kt * 4 + i] = x;
-                    mt = fmaxf(mt, x);
-                }
-            mt = rows_max(mt);
-            const float m_new = fmaxf(m_run[t], mt);
-            const float alpha = m_new == -INFINITY ? 1.f : __expf(m_run[t] - m_new);
-            float ps = 0.f;
-            bf16x8 pv;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float p = sv[e] == -INFINITY ? 0.f : __expf(sv[e] - m_new);
-                ps += p;
-                pv[e] = (bf16_t)p;
-            }
-            pf[t] = pv;
-            l_run[t] = l_run[t] * alpha + ps;
-            m_run[t] = m_new;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                oacc[t][dt][0] *= alpha; oacc[t][dt][1] *= alpha;
-                oacc[t][dt][2] *= alpha; oacc[t][dt][3] *= alpha;
-            }
-        }
-        if (cur == 0) {
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int t = 0; t < NQT; ++t)
-                    oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[0][dt].v, pf[t], oacc[t][dt], 0, 0, 0);
-        } else {
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int t = 0; t < NQT; ++t)
-                    oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[1][dt].v, pf[t], oacc[t][dt], 0, 0, 0);
-        }
-    }
-#undef TFF_ATTN_LOAD
-
-#pragma unroll
-    for (int t = 0; t < NQT; ++t) {
-        float l = l_run[t];
-        l = rows_sum(l);
-        if (!c_ok[t]) continue;
-        {
-            const float inv = 1.0f / l;
-            bf16_t* op = out + ((size_t)c_tok[t] * nq + c_head[t]) * D;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                union { bf16_t h[4]; uint2 u; } pk;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) pk.h[i] = (bf16_t)(oacc[t][dt][i] * inv);
-                *reinterpret_cast<uint2*>(op + dt * 16 + kg * 4) = pk.u;
-            }
-        }
-    }
-}
-
 // ------------------------------------------------ one column tile per wave ---
 // Decoding (and portions of a few tokens): one wave, 16 columns.  What counts
 // here is bytes in flight.  The wave's part of the block table goes to LDS
@@ -1145,10 +933,7 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
     } else if (splits > 1) {
         attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
     } else {
-        if (cols_per_wave == 16)
-            attn_wave_kernel<DT, false, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
-        else
-            attn_mfma_kernel<DT, 2><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS);
+        attn_wave_kernel<DT, false, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
     }
 #undef TFF_ATTN_ARGS
     return tff_check_launch("attention_mfma");
@@ -1183,7 +968,7 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
     TFF_REQUIRE((long)nkv * page_size * d < (1L << 31), "attention_mfma: a page of %d x %d x %d elements is too large", nkv, page_size, d);
     TFF_REQUIRE(q_stride >= nq * d && q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0,
                 "attention_mfma: query rows must be 16-byte aligned (stride %d)", q_stride);
-    TFF_REQUIRE(cols_per_wave == 16 || cols_per_wave == 32 || cols_per_wave == 128,
+    TFF_REQUIRE(cols_per_wave == 16 || cols_per_wave == 128,
                 "attention_mfma: bad tile width %d", cols_per_wave);
     TFF_REQUIRE(cols_per_wave != 128 || (work && splits == 1),
                 "attention_mfma: blocks of 128 columns take a work table and no key split");

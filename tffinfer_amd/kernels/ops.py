@@ -580,8 +580,8 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
         launch(None, R * tiles, None, 0, tiles, 16, splits)
         return out
     # long portions: blocks that share their keys through LDS (128 columns); short ones: a wave
-    # of its own per 32 or 16 columns
-    cols = 128 if batch.max_new_tokens * G > 64 else (32 if batch.max_new_tokens * G > 16 else 16)
+    # of its own per 16 columns
+    cols = 128 if batch.max_new_tokens * G > 64 else 16
     which = "all"
     single = _entries(batch, "single")
     if cols == 128 and single and batch.max_context >= 256:
