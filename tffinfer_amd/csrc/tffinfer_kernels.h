@@ -109,8 +109,8 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out,
                                   int window, float scale, int dtype, int cache_dtype,
                                   tff_stream_t stream);
 
-// bfloat16 attention on the matrix cores.  A wave works on `cols_per_wave` (16
-// or 32) columns of one request and kv head; a column is a (token, q head of
+// bfloat16 attention on the matrix cores.  A wave works on `cols_per_wave` (16)
+// columns of one request and kv head; a column is a (token, q head of
 // the group) pair numbered token * G + head.  work != null: pairs (request,
 // first column) per wave; work == null: every request brings one token and
 // gets tiles_per_entry waves.  splits > 1 (entries of one token, 16 columns a
