@@ -103,7 +103,7 @@ def test_linear(M, N, K, dtype):
     _close(out_s, wide[:, :K].double().cpu() @ w.double().T, 2e-6 if dtype == torch.float32 else 2e-5, "strided")
 
 
-@pytest.mark.parametrize("M,N,K", [(40, 1024, 2056), (520, 264, 1544), (8, 64, 64)])
+@pytest.mark.parametrize("M,N,K", [(40, 1024, 2056), (520, 264, 1544), (8, 64, 64), (8, 5120, 8192), (16, 5120, 8200)])
 def test_linear_partial_sums_feed_the_norm(M, N, K):
     """Where the product splits K over blocks it can hand out the partial sums; the fused
     residual sum and norm adds them up itself, in order, to what the whole product gives."""
@@ -114,7 +114,12 @@ def test_linear_partial_sums_feed_the_norm(M, N, K):
     pw = ops.pack_weight(w.to(DEV))
     whole = ops.linear(x, pw, out_dtype=torch.float32)
     parts = ops.linear(x, pw, out_dtype=torch.float32, partials=True)
-    if M == 8:
+    # a few rows and 320 column groups: the whole product streams, the partial sums come from
+    # tiles that split K; the two kernels add in different orders
+    other_kernel = M <= 16 and N == 5120
+    same = (lambda a, b: torch.allclose(a.float(), b.float(), rtol=2e-2 if a.dtype == torch.bfloat16 else 1e-4,
+                                        atol=2e-2 if a.dtype == torch.bfloat16 else 1e-3)) if other_kernel else torch.equal
+    if M == 8 and not other_kernel:
         assert isinstance(parts, ops.PendingProduct)   # a few rows: run by whoever consumes it
         assert torch.equal(parts.run(), whole)
     else:
@@ -122,17 +127,17 @@ def test_linear_partial_sums_feed_the_norm(M, N, K):
         acc = parts[0].clone()
         for p in parts[1:]:
             acc += p
-        assert torch.equal(acc, whole)
+        assert same(acc, whole)
     resid = torch.randn(M, N, generator=g).to(DEV)
     nw = (1 + 0.1 * torch.randn(N, generator=g)).to(DEV)
     r1, r2 = resid.clone(), resid.clone()
     y1 = ops.add_rmsnorm(r1, whole, nw, 1e-6, torch.float32)
     y2 = ops.add_rmsnorm(r2, parts, nw, 1e-6, torch.float32)
-    assert torch.equal(r1, r2) and torch.equal(y1, y2)
+    assert same(r1, r2) and same(y1, y2)
     rows = torch.tensor([M - 1, 0], dtype=torch.int32, device=DEV)
     z1 = ops.add_rmsnorm(resid.clone(), whole, nw, 1e-6, torch.bfloat16, rows=rows)
     z2 = ops.add_rmsnorm(resid.clone(), parts, nw, 1e-6, torch.bfloat16, rows=rows)
-    assert torch.equal(z1, z2)
+    assert same(z1, z2)
 
 
 @pytest.mark.parametrize("glu", [False, True])
@@ -254,6 +259,11 @@ def test_gemm_plan():
         return r.value, c.value, s.value
 
     assert plan(8, 4096, 4096) == (0, 0, 1)
+    # a few rows, 320 column groups (two rounds for 64 CUs, one for the rest), partial sums wanted
+    # anyway and a weight large enough: tiles that split K instead of the streaming kernel
+    assert plan(8, 5120, 8192, keep=1)[:2] == (64, 128) and plan(8, 5120, 8192, keep=1)[2] > 1
+    assert plan(8, 5120, 8192) == (0, 0, 1) and plan(8, 5120, 5120, keep=1) == (0, 0, 1)
+    assert plan(8, 4096, 12288, keep=1) == (0, 0, 1)
     assert plan(64, 4096, 12288) == (64, 128, 8)
     assert plan(64, 151936, 4096) == (64, 128, 1)
     assert plan(2048, 24576, 4096, 1) == (256, 256, 1)

@@ -623,7 +623,16 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
 // where its pick is within 7 % of the best candidate everywhere and 0.3 % from it on average.
 struct GemmPlan { int tile; int bn; int splits; };   // tile = rows of a block tile
 static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
-    if (M <= 16) return {0, 0, 1};
+    // Up to 16 rows: the streaming kernel, a block per 16 columns, unless those blocks go badly
+    // round the 256 CUs (320 of them take as long as 512 would: N = 5120), the caller takes
+    // partial sums anyway and the weight is large enough for the gain (three eighths of its
+    // stream) to pay for the norm's own kernel, which the streaming kernel would have taken into
+    // its epilogue: then the tiles below, whose blocks split K as finely as it takes.
+    if (M <= 16) {
+        const int nb = (N + 15) / 16;
+        const double fill = (double)nb / (((nb + 255) / 256) * 256.0);
+        if (glu || !keep || fill >= 0.8 || (double)N * K < 40e6) return {0, 0, 1};
+    }
     const int nk = (K + 63) / 64;
     if (M <= 64) {
         // A stream of W: a CU pulls a block's k-tile of 64 (16 KB) in some 0.63 us whatever else
@@ -737,7 +746,7 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
             return launch_async_g<2, 4, 4, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         return launch_async_g<4, 4, 4, 4, 5, true, 1, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
     }
-    if (M <= 16) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, nullptr);
+    if (plan.tile == 0) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, nullptr);
     if (plan.tile == 64) {
         // few columns and no room for partial sums: the streaming kernel, whose blocks split K
         // among their waves

@@ -12,6 +12,7 @@ with a device dispatch; here the table has one entry per op and no dispatch.
 """
 from __future__ import annotations
 
+import ctypes
 import math
 
 import torch
@@ -280,6 +281,19 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return out
 
 
+_plan_cache: dict = {}
+
+
+def _plan_tile(L, M: int, N: int, K: int) -> int:
+    """Rows of the tile the product's plan takes when partial sums are kept (0: the streaming kernel)."""
+    key = (M, N, K)
+    if key not in _plan_cache:
+        r, c, s = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        _lib.check(L.tff_gemm_plan(M, N, K, 0, 1, ctypes.byref(r), ctypes.byref(c), ctypes.byref(s)))
+        _plan_cache[key] = r.value
+    return _plan_cache[key]
+
+
 def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
            out: torch.Tensor | None = None, partials: bool = False) -> torch.Tensor:
     """``x . weight^T`` for x [M, K] (rows may be strided) and weight [N, K]:
@@ -316,7 +330,9 @@ def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
     # some shapes (few columns for the rows) split K over blocks and need room for partial sums
     want = bool(partials and packed and out is None and out_dtype == torch.float32 and not glu_out)
     if want and M <= 16 and N % 8 == 0 and x.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0 and lda % 8 == 0:
-        return PendingProduct(x, weight)   # a few rows: the consumer runs it with its own work in the epilogue
+        if _plan_tile(L, M, N, K) == 0:
+            return PendingProduct(x, weight)   # a few rows: the consumer runs it with its own work in the epilogue
+        # (else the streaming kernel's blocks would go badly round the CUs: tiles that split K, partial sums kept)
     ws_bytes = (L.tff_gemm_workspace_bytes(M, N, K, dtype_code(x.dtype), 1 if glu_out else 0, 1 if want else 0)
                 if packed else 0)
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=x.device) if ws_bytes else None
