@@ -183,6 +183,10 @@ def main():
     L_full = cfg["num_hidden_layers"]
     L = args.layers or L_full
     cfg["num_hidden_layers"] = L
+    # a context beyond the shape's own limit: the limit grows with it (it sizes the rotation table only)
+    longest = args.context + args.steps + args.warmup + decode_slack(max(args.batch, 64), args.context) + 16
+    if not args.mixed and longest > cfg["max_position_embeddings"]:
+        cfg["max_position_embeddings"] = 1 << (longest - 1).bit_length()
     vocab = cfg["vocab_size"]
     gen = torch.Generator().manual_seed(args.seed)
     model = build_model_skeleton(config_from_dict(cfg))
@@ -198,7 +202,7 @@ def main():
         res = measure_mixed(engine, gen, args.mixed, vocab)
         print(json.dumps({"workload": "mixed", "model": shape_name, "layers_run": L, "chunk": args.chunk, **res}))
         return
-    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    max_batch = args.batch if (args.no_points or args.only) else max(args.batch, 64)
     total_steps = args.steps + args.warmup + decode_slack(max_batch, args.context) + 16
     kv_tokens = max_batch * (args.context + total_steps + args.page_size) + args.prefill_tokens
     opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=kv_tokens, max_num_seqs=max_batch,
