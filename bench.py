@@ -184,7 +184,7 @@ def main():
     L = args.layers or L_full
     cfg["num_hidden_layers"] = L
     # a context beyond the shape's own limit: the limit grows with it (it sizes the rotation table only)
-    longest = args.context + args.steps + args.warmup + decode_slack(max(args.batch, 64), args.context) + 16
+    longest = max(args.prefill_tokens, args.context + args.steps + args.warmup + decode_slack(max(args.batch, 64), args.context) + 16)
     if not args.mixed and longest > cfg["max_position_embeddings"]:
         cfg["max_position_embeddings"] = 1 << (longest - 1).bit_length()
     vocab = cfg["vocab_size"]
