@@ -1,0 +1,185 @@
+"""The engine's faster paths against the plain implementation: decode graphs
+through preemptions (a request that comes back to its graph row with other
+pages), and decode steps launched ahead of the tokens of the step in flight
+(with a request that ends on a stop token while a step is ahead, and one that
+is aborted then).  Every kept row of logits is compared with the plain logits
+of the engine's own sequence, and every chosen token with the plain sampler's
+choice from that row."""
+import pytest
+import torch
+
+from helpers import oracle_logits, random_tokens, read_config
+from test_generate_gpu import check_choices
+
+pytestmark = pytest.mark.gpu
+
+
+def drive(eng, arrivals, on_step=None):
+    """Steps the engine until nothing is left; ``arrivals`` maps a step number to the
+    requests (keyword arguments of add_request) that arrive before it."""
+    step = 0
+    pending = dict(arrivals)
+    while eng.has_work or pending:
+        if not eng.has_work and step not in pending:
+            step = min(pending)
+        for kw in pending.pop(step, []):
+            eng.add_request(**kw)
+        if on_step:
+            on_step(step)
+        eng.step()
+        eng.runner.cache.check()
+        step += 1
+        assert step < 2000
+
+
+def watch_graph_rows(eng):
+    """Counts the fills of a decode graph's row that find the same request id in the row but
+    other pages than the request holds now: it went away and came back."""
+    from tffinfer_amd.engine.graphs import DecodeTables
+    seen = {"returns": 0, "fills": 0}
+    inner = DecodeTables.fill
+
+    def fill(self, entries):
+        for r, e in enumerate(entries):
+            prev = self._row_state[r]
+            if prev is None or prev[0] != e.req:
+                continue
+            for gi, g in enumerate(self.cache.groups):
+                n = min(prev[-1][gi], len(self.cache.block_table(gi, e.req)))
+                if g.spec.window == 0 and list(self.block_table_row(gi, r)[:n]) != self.cache.block_table(gi, e.req)[:n]:
+                    seen["returns"] += 1
+        seen["fills"] += 1
+        return inner(self, entries)
+
+    return seen, fill
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_preempted_request_decodes_again_in_its_graph_row(model_dirs, dtype, name, monkeypatch):
+    """Three requests arrive one after the other on 11 pages of 8 tokens; the newest is
+    preempted while it decodes, computed again and decodes again in the graph row it had,
+    beside the same neighbours, with pages in another order."""
+    from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
+    from tffinfer_amd.engine.graphs import DecodeTables
+    d = model_dirs[name]
+    V = read_config(d)["vocab_size"]
+    lens, new, arrive = [12, 9, 26], [55, 36, 53], [0, 34, 19]
+    sc = [SamplingConfig(), SamplingConfig("random", temperature=0.8, seed=77), SamplingConfig()]
+    opt = EngineOptions(dtype=dtype, page_size=8, num_pages=11, max_num_seqs=3, max_num_batched_tokens=48,
+                        prefill_chunk=24, max_model_len=128, use_graphs=True, run_ahead=False)
+    eng = LLMEngine.from_model_dir(d, opt)
+    eng.keep_logits = True
+    seen, fill = watch_graph_rows(eng)
+    monkeypatch.setattr(DecodeTables, "fill", fill)
+    arrivals = {}
+    for i in range(3):
+        arrivals.setdefault(arrive[i], []).append(dict(
+            prompt_ids=random_tokens(lens[i], V, 300 + i), sampling=sc[i], max_new_tokens=new[i],
+            ignore_eos=True, request_id=i))
+    drive(eng, arrivals)
+    assert eng.scheduler.stats.preemptions > 0
+    assert seen["returns"] > 0, "no request came back to its row: the schedule misses the case"
+    for i in range(3):
+        r = eng.pop_result(i)
+        assert len(r.output) == new[i]
+        check_choices(d, r, dtype, sc[i])
+    assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_request_id_freed_and_used_again_on_a_graph_runner(model_dirs, dtype):
+    """At the step function's level: a request decodes through the graph, is freed, the same id
+    is added again while another request holds pages in between, and decodes again."""
+    from tffinfer_amd.engine import ModelRunner, StepEntry
+    from tffinfer_amd.models import load_model
+    from helpers import TOL, rel_err
+    d = model_dirs["A"]
+    V = read_config(d)["vocab_size"]
+    model = load_model(d, torch.float32 if dtype == "float32" else torch.bfloat16, "cuda:0")
+    rn = ModelRunner(model, page_size=8, num_pages=12, max_seqs=2, max_model_len=96, use_graphs=True)
+
+    def life(rid, toks, n_whole):
+        ref = oracle_logits(d, toks)
+        rn.add_request(rid)
+        out = rn.step([StepEntry(rid, toks[:n_whole], [n_whole - 1])])
+        assert rel_err(out[0], ref[n_whole - 1]) <= TOL[dtype]
+        for j in range(n_whole, len(toks)):
+            out = rn.step([StepEntry(rid, [toks[j]], [0])])       # one token: the graph
+            assert rel_err(out[0], ref[j]) <= TOL[dtype], (rid, j)
+        rn.cache.check()
+
+    first = random_tokens(40, V, 401)
+    life("a", first, 20)
+    rn.add_request("b")
+    rn.step([StepEntry("b", random_tokens(5, V, 402), [])])        # holds a page of its own
+    rn.free_request("a")
+    rn.step([StepEntry("b", random_tokens(9, V, 403), [])])        # and takes one of a's
+    life("a", random_tokens(40, V, 404), 34)                       # same id, as many pages, other ones
+    rn.free_request("a")
+    rn.free_request("b")
+    assert all(g.pool.num_used == 0 for g in rn.cache.groups)
+
+
+@pytest.mark.parametrize("dtype,use_graphs", [("float32", True), ("bfloat16", True), ("bfloat16", False),
+                                              ("float32", False)])
+def test_steps_launched_ahead_against_the_plain_implementation(model_dirs, dtype, use_graphs):
+    """Steps launched ahead, with kept logits: six requests of different lengths on four slots and a
+    pool that runs out; then the same with one request that stops on a token of its own choosing
+    while a step is ahead, and one that is aborted while a step is ahead."""
+    from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
+    d = model_dirs["B"]
+    V = read_config(d)["vocab_size"]
+    prompts = [random_tokens(n, V, 170 + n) for n in (3, 17, 31, 9, 26, 5)]
+    sc = [SamplingConfig("random", temperature=0.7, seed=30 + i) if i % 2 else SamplingConfig() for i in range(6)]
+    lens = [24, 7, 30, 16, 1, 21]
+    opt = EngineOptions(dtype=dtype, page_size=8, num_pages=24, max_num_seqs=4, max_num_batched_tokens=48,
+                        prefill_chunk=24, run_ahead=True, use_graphs=use_graphs)
+    eng = LLMEngine.from_model_dir(d, opt)
+    eng.keep_logits = True
+
+    def requests(eos_for_2=None):
+        return {0: [dict(prompt_ids=p, sampling=s, max_new_tokens=n, request_id=i,
+                         ignore_eos=not (i == 2 and eos_for_2 is not None),
+                         eos_token_id=eos_for_2 if i == 2 else None)
+                    for i, (p, s, n) in enumerate(zip(prompts, sc, lens))]}
+
+    drive(eng, requests())
+    assert eng.steps_ahead > 10
+    first = {}
+    for i in range(6):
+        r = first[i] = eng.pop_result(i)
+        assert len(r.output) == lens[i] and r.finish_reason == "length"
+        check_choices(d, r, dtype, sc[i])
+    assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
+
+    # request 2 stops at the token it chose as its 12th; request 0 is aborted while a step is ahead
+    eos = first[2].output[11]
+    aborted = {}
+
+    def on_step(step):
+        req0 = eng._requests.get(0)
+        if not aborted and eng._ahead is not None and req0 is not None and len(req0.output) >= 9:
+            assert any(p.request.id == 0 for p in eng._ahead.plan)    # a token of its is in flight
+            assert eng.abort(0)
+            aborted["at"] = len(req0.output)
+
+    before = eng.steps_ahead
+    drive(eng, requests(eos), on_step)
+    assert eng.steps_ahead > before + 10 and aborted
+    for i in range(6):
+        r = eng.pop_result(i)
+        if i == 0:
+            assert r.finish_reason == "abort" and len(r.output) == aborted["at"]
+            if dtype == "float32":     # the same choices whoever else is in the batch
+                assert r.output == first[0].output[:aborted["at"]]
+        elif i == 2:
+            assert r.finish_reason == "stop" and r.output[-1] == eos and eos not in r.output[:-1]
+            if dtype == "float32":
+                assert r.output == first[2].output[:first[2].output.index(eos) + 1]
+        else:
+            assert r.finish_reason == "length" and len(r.output) == lens[i]
+        assert len(r.logits) == len(r.output)
+        check_choices(d, r, dtype, sc[i])
+    assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
+    assert eng.runner.cache.slots.num_free == 4

@@ -50,6 +50,9 @@ class CacheGroup:
 class RequestCacheState:
     slot: int
     num_tokens: int = 0
+    #: unique to this stay of the request in the cache: a request that is released and added
+    #: again under the same id (preemption, an id used twice) gets another one
+    life: int = 0
 
 
 class CacheManager:
@@ -64,6 +67,7 @@ class CacheManager:
         self.max_seqs = int(max_seqs)
         self.slots = StateSlots(max_seqs)
         self.requests: dict = {}
+        self._lives = 0
         self.groups: list[CacheGroup] = []
         self._group_of_cache: dict[int, int] = {}
         self._state_specs: dict[int, StateSpec] = {}
@@ -121,6 +125,12 @@ class CacheManager:
     def slot(self, req) -> int:
         return self.requests[req].slot
 
+    def life(self, req) -> int:
+        """A number that no other stay of any request in this cache has had.  Whoever keeps
+        a copy of a request's block table keys it on this, never on the request's id alone:
+        the id comes back with other pages after a preemption."""
+        return self.requests[req].life
+
     def has_request(self, req) -> bool:
         return req in self.requests
 
@@ -139,7 +149,8 @@ class CacheManager:
         if req in self.requests:
             raise ValueError(f"request {req!r} is already live")
         slot = self.slots.acquire()
-        self.requests[req] = RequestCacheState(slot)
+        self._lives += 1
+        self.requests[req] = RequestCacheState(slot, life=self._lives)
         for g in self.groups:
             g.tables[req] = []
         for t in self.state_tensors.values():

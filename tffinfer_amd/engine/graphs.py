@@ -28,60 +28,57 @@ def _pad4(n: int) -> int:
     return (n + 3) & ~3
 
 
-class DecodeGraph:
-    def __init__(self, runner, bucket: int):
-        self._runner = weakref.ref(runner)   # the runner owns its graphs; no reference cycle
+def table_layout(bucket: int, widths: list[int]) -> tuple[list[int], int]:
+    """Offsets of the sections of a decode step's packed tables (the order of
+    build_step_batch) and their total length, for ``bucket`` rows."""
+    B = bucket
+    sizes = [B, B, B, B + 1, B, B, B, B, B]
+    for w in widths:
+        sizes += [B * w, B]
+    offs, total = [], 0
+    for n in sizes:
+        offs.append(total)
+        total += _pad4(n)
+    return offs, total
+
+
+class DecodeTables:
+    """The host side of a decode graph: the packed tables of a step of one token
+    per request, kept between steps in one int32 array so that a step writes
+    only what changed.  Pure host code (numpy), no device.
+
+    A row remembers whose block table it holds as (request id, the request's
+    *life* in the cache, table lengths).  Only for the same life may the row be
+    extended instead of rewritten: a request that was released and added again
+    (preempted and computed again, or an id used twice) comes back under the
+    same id with other pages.  The reference looks every location up in the
+    page table itself and keeps no copy (src/core/runtime/KVCache.h:221-240);
+    this copy must behave as if it did."""
+
+    def __init__(self, cache, bucket: int, max_model_len: int, hv: np.ndarray | None = None):
+        self.cache = cache
         self.B = B = int(bucket)
-        cache = runner.cache
         ps = cache.page_size
-        self.widths = [-(-runner.max_model_len // ps) for _ in cache.groups]
-        # sections of the packed table buffer, as in build_step_batch
-        sizes = [B, B, B, B + 1, B, B, B, B, B]
-        for w in self.widths:
-            sizes += [B * w, B]
-        self.offs, total = [], 0
-        for n in sizes:
-            self.offs.append(total)
-            total += _pad4(n)
-        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
-        self.hv = self.host.numpy()
-        self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
+        self.widths = [-(-max_model_len // ps) for _ in cache.groups]
+        self.offs, self.total = table_layout(B, self.widths)
+        if hv is None:
+            hv = np.zeros(self.total, dtype=np.int32)
+        if hv.dtype != np.int32 or hv.shape != (self.total,):
+            raise ValueError(f"the table buffer must be int32 [{self.total}]")
+        self.hv = hv
         o = self.offs
-
-        def sl(i, n):
-            return self.dev[o[i]:o[i] + n]
-
-        b = StepBatch()
-        b.num_tokens = b.num_reqs = b.num_logit_rows = B
-        b.max_new_tokens = 1
-        b.max_context = runner.max_model_len
-        b.token_ids, b.positions, b.token_req = sl(0, B), sl(1, B), sl(2, B)
-        b.cu_tokens, b.start_pos, b.context_lens = sl(3, B + 1), sl(4, B), sl(5, B)
-        b.state_slots, b.logit_rows = sl(6, B), sl(7, B)
-        no_slot = sl(8, B)
-        for gi, w in enumerate(self.widths):
-            bt = self.dev[o[9 + 2 * gi]:o[9 + 2 * gi] + B * w].view(B, w)
-            b.groups.append(GroupTables(bt, sl(10 + 2 * gi, B), no_slot))
-        b.host_cu_tokens = list(range(B + 1))
-        b.host_start_pos = [0] * B
-        b.host_state_slots = [0] * B
-        b.reqs = [None] * B
-        self.batch = b
-        # fixed parts of the tables
-        hv = self.hv
+        hv[:] = 0
         hv[o[2]:o[2] + B] = np.arange(B)            # token_req
         hv[o[3]:o[3] + B + 1] = np.arange(B + 1)    # cu_tokens
         hv[o[7]:o[7] + B] = np.arange(B)            # logit rows: every row
         hv[o[8]:o[8] + B] = -1                      # no-slot mapping
-        self._row_state = [None] * B                # (request, table lengths) last written per row
+        self._row_state = [None] * B                # (request, life, table lengths) last written per row
         self._pad_rows(0)
-        self.graph = None
-        self.logits = None
-        self._copied = torch.cuda.Event()
 
-    @property
-    def runner(self):
-        return self._runner()
+    def block_table_row(self, group: int, row: int) -> np.ndarray:
+        w = self.widths[group]
+        base = self.offs[9 + 2 * group] + row * w
+        return self.hv[base:base + w]
 
     def _pad_rows(self, first: int) -> None:
         o, hv, B = self.offs, self.hv, self.B
@@ -102,12 +99,14 @@ class DecodeGraph:
 
     def fill(self, entries) -> None:
         """Writes the step's tables for ``entries`` (one token each, pages reserved)."""
-        cache, o, hv = self.runner.cache, self.offs, self.hv
+        cache, o, hv = self.cache, self.offs, self.hv
         ps = cache.page_size
         R = len(entries)
-        self._copied.synchronize()      # the last copy out of the host buffer is done
+        if R > self.B:
+            raise ValueError(f"{R} entries do not fit a graph of {self.B} rows")
         for r, e in enumerate(entries):
             P = cache.num_tokens(e.req)
+            life = cache.life(e.req)
             hv[o[0] + r] = e.tokens[0]
             hv[o[1] + r] = P
             hv[o[4] + r] = P
@@ -119,19 +118,66 @@ class DecodeGraph:
                 table = cache.block_table(gi, e.req)
                 base = o[9 + 2 * gi] + r * w
                 n = len(table)
-                same = prev is not None and prev[0] == e.req and cache.groups[gi].spec.window == 0
-                if same:
-                    # a table that keeps all keys only grows: write what is new
-                    if n > prev[1][gi]:
-                        hv[base + prev[1][gi]:base + n] = table[prev[1][gi]:]
+                old = prev[2][gi] if prev is not None else 0
+                grown = prev is not None and prev[0] == e.req and prev[1] == life \
+                    and cache.groups[gi].spec.window == 0 and n >= old
+                if grown:
+                    # same stay in the cache and a table that keeps all keys: it only grew
+                    if n > old:
+                        hv[base + old:base + n] = table[old:]
                 else:
                     hv[base:base + n] = [p if p >= 0 else 0 for p in table]
-                    if prev is not None and prev[1][gi] > n:
-                        hv[base + n:base + prev[1][gi]] = 0
+                    if old > n:
+                        hv[base + n:base + old] = 0
                 lens.append(n)
                 hv[o[10 + 2 * gi] + r] = table[P // ps] * ps + P % ps
-            self._row_state[r] = (e.req, lens)
+            self._row_state[r] = (e.req, life, lens)
         self._pad_rows(R)
+
+
+class DecodeGraph:
+    def __init__(self, runner, bucket: int):
+        self._runner = weakref.ref(runner)   # the runner owns its graphs; no reference cycle
+        self.B = B = int(bucket)
+        cache = runner.cache
+        widths = [-(-runner.max_model_len // cache.page_size) for _ in cache.groups]
+        _, total = table_layout(B, widths)
+        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.tables = DecodeTables(cache, B, runner.max_model_len, self.host.numpy())
+        self.widths = self.tables.widths
+        self.offs = o = self.tables.offs
+        self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
+
+        def sl(i, n):
+            return self.dev[o[i]:o[i] + n]
+
+        b = StepBatch()
+        b.num_tokens = b.num_reqs = b.num_logit_rows = B
+        b.max_new_tokens = 1
+        b.max_context = runner.max_model_len
+        b.token_ids, b.positions, b.token_req = sl(0, B), sl(1, B), sl(2, B)
+        b.cu_tokens, b.start_pos, b.context_lens = sl(3, B + 1), sl(4, B), sl(5, B)
+        b.state_slots, b.logit_rows = sl(6, B), sl(7, B)
+        no_slot = sl(8, B)
+        for gi, w in enumerate(self.widths):
+            bt = self.dev[o[9 + 2 * gi]:o[9 + 2 * gi] + B * w].view(B, w)
+            b.groups.append(GroupTables(bt, sl(10 + 2 * gi, B), no_slot))
+        b.host_cu_tokens = list(range(B + 1))
+        b.host_start_pos = [0] * B
+        b.host_state_slots = [0] * B
+        b.reqs = [None] * B
+        self.batch = b
+        self.graph = None
+        self.logits = None
+        self._copied = torch.cuda.Event()
+
+    @property
+    def runner(self):
+        return self._runner()
+
+    def fill(self, entries) -> None:
+        self._copied.synchronize()      # the last copy out of the host buffer is done
+        self.tables.fill(entries)
 
     def _forward(self):
         from .runner import StepContext

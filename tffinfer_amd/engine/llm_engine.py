@@ -51,6 +51,7 @@ class _Launched:
     tokens: torch.Tensor | None     # int32 [rows] on the device
     host: torch.Tensor | None       # the same in pinned host memory, valid after ``ready``
     ready: torch.cuda.Event | None
+    logits: torch.Tensor | None = None   # float32 [rows, vocab] in pinned host memory, if kept
 
 
 @dataclass
@@ -91,6 +92,7 @@ class LLMEngine:
         self._ids = itertools.count()
         self.keep_logits = False
         self._results: dict = {}
+        self._requests: dict = {}
         self._ahead: _Launched | None = None   # a decode step launched ahead of its predecessor's tokens
         self.steps_ahead = 0                   # how many steps were launched that way
 
@@ -127,8 +129,22 @@ class LLMEngine:
         if eos_token_id is None and not ignore_eos:
             eos_token_id = getattr(self.model.config, "eos_token_id", None)
         req = Request(rid, prompt, sampling or SamplingConfig(), int(max_new_tokens), eos_token_id, ignore_eos)
+        if rid in self._requests and self._requests[rid].status != "finished":
+            raise ValueError(f"request id {rid!r} is in use")
         self.scheduler.add_request(req)
+        self._requests[rid] = req
+        self._results.pop(rid, None)
         return rid
+
+    def pop_result(self, request_id) -> GenerationResult:
+        """The result of a request that has finished (by length, stop token or abort); the
+        engine forgets the request."""
+        r = self._requests[request_id]
+        if r.status != "finished":
+            raise ValueError(f"request {request_id!r} has not finished")
+        del self._requests[request_id]
+        return GenerationResult(r.id, r.prompt, r.output, r.finish_reason, r.num_preemptions,
+                                self._results.pop(r.id, []))
 
     def abort(self, request_id) -> bool:
         return self.scheduler.abort(request_id)
@@ -159,10 +175,12 @@ class LLMEngine:
         logits = self.runner.step(entries, token_source)
         if not rows:
             return _Launched(plan, rows, None, None, None)
+        kept = None
         if self.keep_logits:
-            host = logits.float().cpu()
-            for r, req in enumerate(rows):
-                self._results.setdefault(req.id, []).append(host[r].clone())
+            # copied on the stream, before a penalty changes the rows and before the next
+            # replay of a decode graph writes its logits tensor again
+            kept = torch.empty(logits.shape, dtype=torch.float32, pin_memory=True)
+            kept.copy_(logits, non_blocking=True)
         ahead = 0 if token_source is None else 1      # outputs the host has not appended yet
         tokens = self.sampler.sample_on_device(
             logits, [r.sampling for r in rows], [len(r.output) + ahead for r in rows],
@@ -171,7 +189,7 @@ class LLMEngine:
         host.copy_(tokens, non_blocking=True)
         ready = torch.cuda.Event()
         ready.record()
-        return _Launched(plan, rows, tokens, host, ready)
+        return _Launched(plan, rows, tokens, host, ready, kept)
 
     def _complete(self, st: _Launched) -> list[tuple]:
         """Reads the step's tokens and tells the scheduler.  Requests that ended
@@ -180,9 +198,11 @@ class LLMEngine:
         sampled = {}
         if st.rows:
             st.ready.synchronize()
-            for req, t in zip(st.rows, st.host.tolist()):
+            for r, (req, t) in enumerate(zip(st.rows, st.host.tolist())):
                 if req.status == "running":
                     sampled[req.id] = t
+                    if st.logits is not None:
+                        self._results.setdefault(req.id, []).append(st.logits[r].clone())
         finished = self.scheduler.update(plan, sampled)
         done = {r.id for r in finished}
         return [(rid, tok, rid in done) for rid, tok in sampled.items()]
@@ -192,7 +212,7 @@ class LLMEngine:
         of ``st`` that its length does not end goes on.  None when the step after
         needs the scheduler (admissions, prompts, pages running out, a penalty on
         seen tokens)."""
-        if not self.options.run_ahead or self.keep_logits or not st.rows:
+        if not self.options.run_ahead or not st.rows:
             return None
         sch = self.scheduler
         if any(p.count != 1 or not p.samples for p in st.plan) or len(st.plan) != len(sch.running):
@@ -246,12 +266,8 @@ class LLMEngine:
         for all or a list with one per prompt."""
         if sampling is None or isinstance(sampling, SamplingConfig):
             sampling = [sampling or SamplingConfig()] * len(prompts)
-        reqs = []
-        for prompt, sc in zip(prompts, sampling):
-            rid = self.add_request(prompt, sc, max_new_tokens, eos_token_id, ignore_eos)
-            reqs.append(self.scheduler.waiting[-1])
-            assert reqs[-1].id == rid
+        ids = [self.add_request(prompt, sc, max_new_tokens, eos_token_id, ignore_eos)
+               for prompt, sc in zip(prompts, sampling)]
         while self.has_work:
             self.step()
-        return [GenerationResult(r.id, r.prompt, r.output, r.finish_reason, r.num_preemptions,
-                                 self._results.pop(r.id, [])) for r in reqs]
+        return [self.pop_result(rid) for rid in ids]
