@@ -7,7 +7,7 @@ import sys
 import pytest
 import torch
 
-from helpers import TOL, oracle_logits, random_tokens, read_config, rel_err
+from helpers import tol, oracle_logits, random_tokens, read_config, rel_err
 from plain_qwen3 import plain_greedy, plain_inverse_cdf, plain_probs
 
 pytestmark = pytest.mark.gpu
@@ -31,7 +31,7 @@ def check_choices(model_dir, result, dtype, sampling=None):
     assert len(result.logits) == len(result.output)
     for i, (row, tok) in enumerate(zip(result.logits, result.output)):
         pos = len(result.prompt) + i - 1
-        assert rel_err(row, ref[pos]) <= TOL[dtype], f"output {i}"
+        assert rel_err(row, ref[pos]) <= tol(dtype, model_dir), f"output {i}"
         if sampling is None or sampling.greedy:
             assert tok == plain_greedy(row)
         else:

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import replay_lib as rl
-from helpers import PAGE_SIZE, TOL, random_tokens, read_config, rel_err
+from helpers import PAGE_SIZE, tol, random_tokens, read_config, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -38,7 +38,7 @@ def test_replay_modes(model_dirs, name, dtype, mode):
     num_pages = rl.max_live_tokens(steps, unit=ps) // ps
     runner = make_runner(model_dir, dtype, ps, num_pages)
     results = rl.run_steps_in_process(runner, steps)
-    worst = rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
+    worst = rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name))
     print(f"{name} {dtype} {mode}: worst rel. error {worst:.3e} over {len(steps)} steps, {num_pages} pages")
     assert all(g.pool.num_used == 0 for g in runner.cache.groups)
 
@@ -55,7 +55,7 @@ def test_replay_with_pages_that_are_no_power_of_two(model_dirs, name, ps, dtype)
     steps = rl.trace_mixed(reqs)
     runner = make_runner(model_dir, dtype, ps, rl.max_live_tokens(steps, unit=ps) // ps)
     results = rl.run_steps_in_process(runner, steps)
-    rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
+    rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -68,7 +68,7 @@ def test_trace_run_program(model_dirs, tmp_path, dtype):
     assert any(not any(e["want"] for e in s["entries"]) for s in steps)
     out = rl.run_steps_subprocess(model_dir, dtype, steps, str(tmp_path / "out"),
                                   rl.max_live_tokens(steps, 64))
-    rl.check_against_oracle(model_dir, reqs, steps, out, TOL[dtype])
+    rl.check_against_oracle(model_dir, reqs, steps, out, tol(dtype, "B"))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -92,7 +92,7 @@ def test_replay_with_decode_graphs(model_dirs, name, dtype, mode):
     assert runner._graphs, "no decode step went through a graph"
     decode_only = sum(1 for s in steps if s["entries"] and all(len(e["tokens"]) == 1 for e in s["entries"]))
     assert decode_only >= 3
-    rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
+    rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -150,7 +150,7 @@ def test_long_decoding(model_dirs, name, dtype, n, graphs):
     runner = ModelRunner(load_model(model_dir, DTYPES[dtype], "cuda:0"), page_size=ps,
                          num_pages=-(-n // ps), max_seqs=2, use_graphs=graphs)
     results = rl.run_steps_in_process(runner, steps)
-    rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
+    rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name))
     if name in ("B", "D"):   # the window groups gave pages back on the way
         assert any(g.spec.window > 0 for g in runner.cache.groups)
 
@@ -165,7 +165,7 @@ def test_first_tokens(model_dirs, name, dtype):
     for steps in (rl.trace_whole(reqs), rl.trace_tail(reqs, tail=3)):
         runner = make_runner(model_dir, dtype, PAGE_SIZE[name], 4)
         results = rl.run_steps_in_process(runner, steps)
-        rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
+        rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name))
 
 
 MID = dict(
@@ -198,7 +198,7 @@ def test_midsize_model_long_prompt(tmp_path_factory, dtype):
     for steps in (whole, parts):
         runner = make_runner(model_dir, dtype, 16, 72, max_seqs=2)
         results = rl.run_steps_in_process(runner, steps)
-        worst = rl.check_against_oracle(model_dir, reqs, steps, results, TOL[dtype])
+        worst = rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, "mid"))
         print(f"mid {dtype}: worst rel. error {worst:.3e}")
 
 
@@ -242,4 +242,4 @@ def test_bfloat16_against_float32_at_large_layer_sizes(shape):
     assert out[torch.float32].shape[0] == 3 + 2 + 14 + 2
     worst = rel_err(out[torch.bfloat16], out[torch.float32])
     print(f"{shape}: bfloat16 against float32, worst rel. error {worst:.3e}")
-    assert worst <= TOL["bfloat16"]
+    assert worst <= tol("bfloat16", "large")

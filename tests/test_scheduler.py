@@ -225,3 +225,21 @@ def test_sampling_config_validation():
     assert SamplingConfig().greedy and SamplingConfig("default").greedy
     assert SamplingConfig("random", temperature=0.0).greedy
     assert SamplingConfig("top_k", 0.7, top_k=5).effective() == (0.7, 5, 1.0, 0.0)
+
+
+def test_a_head_of_the_queue_that_fits_nowhere_is_finished_not_raised():
+    """Pages held by somebody the scheduler does not know (so that its own check at
+    add_request passes): the head cannot get a single token even with nothing running.  It is
+    taken out and finished as "refused"; the requests behind it run once pages are there."""
+    cache, sched, runner = make(num_pages=4, ps=8)
+    cache.add_request("elsewhere")
+    cache.reserve("elsewhere", 32)                    # every page
+    a, b = Request("a", [1] * 5, max_new_tokens=3), Request("b", [2] * 5, max_new_tokens=3)
+    sched.add_request(a)
+    assert sched.schedule() == []
+    assert a.status == "finished" and a.finish_reason == "refused" and sched.refused == [a]
+    assert not sched.has_work
+    cache.release("elsewhere")
+    sched.add_request(b)
+    run_all(sched, runner, cache)
+    assert b.output == expected_output(b.prompt, 3)

@@ -240,13 +240,19 @@ class LLMEngine:
 
     def step(self) -> list[tuple]:
         """Plans and runs one step.  Returns (request id, new token, finished)
-        for every request that got a token."""
+        for every request that got a token, and (request id, None, True) for a
+        request that was dropped because the cache cannot hold it even alone
+        (finish reason "refused")."""
         st = self._ahead
         self._ahead = None
+        dropped = []
         if st is None:
             plan = self.scheduler.schedule()
+            # requests that turned out not to fit the cache even alone: finished without a token
+            dropped = [(r.id, None, True) for r in self.scheduler.refused]
+            self.scheduler.refused.clear()
             if not plan:
-                return []
+                return dropped
             st = self._launch(plan)
         nxt = self._plan_ahead(st)
         if nxt is not None:
@@ -256,7 +262,7 @@ class LLMEngine:
                 src = st.tokens[torch.tensor(keep, device=st.tokens.device)]
             self._ahead = self._launch(nxt, src)
             self.steps_ahead += 1
-        return self._complete(st)
+        return dropped + self._complete(st)
 
     # ---- whole generations ----------------------------------------------
     def generate(self, prompts, sampling=None, max_new_tokens: int = 64, eos_token_id: int | None = None,

@@ -25,7 +25,11 @@ Rules of a step, in this order:
    recently admitted one is preempted and the step is planned again.
 
 A request that could never fit the pool or the model's length is refused when
-it is added, with an error, not truncated.
+it is added, with an error, not truncated.  The check at that time is a bound
+for caches with a window; a request that passes it and still does not fit the
+cache when it is alone is taken out of the queue and finished with the reason
+"refused" (``Scheduler.refused`` holds such requests until the engine reports
+them), so that the requests behind it run.
 """
 from __future__ import annotations
 
@@ -97,6 +101,7 @@ class Scheduler:
         self.max_model_len = int(max_model_len)
         self.waiting: deque[Request] = deque()
         self.running: list[Request] = []   # in order of admission
+        self.refused: list[Request] = []   # finished as "refused" by schedule(), not yet reported
         self.stats = SchedulerStats()
 
     # ---- requests --------------------------------------------------------
@@ -170,13 +175,15 @@ class Scheduler:
         """Plans one step and reserves its pages.  Empty when nothing is left to do."""
         while True:
             plan = self._plan()
-            if plan or not self.running:
-                if not plan and self.waiting and not self.running:
-                    # nothing runs and the head of the queue still does not fit: it never will
-                    head = self.waiting[0]
-                    raise RequestRefused(f"request {head.id!r} does not fit the cache even alone")
+            if plan or not (self.running or self.waiting):
                 return plan
-            self._preempt_last()
+            if self.running:
+                self._preempt_last()
+            else:
+                # nothing runs and the head of the queue still does not fit: it never will
+                head = self.waiting.popleft()
+                self._finish(head, "refused", live=False)
+                self.refused.append(head)
 
     def _plan(self) -> list[ScheduledPortion]:
         budget = self.opt.max_num_batched_tokens

@@ -18,6 +18,12 @@ class NoPosition(PositionEncoding):
         return None
 
 
+# Rotation tables by (class, rotary size, theta, positions, device).  Layers with the same law share one
+# tensor, and a table is never dropped: a captured decode graph holds its address for as long as
+# the graph lives, whatever other runner asks for another length meanwhile.
+_TABLES: dict = {}
+
+
 @register_position_encoding("rope")
 class RotaryEmbedding(PositionEncoding):
     """angle(pos, i) = pos * theta^(-2i/rot), i < rot/2, as (cos, sin) pairs.
@@ -40,7 +46,6 @@ class RotaryEmbedding(PositionEncoding):
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
             raise ConfigError(f"rope: rotary size {self.rotary_dim} must be even and at most {self.head_dim}")
         self.pairing = pairing
-        self._tables = {}
 
     def angles(self, max_positions: int) -> torch.Tensor:
         half = self.rotary_dim // 2
@@ -49,10 +54,10 @@ class RotaryEmbedding(PositionEncoding):
         return torch.arange(max_positions, dtype=torch.float64)[:, None] * inv[None, :]
 
     def table(self, max_positions, device):
-        key = (int(max_positions), str(device))
-        t = self._tables.get(key)
+        key = (type(self), self.rotary_dim, self.theta, int(max_positions), str(torch.device(device)))
+        t = _TABLES.get(key)
         if t is None:
             a = self.angles(max_positions)
             t = torch.stack([torch.cos(a), torch.sin(a)], -1).to(torch.float32).contiguous().to(device)
-            self._tables = {key: t}
+            _TABLES[key] = t
         return t
