@@ -21,6 +21,8 @@
 //       the first and of the second tile: exactly what the lane already holds
 //       of P, and two 8-byte runs of a value page, which is kept transposed
 //       ([element][slot]) for this purpose.  No operand goes through LDS.
+#include <mutex>
+
 #include "common.h"
 #include "tffinfer_kernels.h"
 
@@ -1075,4 +1077,75 @@ TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml
         attn_split_reduce_kernel<<<dim3(n, nq), 256, 0, (hipStream_t)stream>>>(
             part_o, part_ml, (bf16_t*)out, splits, R_total, nq, d, rows);
     return tff_check_launch("attention_split_reduce");
+}
+
+// ------------------------------------------ decoding without any allocation ---
+// The partial results of split keys need device memory besides the inputs and outputs.  The
+// entry points above take it from the caller; this one keeps it in the library: one array per
+// GPU, part of the code object, there from the moment the library is loaded on a device until
+// the process ends.  Nothing in it has to start at zero (every wave of a split launch writes its
+// rows, the empty ones too: maximum -inf, sum 0), so a call leaves nothing that the next one
+// has to clear.
+#define TFF_ATTN_STATIC_FLOATS (TFF_ATTENTION_STATIC_SCRATCH_BYTES / sizeof(float))   // 16 MiB a GPU
+static __device__ __align__(256) float attn_static_scratch[TFF_ATTN_STATIC_FLOATS];
+
+#define TFF_MAX_DEVICES 64
+static float* attn_static_ptr[TFF_MAX_DEVICES];   // the array's address on each device, once asked for
+static std::mutex attn_static_mutex;
+
+// The device address of the current device's copy of the array.  The array's name is a host-side
+// handle, not an address a kernel could use; every GPU has its own copy at its own address.
+static int attn_static_address(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return tff_fail("attention_decode_fused_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= TFF_MAX_DEVICES)
+        return tff_fail("attention_decode_fused_static: device %d is beyond the %d this library keeps scratch for",
+                        dev, TFF_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(attn_static_mutex);
+    if (!attn_static_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(attn_static_scratch));
+        if (e != hipSuccess || !p)
+            return tff_fail("attention_decode_fused_static: hipGetSymbolAddress on device %d: %s", dev,
+                            hipGetErrorString(e));
+        attn_static_ptr[dev] = (float*)p;
+    }
+    *out = attn_static_ptr[dev];
+    return 0;
+}
+
+TFF_API int tff_attention_decode_fused_static(const void* qkv, int qkv_stride, void* out, void* k_cache,
+                                              void* v_cache, const int32_t* block_tables, int bt_stride,
+                                              const int32_t* cu_tokens, const int32_t* start_pos,
+                                              const int32_t* slot_mapping, const float* q_weight,
+                                              const float* k_weight, float eps, const float* cos_sin,
+                                              int max_pos, int pairing, int splits, int R, int nq, int nkv,
+                                              int d, int page_size, int num_pages, int window, float scale,
+                                              tff_stream_t stream) {
+    TFF_REQUIRE(splits >= 1 && splits <= 256 && R >= 0 && nq > 0 && d > 0,
+                "attention_decode_fused_static: bad sizes (splits %d, entries %d, heads %d, head size %d)",
+                splits, R, nq, d);
+    float *part_o = nullptr, *part_ml = nullptr;
+    if (splits > 1 && R > 0) {
+        const size_t rows = (size_t)splits * R * nq;
+        const size_t need = rows * ((size_t)d + 2);
+        TFF_REQUIRE(need <= TFF_ATTN_STATIC_FLOATS,
+                    "attention_decode_fused_static: %d splits x %d entries x %d heads of %d need %zu bytes of "
+                    "partial results, the library keeps %zu a GPU (use fewer splits, or tff_attention_decode_fused "
+                    "with a workspace of your own)",
+                    splits, R, nq, d, need * sizeof(float), (size_t)TFF_ATTN_STATIC_FLOATS * sizeof(float));
+        float* base = nullptr;
+        if (int rc = attn_static_address(&base)) return rc;
+        part_o = base;
+        part_ml = base + rows * d;      // rows * d is a multiple of 16 floats: d is
+    }
+    if (int rc = tff_attention_decode_fused(qkv, qkv_stride, out, part_o, part_ml, k_cache, v_cache, block_tables,
+                                            bt_stride, cu_tokens, start_pos, slot_mapping, q_weight, k_weight, eps,
+                                            cos_sin, max_pos, pairing, splits, R, nq, nkv, d, page_size, num_pages,
+                                            window, scale, stream))
+        return rc;
+    if (splits > 1 && R > 0)
+        return tff_attention_split_reduce(part_o, part_ml, out, splits, R, nq, d, nullptr, 0, stream);
+    return 0;
 }

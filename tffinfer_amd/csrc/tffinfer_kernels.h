@@ -155,6 +155,28 @@ TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml
                                        int splits, int R_total, int nq, int d, const int32_t* rows,
                                        int num_rows, tff_stream_t stream);
 
+// tff_attention_decode_fused followed by tff_attention_split_reduce, for callers that cannot
+// allocate device memory: code under HIP graph capture, tight serving loops, harnesses that
+// forbid hipMalloc.  It has no counterpart in the reference.  The partial results of split keys
+// live in an array that is part of the library, TFF_ATTENTION_STATIC_SCRATCH_BYTES (16 MiB)
+// on every GPU the library runs on, held until the process ends; the call allocates and frees
+// nothing, on the device or through any library.  It refuses, with a message, sizes whose
+// partial results (splits * R * nq * (d + 2) floats) do not fit.  All calls on one GPU share
+// that GPU's array: calls that overlap there (two streams, two threads) race; calls on one
+// stream, or otherwise ordered, do not.  The array keeps the last call's contents and nothing
+// in it has to be cleared between calls.  The array's address on a device is looked up at the
+// first call on that device (make it outside a graph capture).  Arguments as for
+// tff_attention_decode_fused, without the workspace; out [R, nq * d] is final.
+#define TFF_ATTENTION_STATIC_SCRATCH_BYTES (16u << 20)
+TFF_API int tff_attention_decode_fused_static(const void* qkv, int qkv_stride, void* out, void* k_cache,
+                                              void* v_cache, const int32_t* block_tables, int bt_stride,
+                                              const int32_t* cu_tokens, const int32_t* start_pos,
+                                              const int32_t* slot_mapping, const float* q_weight,
+                                              const float* k_weight, float eps, const float* cos_sin,
+                                              int max_pos, int pairing, int splits, int R, int nq, int nkv,
+                                              int d, int page_size, int num_pages, int window, float scale,
+                                              tff_stream_t stream);
+
 // out[t, i] = silu(gu[t, i]) * gu[t, I + i]
 TFF_API int tff_swiglu(const void* gu, void* out, int T, int I, int dtype, tff_stream_t stream);
 

@@ -40,6 +40,8 @@ _SIGNATURES = {
                            _I, _I, _I, _I, _I, _I, _F, _P],
     "tff_attention_decode_fused": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _F, _P, _I, _I,
                                    _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
+    "tff_attention_decode_fused_static": [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _F, _P, _I, _I,
+                                          _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "tff_attention_split_reduce": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _P],
     "tff_swiglu": [_P, _P, _I, _I, _I, _P],
     "tff_cast": [_P, _I, _P, _I, c_int64, _P],
