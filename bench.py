@@ -11,12 +11,7 @@ of the HBM peak, and decode throughput at batch 1 and 64.
 """
 import argparse
 import json
-import statistics
 import sys
-import time
-
-HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
-MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense, published
 
 # layer sizes of the benchmark configuration (Qwen3-8B shape) and of the two larger shapes
 QWEN3_8B = dict(
@@ -58,108 +53,69 @@ def parse_args():
                     help="tokens of a step of the --mixed workload (default: a portion beside every decoding request, at least 1,024)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--ceilings", action="store_true",
-                    help="measure streaming-read bandwidth and back-to-back MFMA rate on this machine and stop")
+                    help="measure streaming-read bandwidth, back-to-back MFMA rates and a large square product "
+                         "on this machine and stop")
+    ap.add_argument("--no-large-points", action="store_true",
+                    help="skip the two points at the larger shapes (32 mixed requests at the 14B shape; batch 16 "
+                         "at 8,192 tokens of context at the 32B shape), which the default run adds to 'points'")
     return ap.parse_args()
 
 
-def random_prompt(gen, n, vocab):
+def build_model(cfg, seed):
     import torch
-    return torch.randint(0, vocab, (n,), generator=gen).tolist()
-
-
-def matmul_params_per_layer(c):
-    H, nq, nkv, d, I = (c["hidden_size"], c["num_attention_heads"], c["num_key_value_heads"],
-                        c["head_dim"], c["intermediate_size"])
-    return (nq + 2 * nkv) * d * H + nq * d * H + 3 * I * H
-
-
-def prefill_flops(c, L, T):
-    gemm = 2.0 * T * matmul_params_per_layer(c) * L
-    attn = 4.0 * c["num_attention_heads"] * c["head_dim"] * (T * (T + 1) / 2) * L
-    head = 2.0 * c["hidden_size"] * c["vocab_size"]
-    return gemm + attn + head
-
-
-def decode_bytes(c, L, batch, context, esz=2):
-    weights = (matmul_params_per_layer(c) * L + c["hidden_size"] * c["vocab_size"]) * esz
-    kv = 2 * L * c["num_key_value_heads"] * c["head_dim"] * esz * batch * context
-    return weights + kv
-
-
-def sync():
-    import torch
+    from tffinfer_amd.models import build_model_skeleton, config_from_dict
+    model = build_model_skeleton(config_from_dict(cfg))
+    model.init_random(seed, torch.bfloat16, "cuda:0", on_device=True)
     torch.cuda.synchronize()
+    return model
 
 
-def measure_prefill(engine, gen, T, vocab, reps=5, warm=2):
-    from tffinfer_amd.engine.batch import StepEntry
-    times = []
-    for i in range(reps + warm):
-        rid = f"prefill{i}"
-        toks = random_prompt(gen, T, vocab)
-        engine.runner.add_request(rid)
-        sync()
-        t0 = time.perf_counter()
-        logits = engine.runner.step([StepEntry(rid, toks, [T - 1])])
-        sync()
-        dt = time.perf_counter() - t0
-        assert logits.shape[0] == 1
-        engine.runner.free_request(rid)
-        if i >= warm:   # the first runs warm up (allocator, work tables, clocks)
-            times.append(dt)
-    return statistics.median(times)
-
-
-def decode_slack(batch, context, chunk=2048):
-    """Steps the first request may decode while the last one still reads its prompt."""
-    return batch * (-(-context // chunk) + 1)
-
-
-def measure_decode(engine, gen, batch, context, steps, warmup, vocab):
-    """Fills ``batch`` requests with ``context`` tokens each (untimed prefill),
-    then times ``steps`` decode steps of the engine."""
-    for _ in range(batch):
-        # requests that finish their prompt early decode while the others still prefill
-        engine.add_request(random_prompt(gen, context, vocab),
-                           max_new_tokens=warmup + steps + decode_slack(batch, context) + 8, ignore_eos=True)
-    # untimed: prompts, up to the first decode-only step
-    while any(r.num_pending > 1 for r in engine.scheduler.running) or engine.scheduler.waiting:
-        engine.step()
-    for _ in range(warmup):
-        out = engine.step()
-        assert len(out) == batch
-    sync()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        out = engine.step()
-    sync()
-    dt = time.perf_counter() - t0
-    assert len(out) == batch
-    for r in list(engine.scheduler.running):
-        engine.abort(r.id)
-    return dt
-
-
-def measure_mixed(engine, gen, requests, vocab, new_tokens=256, lo=128, hi=4096):
-    """Continuous batching: all requests arrive at once, the scheduler admits them as
-    slots and pages allow, cuts prompts into portions and decodes the others beside them."""
+def large_points(args, gen) -> dict:
+    """Two workloads at the larger shapes, each with a model of its own: 32 requests with prompts
+    of 128 to 4,096 tokens in portions of 512 beside decoding requests at the 14B shape (all
+    tokens, prompt and generated, a second), and decode steps of 16 requests at 8,192 tokens of
+    context at the 32B shape (decoded tokens a second).  A point that fails is left null."""
+    import gc
     import torch
-    lens = torch.randint(lo, hi + 1, (requests,), generator=gen).tolist()
-    for n in lens:
-        engine.add_request(random_prompt(gen, n, vocab), max_new_tokens=new_tokens, ignore_eos=True)
-    sync()
-    t0 = time.perf_counter()
-    steps = 0
-    while engine.has_work:
-        engine.step()
-        steps += 1
-    sync()
-    dt = time.perf_counter() - t0
-    st = engine.scheduler.stats
-    return {"requests": requests, "prompt_tokens": sum(lens), "generated_tokens": requests * new_tokens,
-            "seconds": round(dt, 3), "engine_steps": steps, "preemptions": st.preemptions,
-            "total_tokens_per_s": round((sum(lens) + requests * new_tokens) / dt, 1),
-            "generated_tokens_per_s": round(requests * new_tokens / dt, 1)}
+    from tffinfer_amd import EngineOptions, LLMEngine
+    from tffinfer_amd import measure as M
+    out = {}
+
+    def release():
+        gc.collect()
+        torch.cuda.empty_cache()
+
+    try:
+        cfg = dict(SHAPES["14b"][1])
+        model = build_model(cfg, args.seed)
+        opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=32 * (4096 + 256 + args.page_size),
+                            max_num_seqs=32, max_num_batched_tokens=1024, prefill_chunk=512,
+                            max_model_len=cfg["max_position_embeddings"], use_graphs=not args.no_graphs)
+        engine = LLMEngine(model, opt)
+        out["mixed32_14b_tokens_per_s"] = M.measure_mixed(engine, gen, 32, cfg["vocab_size"])["total_tokens_per_s"]
+        del engine, model
+    except Exception as e:      # the headline figures must not be lost to a side measurement
+        print(f"bench: the 14B point failed: {e}", file=sys.stderr)
+        out["mixed32_14b_tokens_per_s"] = None
+    release()
+    try:
+        cfg = dict(SHAPES["32b"][1])
+        batch, context, steps, warmup = 16, 8192, 20, 4
+        model = build_model(cfg, args.seed)
+        total = steps + warmup + M.decode_slack(batch, context) + 16
+        opt = EngineOptions(dtype="bfloat16", page_size=args.page_size,
+                            kv_tokens=batch * (context + total + args.page_size), max_num_seqs=batch,
+                            max_num_batched_tokens=4096, prefill_chunk=2048,
+                            max_model_len=cfg["max_position_embeddings"], use_graphs=not args.no_graphs)
+        engine = LLMEngine(model, opt)
+        r = M.measure_decode(engine, gen, batch, context, steps, warmup, cfg["vocab_size"])
+        out["decode_b16_ctx8192_32b"] = round(batch * steps / r["wall_s"], 1)
+        del engine, model
+    except Exception as e:
+        print(f"bench: the 32B point failed: {e}", file=sys.stderr)
+        out["decode_b16_ctx8192_32b"] = None
+    release()
+    return out
 
 
 def main():
@@ -169,14 +125,16 @@ def main():
         sys.exit(2)
     import torch
     from tffinfer_amd import EngineOptions, LLMEngine
+    from tffinfer_amd import measure as M
     from tffinfer_amd.kernels import lib as kernel_lib
-    from tffinfer_amd.models import build_model_skeleton, config_from_dict
 
     kernel_lib.load()
     if args.ceilings:
         from tffinfer_amd.kernels import ops
-        print(json.dumps({"ceilings": ops.measure_ceilings("cuda:0"),
-                          "published": {"hbm_GBps": HBM_PEAK_GBS, "bf16_TFLOPs": MFMA_PEAK["bf16"] / 1e12}}))
+        c = ops.measure_ceilings("cuda:0")
+        c.update(M.square_product_rates("cuda:0"))
+        print(json.dumps({"ceilings": c,
+                          "published": {"hbm_GBps": M.HBM_PEAK_GBS, "bf16_TFLOPs": M.MFMA_PEAK["bf16"] / 1e12}}))
         return
     shape_name, shape = SHAPES[args.shape]
     cfg = dict(shape)
@@ -184,14 +142,13 @@ def main():
     L = args.layers or L_full
     cfg["num_hidden_layers"] = L
     # a context beyond the shape's own limit: the limit grows with it (it sizes the rotation table only)
-    longest = max(args.prefill_tokens, args.context + args.steps + args.warmup + decode_slack(max(args.batch, 64), args.context) + 16)
+    longest = max(args.prefill_tokens,
+                  args.context + args.steps + args.warmup + M.decode_slack(max(args.batch, 64), args.context) + 16)
     if not args.mixed and longest > cfg["max_position_embeddings"]:
         cfg["max_position_embeddings"] = 1 << (longest - 1).bit_length()
     vocab = cfg["vocab_size"]
     gen = torch.Generator().manual_seed(args.seed)
-    model = build_model_skeleton(config_from_dict(cfg))
-    model.init_random(args.seed, torch.bfloat16, "cuda:0", on_device=True)
-    sync()
+    model = build_model(cfg, args.seed)
     if args.mixed:
         kv_tokens = args.mixed * (4096 + 256 + args.page_size)
         opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=kv_tokens,
@@ -199,43 +156,50 @@ def main():
                             prefill_chunk=args.chunk, max_model_len=cfg["max_position_embeddings"],
                             use_graphs=not args.no_graphs)
         engine = LLMEngine(model, opt)
-        res = measure_mixed(engine, gen, args.mixed, vocab)
+        res = M.measure_mixed(engine, gen, args.mixed, vocab)
         print(json.dumps({"workload": "mixed", "model": shape_name, "layers_run": L, "chunk": args.chunk, **res}))
         return
     max_batch = args.batch if (args.no_points or args.only) else max(args.batch, 64)
-    total_steps = args.steps + args.warmup + decode_slack(max_batch, args.context) + 16
+    total_steps = args.steps + args.warmup + M.decode_slack(max_batch, args.context) + 16
     kv_tokens = max_batch * (args.context + total_steps + args.page_size) + args.prefill_tokens
     opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=kv_tokens, max_num_seqs=max_batch,
                         max_num_batched_tokens=max(4096, max_batch), prefill_chunk=2048,
                         max_model_len=cfg["max_position_embeddings"], use_graphs=not args.no_graphs)
     engine = LLMEngine(model, opt)
 
-    t_prefill = t_decode = None
+    pre = dec = None
     if args.only != "decode":
-        t_prefill = measure_prefill(engine, gen, args.prefill_tokens, vocab)
+        pre = M.measure_prefill(engine, gen, args.prefill_tokens, vocab)
     if args.only != "prefill":
-        t_decode = measure_decode(engine, gen, args.batch, args.context, args.steps, args.warmup, vocab)
+        dec = M.measure_decode(engine, gen, args.batch, args.context, args.steps, args.warmup, vocab)
     if args.only:
-        part = ({"prefill_ms": round(1000 * t_prefill, 3)} if t_prefill else
-                {"decode_ms_per_step": round(1000 * t_decode / args.steps, 4)})
+        part = ({"prefill_ms": round(1000 * pre["wall_s"], 3), "prefill_ms_device": round(1000 * pre["device_s"], 3)}
+                if pre else
+                {"decode_ms_per_step": round(1000 * dec["wall_s"] / args.steps, 4),
+                 "decode_ms_per_step_median": round(1000 * dec["step_median_s"], 4)})
         print(json.dumps({"only": args.only, **part, "batch": args.batch, "context": args.context}))
         return
     points = {}
     if not args.no_points:
         for b, key in ((1, "decode_b1"), (64, "decode_b64")):
             k = min(args.steps, 32)
-            dt = measure_decode(engine, gen, b, args.context, k, min(args.warmup, 4), vocab)
-            points[key] = round(b * k / dt, 1)
+            r = M.measure_decode(engine, gen, b, args.context, k, min(args.warmup, 4), vocab)
+            points[key] = round(b * k / r["wall_s"], 1)
+    ceilings = M.quick_ceilings("cuda:0")
 
+    t_decode, t_prefill = dec["wall_s"], pre["wall_s"]
     ms_step = 1000.0 * t_decode / args.steps
     value = args.batch * args.steps / t_decode
     mean_context = args.context + args.warmup + args.steps / 2.0
-    nbytes = decode_bytes(cfg, L, args.batch, mean_context)
+    nbytes = M.decode_bytes(cfg, L, args.batch, mean_context)
     achieved = nbytes / (t_decode / args.steps) / 1e9
-    pf = prefill_flops(cfg, L, args.prefill_tokens)
+    pf = M.prefill_flops(cfg, L, args.prefill_tokens)
     out = {
         "metric": "decode_tokens_per_s", "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
+        # the same steps by device events, step by step: their median (the wall clock above is their mean
+        # plus what the host adds)
+        "ms_per_step_median": round(1000.0 * dec["step_median_s"], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic (seeded random weights and token ids)",
         "config": {
@@ -248,11 +212,23 @@ def main():
             "hip_graphs": not args.no_graphs, "parallelism": "single GPU",
         },
         "prefill": {"value": round(args.prefill_tokens / t_prefill, 1), "tokens": args.prefill_tokens,
-                    "ms": round(1000.0 * t_prefill, 3), "frac": round(pf / t_prefill / MFMA_PEAK["bf16"], 4)},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+                    "ms": round(1000.0 * t_prefill, 3), "frac": round(pf / t_prefill / M.MFMA_PEAK["bf16"], 4),
+                    "ms_device": round(1000.0 * pre["device_s"], 3),
+                    "frac_of_measured": round(pf / t_prefill / (ceilings["mfma_bf16_TFLOPs"] * 1e12), 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": M.HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / M.HBM_PEAK_GBS, 4),
+                     "frac_of_measured": round(achieved / ceilings["stream_read_GBps"], 4)},
+        # what this machine gives, in this process, to a kernel that only reads and to one that only
+        # issues bfloat16 MFMAs from registers
+        "ceilings": ceilings,
         "points": points,
     }
+    if args.shape == "8b" and args.layers is None and not args.no_points and not args.no_large_points:
+        del engine, model
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        out["points"].update(large_points(args, gen))
     print(json.dumps(out))
 
 

@@ -32,6 +32,13 @@ def test_one_json_line_with_the_contract_keys():
         assert key in rec, key
     assert rec["n_gpus"] == 1 and rec["steps"] == 4 and rec["warmup"] == 2 and rec["dtype"] == "bf16"
     assert rec["value"] == pytest.approx(2 * 1000.0 / rec["ms_per_step"], rel=1e-3)
+    # the steps by device events: a median that the wall-clock mean cannot be far below
+    assert 0 < rec["ms_per_step_median"] < 3 * rec["ms_per_step"]
+    ceil = rec["ceilings"]
+    assert 2000 < ceil["stream_read_GBps"] < 8000 and 500 < ceil["mfma_bf16_TFLOPs"] < 2500
+    assert rec["roofline"]["frac_of_measured"] == pytest.approx(rec["roofline"]["achieved"] / ceil["stream_read_GBps"], abs=1e-3)
+    assert rec["prefill"]["frac_of_measured"] == pytest.approx(rec["prefill"]["frac"] * 2500.0 / ceil["mfma_bf16_TFLOPs"], rel=2e-2)
+    assert rec["prefill"]["ms_device"] <= rec["prefill"]["ms"] * 1.05
     cfg = rec["config"]
     assert len(cfg) <= 20 and all(not isinstance(v, (dict, list)) for v in cfg.values())
     assert cfg["layers"] == 36 and cfg["layers_run"] == 1 and cfg["global_batch"] == 2 and cfg["seq_len"] == 256

@@ -70,6 +70,18 @@ class ModelConfig:
     def to_dict(self) -> dict:
         raise NotImplementedError
 
+    def with_overrides(self, **values) -> "ModelConfig":
+        """The configuration with some of its config.json keys replaced, checked again as
+        a whole (a caller's option that overrides the file, like the reference's
+        ``_rope_freq_base``, test/main.cu:26).  A key the architecture does not have is an
+        error, not a silent no-op."""
+        d = self.to_dict()
+        unknown = [k for k in values if k not in d and not hasattr(self, k)]
+        if unknown:
+            raise ConfigError(f"{type(self).__name__} has no option {unknown}")
+        d.update(values)
+        return type(self).from_dict(d)
+
     def layer_specs(self) -> list[LayerSpec]:
         raise NotImplementedError
 

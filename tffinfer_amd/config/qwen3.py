@@ -42,6 +42,8 @@ class Qwen3Config(ModelConfig):
     extra: dict = field(default_factory=dict, repr=False)
 
     architecture = ARCHITECTURE
+    #: which config.json key an option of the caller overrides (the reference's _rope_freq_base)
+    caller_options = {"rope_freq_base": "rope_theta"}
 
     @classmethod
     def from_dict(cls, d: dict) -> "Qwen3Config":

@@ -33,6 +33,8 @@ class EngineOptions:
     num_pages: int | None = None
     #: tokens the cache holds; if None too, max_num_seqs * max_model_len capped by free memory
     kv_tokens: int | None = None
+    #: or bytes of device memory for keys and values, all layers together (whole pages of it are used)
+    kv_bytes: int | None = None
     max_num_seqs: int = 8
     max_num_batched_tokens: int = 2048
     prefill_chunk: int = 512
@@ -78,7 +80,15 @@ class LLMEngine:
         cfg = model.config
         max_len = min(opt.max_model_len or cfg.max_position_embeddings, cfg.max_position_embeddings)
         num_pages = opt.num_pages
-        if num_pages is None:
+        if sum(x is not None for x in (opt.num_pages, opt.kv_tokens, opt.kv_bytes)) > 1:
+            raise ValueError("give one of num_pages, kv_tokens and kv_bytes")
+        if num_pages is None and opt.kv_bytes is not None:
+            per_page = self._bytes_per_page(model, opt.page_size)
+            num_pages = int(opt.kv_bytes) // per_page if per_page else 1
+            if num_pages < 1:
+                raise ValueError(f"kv_bytes={opt.kv_bytes} holds no page: one page of {opt.page_size} tokens "
+                                 f"takes {per_page} bytes over all layers")
+        elif num_pages is None:
             tokens = opt.kv_tokens or opt.max_num_seqs * max_len
             num_pages = -(-tokens // opt.page_size) + opt.max_num_seqs
             num_pages = self._cap_pages_by_memory(model, num_pages, opt)
@@ -103,15 +113,21 @@ class LLMEngine:
         return cls(model, opt)
 
     @staticmethod
-    def _cap_pages_by_memory(model, num_pages: int, opt: EngineOptions) -> int:
-        free, _ = torch.cuda.mem_get_info(model.device)
+    def _bytes_per_page(model, page_size: int) -> int:
+        """Device bytes of one page number over all caches (every group gets as many pages)."""
         esz = 2 if model.dtype == torch.bfloat16 else 4
         per_page = 0
         seen = set()
         for cache_id, _, kv, _ in model.call_requirements():
             if kv is not None and cache_id not in seen:
                 seen.add(cache_id)
-                per_page += 2 * kv.num_kv_heads * kv.head_dim * opt.page_size * esz
+                per_page += 2 * kv.num_kv_heads * kv.head_dim * page_size * esz
+        return per_page
+
+    @classmethod
+    def _cap_pages_by_memory(cls, model, num_pages: int, opt: EngineOptions) -> int:
+        free, _ = torch.cuda.mem_get_info(model.device)
+        per_page = cls._bytes_per_page(model, opt.page_size)
         if per_page == 0:
             return max(1, num_pages)
         fit = int(free * opt.memory_fraction) // per_page

@@ -18,6 +18,8 @@ import threading
 import time
 from concurrent.futures import ThreadPoolExecutor
 
+from .. import log
+
 PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_NAME = "libtffinfer_hip.so"
@@ -112,7 +114,7 @@ def build(verbose: bool = True) -> str:
 
     def say(msg):
         if verbose:
-            print(f"[tffinfer_amd build] {msg}", file=sys.stderr, flush=True)
+            log.info("build: %s", msg)
 
     def ticker():
         while not done.wait(10.0):

@@ -796,13 +796,14 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tenso
     return (out, probs) if return_probs else out
 
 
-def measure_ceilings(device="cuda:0", gib: float = 4.0) -> dict:
+def measure_ceilings(device="cuda:0", gib: float = 4.0, quick: bool = False) -> dict:
     """What this machine gives to kernels that do nothing else: streaming reads
     from HBM into registers (a buffer of ``gib`` GiB, far larger than the
     caches) and back-to-back bfloat16 MFMAs at 1, 2 and 4 waves per SIMD, with
     operands that never change and (``..._varied_operands``) with operands that
     change from one instruction to the next as a real product's do: the matrix
-    cores then draw more power and the clock settles lower."""
+    cores then draw more power and the clock settles lower.  ``quick``: the
+    streaming read and the four-wave MFMA figure only (some 50 ms)."""
     L = _lib.load()
     dev = torch.device(device)
     cus = _num_cus(dev)
@@ -828,9 +829,11 @@ def measure_ceilings(device="cuda:0", gib: float = 4.0) -> dict:
                 for b in (8, 16, 32))
         out["stream_read_GBps"] = round(nbytes / t / 1e9, 1)
         iters = 20000
-        for waves in (1, 2, 4):
+        for waves in ((4,) if quick else (1, 2, 4)):
             t = timed(lambda: _lib.check(L.tff_probe_mfma(sink.data_ptr(), cus * waves, iters, 0, st)), 2)
             out[f"mfma_bf16_TFLOPs_{waves}_waves_per_simd"] = round(cus * waves * 4 * iters * 16 * 16384 / t / 1e12, 1)
+        if quick:
+            return out
         iters = 100000   # long enough for the clock to settle
         t = timed(lambda: _lib.check(L.tff_probe_mfma(sink.data_ptr(), cus * 4, iters, 1, st)), 2)
         out["mfma_bf16_TFLOPs_varied_operands"] = round(cus * 4 * 4 * iters * 16 * 16384 / t / 1e12, 1)

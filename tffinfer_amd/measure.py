@@ -1,0 +1,175 @@
+"""Measuring the engine: decode steps, prefill, a mixed workload, and what the
+machine gives to kernels that do nothing else.
+
+The reference's only timing is a wall clock around its decode loop that prints
+tokens per second (src/core/runtime/InferRuntime.cu:347, :377-378).  Here a
+phase is timed twice: by the wall clock around the whole phase, bracketed by
+device synchronisations (what a caller sees, host work included), and by
+device events between the steps, of which the median is reported (what the
+device needs for a step, without the odd slow one).  ``bench.py`` at the
+repository root and ``tffinfer --bench`` both call these functions.
+"""
+from __future__ import annotations
+
+import statistics
+import time
+
+import torch
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense, published
+
+
+def _get(c, key):
+    return c[key] if isinstance(c, dict) else getattr(c, key)
+
+
+def matmul_params_per_layer(c) -> int:
+    """Weights of a layer's four products, from a config.json dict or a typed configuration
+    of an attention + gated feed-forward layer."""
+    H, nq, nkv, d, I = (_get(c, "hidden_size"), _get(c, "num_attention_heads"), _get(c, "num_key_value_heads"),
+                        _get(c, "head_dim"), _get(c, "intermediate_size"))
+    return (nq + 2 * nkv) * d * H + nq * d * H + 3 * I * H
+
+
+def prefill_flops(c, L: int, T: int) -> float:
+    """Flops of one prompt of T tokens: the products of L layers, causal attention, the head
+    for one row."""
+    gemm = 2.0 * T * matmul_params_per_layer(c) * L
+    attn = 4.0 * _get(c, "num_attention_heads") * _get(c, "head_dim") * (T * (T + 1) / 2) * L
+    head = 2.0 * _get(c, "hidden_size") * _get(c, "vocab_size")
+    return gemm + attn + head
+
+
+def decode_bytes(c, L: int, batch: int, context: float, esz: int = 2) -> float:
+    """Bytes a decode step has to read: every weight once, and the cache of the live requests."""
+    weights = (matmul_params_per_layer(c) * L + _get(c, "hidden_size") * _get(c, "vocab_size")) * esz
+    kv = 2 * L * _get(c, "num_key_value_heads") * _get(c, "head_dim") * esz * batch * context
+    return weights + kv
+
+
+def random_prompt(gen, n: int, vocab: int) -> list:
+    return torch.randint(0, vocab, (n,), generator=gen).tolist()
+
+
+def decode_slack(batch: int, context: int, chunk: int = 2048) -> int:
+    """Steps the first request may decode while the last one still reads its prompt."""
+    return batch * (-(-context // chunk) + 1)
+
+
+def measure_prefill(engine, gen, T: int, vocab: int, reps: int = 5, warm: int = 2) -> dict:
+    """One prompt of T tokens through the step function, ``reps`` times after ``warm`` untimed
+    runs.  Returns the medians of the wall-clock times and of the device-event times, seconds."""
+    from .engine.batch import StepEntry
+    wall, dev = [], []
+    for i in range(reps + warm):
+        rid = f"prefill{i}"
+        toks = random_prompt(gen, T, vocab)
+        engine.runner.add_request(rid)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        logits = engine.runner.step([StepEntry(rid, toks, [T - 1])])
+        e1.record()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert logits.shape[0] == 1
+        engine.runner.free_request(rid)
+        if i >= warm:   # the first runs warm up (allocator, work tables, clocks)
+            wall.append(dt)
+            dev.append(e0.elapsed_time(e1) / 1e3)
+    return {"wall_s": statistics.median(wall), "device_s": statistics.median(dev), "reps": reps}
+
+
+def measure_decode(engine, gen, batch: int, context: int, steps: int, warmup: int, vocab: int) -> dict:
+    """Fills ``batch`` requests with ``context`` tokens each (untimed prefill), then times
+    ``steps`` decode steps of the whole engine (plan, tables, model, sampling, tokens back on
+    the host).  ``wall_s``: all the steps by the wall clock between two synchronisations;
+    ``step_median_s``: the median of the device-event intervals between consecutive steps."""
+    for _ in range(batch):
+        # requests that finish their prompt early decode while the others still prefill
+        engine.add_request(random_prompt(gen, context, vocab),
+                           max_new_tokens=warmup + steps + decode_slack(batch, context) + 8, ignore_eos=True)
+    # untimed: prompts, up to the first decode-only step
+    while any(r.num_pending > 1 for r in engine.scheduler.running) or engine.scheduler.waiting:
+        engine.step()
+    for _ in range(warmup):
+        out = engine.step()
+        assert len(out) == batch
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    events[0].record()
+    for i in range(steps):
+        out = engine.step()
+        events[i + 1].record()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert len(out) == batch
+    for r in list(engine.scheduler.running):
+        engine.abort(r.id)
+    while engine.has_work:      # a step launched ahead of the abort
+        engine.step()
+    gaps = [events[i].elapsed_time(events[i + 1]) / 1e3 for i in range(steps)]
+    return {"wall_s": dt, "step_median_s": statistics.median(gaps), "step_min_s": min(gaps),
+            "step_max_s": max(gaps), "steps": steps}
+
+
+def measure_mixed(engine, gen, requests: int, vocab: int, new_tokens: int = 256, lo: int = 128,
+                  hi: int = 4096) -> dict:
+    """Continuous batching: all requests arrive at once, the scheduler admits them as
+    slots and pages allow, cuts prompts into portions and decodes the others beside them."""
+    lens = torch.randint(lo, hi + 1, (requests,), generator=gen).tolist()
+    for n in lens:
+        engine.add_request(random_prompt(gen, n, vocab), max_new_tokens=new_tokens, ignore_eos=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    steps = 0
+    while engine.has_work:
+        engine.step()
+        steps += 1
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    st = engine.scheduler.stats
+    return {"requests": requests, "prompt_tokens": sum(lens), "generated_tokens": requests * new_tokens,
+            "seconds": round(dt, 3), "engine_steps": steps, "preemptions": st.preemptions,
+            "total_tokens_per_s": round((sum(lens) + requests * new_tokens) / dt, 1),
+            "generated_tokens_per_s": round(requests * new_tokens / dt, 1)}
+
+
+def quick_ceilings(device="cuda:0") -> dict:
+    """The two ceilings the benchmark line prices its fractions against besides the published
+    peaks, measured in the same process: streaming reads (GB/s) and back-to-back bfloat16
+    MFMAs from registers (TFLOP/s)."""
+    from .kernels import ops
+    c = ops.measure_ceilings(device, gib=2.0, quick=True)
+    return {"stream_read_GBps": c["stream_read_GBps"], "mfma_bf16_TFLOPs": c["mfma_bf16_TFLOPs_4_waves_per_simd"]}
+
+
+def square_product_rates(device="cuda:0", n: int = 8192, reps: int = 5) -> dict:
+    """A large square bfloat16 product [n, n] x [n, n]: the engine's own tiled kernel and, as a
+    yardstick only (it is not on the engine's path), the vendor library's through torch."""
+    from .kernels import ops
+    dev = torch.device(device)
+    a = torch.randn(n, n, dtype=torch.bfloat16, device=dev)
+    w = torch.randn(n, n, dtype=torch.bfloat16, device=dev)
+    wp = ops.pack_weight(w)
+
+    def timed(fn):
+        for _ in range(2):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize(dev)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize(dev)
+        return e0.elapsed_time(e1) / 1e3 / reps
+
+    flops = 2.0 * n * n * n
+    ours = timed(lambda: ops.linear(a, wp))
+    lib = timed(lambda: torch.matmul(a, w.t()))
+    return {"square_product_n": n, "square_product_TFLOPs": round(flops / ours / 1e12, 1),
+            "square_product_library_TFLOPs": round(flops / lib / 1e12, 1)}

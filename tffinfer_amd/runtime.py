@@ -16,14 +16,15 @@ ids, since the engine holds no tokenizer.
 """
 from __future__ import annotations
 
-import dataclasses
+import json
 import os
 from dataclasses import dataclass, field
 
 import torch
 
+from . import log
 from .engine.llm_engine import EngineOptions, LLMEngine
-from .models import build_model_skeleton, load_config
+from .models import build_model_skeleton, config_from_dict, load_config
 from .sampling import SamplingConfig
 from .weights import load_model_dir
 
@@ -49,7 +50,10 @@ class ModelConfig:
     _max_batches: int = 8              # most sequences in flight
     _max_batch_tokens: int = 2048      # token budget of a step
     _prefill_chunk: int = 512
-    _kv_tokens: int | None = None
+    _kv_tokens: int | None = None      # tokens the cache holds, or
+    _num_pages: int | None = None      # pages per group of layers, or
+    _kv_bytes: int | None = None       # bytes of device memory for keys and values
+    _use_graphs: bool = True
 
 
 class LLMInferRuntime:
@@ -60,12 +64,7 @@ class LLMInferRuntime:
         self._engine = None
         self._prompts = []
 
-    def load_model(self, model_files_path, params: ModelConfig) -> bool:
-        """``model_files_path``: a list whose first entry is the model folder
-        (or a file in it), as the reference takes a list of files."""
-        path = model_files_path[0] if isinstance(model_files_path, (list, tuple)) else model_files_path
-        if os.path.isfile(path):
-            path = os.path.dirname(path)
+    def _check_params(self, params: ModelConfig) -> torch.dtype:
         if params._rope_freq_scale != 1.0:
             raise ValueError("_rope_freq_scale other than 1 is not supported")
         if params._n_output != 1:
@@ -77,12 +76,49 @@ class LLMInferRuntime:
             if want != dtype:
                 raise ValueError(f"_kv_data_type={params._kv_data_type!r} does not match the "
                                  f"{'16' if params._use_f16 else '32'}-bit path")
-        config = load_config(path)
-        if params._rope_freq_base is not None and hasattr(config, "rope_theta"):
-            config = dataclasses.replace(config, rope_theta=float(params._rope_freq_base))
+        return dtype
+
+    @staticmethod
+    def _apply_caller_options(config, params: ModelConfig):
+        """Options of the caller that override the model's own configuration.  Which key of the
+        architecture an option means is the configuration class's business (``caller_options``)."""
+        if params._rope_freq_base is not None:
+            key = getattr(config, "caller_options", {}).get("rope_freq_base")
+            if key is None:
+                raise ValueError(f"{type(config).__name__} has no rotation base that _rope_freq_base could override")
+            config = config.with_overrides(**{key: float(params._rope_freq_base)})
+        return config
+
+    def load_model(self, model_files_path, params: ModelConfig) -> bool:
+        """``model_files_path``: a list whose first entry is the model folder
+        (or a file in it), as the reference takes a list of files."""
+        path = model_files_path[0] if isinstance(model_files_path, (list, tuple)) else model_files_path
+        if os.path.isfile(path):
+            path = os.path.dirname(path)
+        dtype = self._check_params(params)
+        config = self._apply_caller_options(load_config(path), params)
         model = build_model_skeleton(config)
         model.load_tensors(load_model_dir(path), dtype, "cuda:0", where=path)
         self._model, self._model_config, self._params = model, config, params
+        log.info("model %s: %s, %s", path, type(config).__name__, "bfloat16" if params._use_f16 else "float32")
+        return True
+
+    def random_model(self, config, seed: int, params: ModelConfig, on_device: bool = False) -> bool:
+        """A model with seeded random weights and no files: ``config`` is a config.json path, its
+        dict or a typed configuration.  The weights are those that ``write_random_model`` puts
+        into a folder for the same seed (``on_device``: drawn on the GPU instead, another stream
+        of numbers, for models too large to draw on the host in reasonable time)."""
+        if isinstance(config, (str, os.PathLike)):
+            with open(config) as f:
+                config = json.load(f)
+        if isinstance(config, dict):
+            config = config_from_dict(config)
+        dtype = self._check_params(params)
+        config = self._apply_caller_options(config, params)
+        model = build_model_skeleton(config)
+        model.init_random(int(seed), dtype, "cuda:0", on_device=on_device)
+        self._model, self._model_config, self._params = model, config, params
+        log.info("random model from seed %d: %s", seed, type(config).__name__)
         return True
 
     def init_runtime_context(self) -> bool:
@@ -93,7 +129,8 @@ class LLMInferRuntime:
         p = self._params
         opt = EngineOptions(dtype=self._model.dtype, page_size=p._page_size, max_num_seqs=p._max_batches,
                             max_num_batched_tokens=p._max_batch_tokens, prefill_chunk=p._prefill_chunk,
-                            max_model_len=p._n_ctx, kv_tokens=p._kv_tokens)
+                            max_model_len=p._n_ctx, kv_tokens=p._kv_tokens, num_pages=p._num_pages,
+                            kv_bytes=p._kv_bytes, use_graphs=p._use_graphs)
         self._engine = LLMEngine(self._model, opt)
         return True
 
