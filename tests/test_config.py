@@ -83,3 +83,13 @@ def test_round_trip_and_layer_data():
     assert specs[0].norm.args["eps"] == 1e-5
     sched = c.layer_schedule()
     assert [(s.layer, s.cache, s.writes_cache) for s in sched] == [(0, 0, True), (1, 1, True), (2, 2, True)]
+
+
+def test_a_model_of_built_in_parts_is_one_graph_piece():
+    """Every built-in part can be captured, so a decode step is one piece: embedding, every
+    entry of the run order, final norm and head."""
+    from helpers import TINY_B
+    from tffinfer_amd.models import build_model_skeleton, config_from_dict
+    model = build_model_skeleton(config_from_dict(dict(TINY_B)))
+    assert model.graph_safe()
+    assert model.graph_pieces() == [(True, ["embed", 0, 1, 2, "finish"])]

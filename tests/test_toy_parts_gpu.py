@@ -215,14 +215,47 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path):
         assert len(runner.cache.groups) == 1 and runner.cache.groups[0].cache_ids == [0, 2, 3]
         assert list(runner.cache.state_tensors) == [1]
         results = rl.run_steps_in_process(runner, steps)
-        done = {rid: 0 for rid in requests}
-        for s in steps:
-            row = 0
-            for e in s["entries"]:
-                for wnt in e["want"]:
-                    got = results[s["step"]][row]
-                    ref = refs[e["id"]][done[e["id"]] + wnt]
-                    err = float((got.double() - ref).abs().max() / ref.abs().max())
-                    assert err < 2e-5, f"{mode.__name__} step {s['step']} request {e['id']} pos {done[e['id']] + wnt}: {err:.2e}"
-                    row += 1
-                done[e["id"]] += len(e["tokens"])
+        _check(requests, refs, steps, results, mode.__name__)
+
+
+def _check(requests, refs, steps, results, what):
+    done = {rid: 0 for rid in requests}
+    for s in steps:
+        row = 0
+        for e in s["entries"]:
+            for wnt in e["want"]:
+                got = results[s["step"]][row]
+                ref = refs[e["id"]][done[e["id"]] + wnt]
+                err = float((got.double() - ref).abs().max() / ref.abs().max())
+                assert err < 2e-5, f"{what} step {s['step']} request {e['id']} pos {done[e['id']] + wnt}: {err:.2e}"
+                row += 1
+            done[e["id"]] += len(e["tokens"])
+
+
+def test_a_part_that_cannot_be_captured_splits_the_graph(tmp_path):
+    """The toy mixer and feed-forward loop on the host, so their layer call cannot go into a HIP
+    graph.  The decode step is then three pieces: a graph (embedding, first call), the toy layer
+    run eagerly on the live rows (it keeps state per request: a padding row must never reach
+    it), a graph (the other calls, final norm, head)."""
+    from safetensors.torch import load_file
+    from tffinfer_amd.engine.runner import ModelRunner
+    from tffinfer_amd.models import load_model
+    from tffinfer_amd.weights import write_random_model
+    ToyConfig = _register()
+    d = write_random_model(str(tmp_path / "toy"), ToyConfig(), seed=78, dtype="float32")
+    raw = load_file(d + "/model.safetensors")
+    model = load_model(d, torch.float32, DEV)
+    assert not model.graph_safe()
+    assert [(safe, items) for safe, items in model.graph_pieces()] == [
+        (True, ["embed", 0]), (False, [1]), (True, [2, 3, 4, "finish"])]
+    requests = {f"t{i}": random_tokens(n, V, 15 + i) for i, n in enumerate([9, 37, 20])}    # three live rows of four
+    refs = {rid: toy_reference(raw, toks) for rid, toks in requests.items()}
+    for mode in (rl.trace_tail, rl.trace_mixed):
+        steps = mode(requests)
+        pages = rl.max_live_tokens(steps, 8) // 8
+        runner = ModelRunner(model, page_size=8, num_pages=pages, max_seqs=4, use_graphs=True)
+        results = rl.run_steps_in_process(runner, steps)
+        assert runner._graphs, "no decode step went through the graphs"
+        for g in runner._graphs.values():
+            assert [pc.graph is not None for pc in g.pieces] == [True, False, True]
+        _check(requests, refs, steps, results, mode.__name__ + " with graphs")

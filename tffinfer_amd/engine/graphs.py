@@ -12,6 +12,13 @@ at position 0 that writes no key and whose logits nobody reads.
 Nothing in a captured step clears memory with a memset node, and the kernels
 take every size from the tables, so one graph serves any mix of context
 lengths.
+
+A model may hold parts that cannot be captured (a mixer that loops on the host
+over the step's entries).  The step is then cut into pieces at those layer
+calls (``DecoderModel.graph_pieces``): the pieces that can be captured are one
+graph each, the others run eagerly between the replays, on the live rows only
+(never on padding: such a part may keep state per request), and hand their
+result to the next graph through a fixed tensor.
 """
 from __future__ import annotations
 
@@ -73,6 +80,7 @@ class DecodeTables:
         hv[o[7]:o[7] + B] = np.arange(B)            # logit rows: every row
         hv[o[8]:o[8] + B] = -1                      # no-slot mapping
         self._row_state = [None] * B                # (request, life, table lengths) last written per row
+        self.host_start_pos, self.host_state_slots = [], []    # of the live rows of the last fill
         self._pad_rows(0)
 
     def block_table_row(self, group: int, row: int) -> np.ndarray:
@@ -104,9 +112,12 @@ class DecodeTables:
         R = len(entries)
         if R > self.B:
             raise ValueError(f"{R} entries do not fit a graph of {self.B} rows")
+        self.host_start_pos, self.host_state_slots = [], []
         for r, e in enumerate(entries):
             P = cache.num_tokens(e.req)
             life = cache.life(e.req)
+            self.host_start_pos.append(P)
+            self.host_state_slots.append(cache.slot(e.req))
             hv[o[0] + r] = e.tokens[0]
             hv[o[1] + r] = P
             hv[o[4] + r] = P
@@ -167,8 +178,7 @@ class DecodeGraph:
         b.host_state_slots = [0] * B
         b.reqs = [None] * B
         self.batch = b
-        self.graph = None
-        self.logits = None
+        self.pieces = [_Piece(safe, items) for safe, items in runner.model.graph_pieces()]
         self._copied = torch.cuda.Event()
 
     @property
@@ -179,11 +189,10 @@ class DecodeGraph:
         self._copied.synchronize()      # the last copy out of the host buffer is done
         self.tables.fill(entries)
 
-    def _forward(self):
+    def _context(self, batch):
         from .runner import StepContext
         rn = self.runner
-        ctx = StepContext(rn.ops, rn.act_dtype, self.batch, rn.max_model_len, rn._calls, rn.cache)
-        return rn.model.forward(ctx)
+        return StepContext(rn.ops, rn.act_dtype, batch, rn.max_model_len, rn._calls, rn.cache)
 
     def capture(self) -> None:
         rn = self.runner
@@ -196,31 +205,97 @@ class DecodeGraph:
         gc.collect()
         gc_was_on = gc.isenabled()
         gc.disable()
+        H = rn.model.config.hidden_size
         try:
             with torch.cuda.stream(side):
                 self.dev.copy_(self.host, non_blocking=True)
-                for _ in range(2):          # warm up: allocations, rotation tables
-                    self._forward()
-                side.synchronize()
-                self.graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(self.graph, stream=side):
-                    self.logits = self._forward()
+                ctx = self._context(self.batch)
+                resid = pending = None
+                for piece in self.pieces:
+                    if not piece.safe:
+                        # Not run here: every row is padding now, and such a part may keep state per
+                        # request.  At every step it runs on the live rows and leaves its result in
+                        # this tensor, which the next graph was captured to read.
+                        piece.pending = torch.zeros(self.B, H, dtype=torch.float32, device=rn.device)
+                        piece.resid, pending = resid, piece.pending
+                        continue
+
+                    def body(piece=piece, resid=resid, pending=pending):
+                        r, p, logits = rn.model.run_items(ctx, piece.items, resid, pending)
+                        if logits is None and p is not None:
+                            p = rn.ops.as_tensor(p)     # handed on as a plain tensor
+                        return r, p, logits
+
+                    for _ in range(2):          # warm up: allocations, rotation tables
+                        body()
+                    side.synchronize()
+                    piece.graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(piece.graph, stream=side):
+                        piece.resid, piece.pending, piece.logits = body()
+                    resid, pending = piece.resid, piece.pending
         finally:
             if gc_was_on:
                 gc.enable()
         torch.cuda.current_stream(rn.device).wait_stream(side)
         torch.cuda.synchronize(rn.device)
 
+    def _live_batch(self, R: int) -> StepBatch:
+        """The first R rows of the graph's tables as a step of their own, with the host's
+        copies that parts looping over entries read."""
+        g, t = self.batch, self.tables
+        b = StepBatch()
+        b.num_tokens = b.num_reqs = b.num_logit_rows = R
+        b.max_new_tokens = 1
+        b.max_context = max(t.host_start_pos) + 1
+        b.token_ids, b.positions, b.token_req = g.token_ids[:R], g.positions[:R], g.token_req[:R]
+        b.cu_tokens, b.start_pos, b.context_lens = g.cu_tokens[:R + 1], g.start_pos[:R], g.context_lens[:R]
+        b.state_slots, b.logit_rows = g.state_slots[:R], g.logit_rows[:R]
+        for gt in g.groups:
+            b.groups.append(GroupTables(gt.block_tables[:R], gt.slot_mapping[:R], gt.no_slot_mapping[:R]))
+        b.host_cu_tokens = list(range(R + 1))
+        b.host_start_pos = list(t.host_start_pos)
+        b.host_state_slots = list(t.host_state_slots)
+        b.reqs = [s[0] for s in t._row_state[:R]]
+        return b
+
     def run(self, entries, token_source: torch.Tensor | None = None) -> torch.Tensor:
         """``token_source``: int32 [len(entries)] on the device with the step's tokens, for a
-        step that is launched before the host knows them."""
+        step that is launched before the host knows them.  Returns the logits of the graph's
+        rows ([bucket, vocab], or [len(entries), vocab] if the step's last piece ran eagerly)."""
         self.fill(entries)
         self.dev.copy_(self.host, non_blocking=True)
         self._copied.record()
+        R = len(entries)
         if token_source is not None:
-            self.dev[self.offs[0]:self.offs[0] + len(entries)].copy_(token_source)
-        self.graph.replay()
-        return self.logits
+            self.dev[self.offs[0]:self.offs[0] + R].copy_(token_source)
+        rn = self.runner
+        logits = live = None
+        for piece in self.pieces:
+            if piece.safe:
+                piece.graph.replay()
+                logits = piece.logits
+                continue
+            if live is None:
+                live = self._context(self._live_batch(R))
+            # the piece before left the residual stream and its pending term in fixed tensors;
+            # this one adds to the stream's live rows in place
+            before = self.pieces[self.pieces.index(piece) - 1]
+            _, p, lg = rn.model.run_items(live, piece.items, piece.resid[:R],
+                                          None if before.pending is None else before.pending[:R])
+            if lg is not None:
+                logits = lg
+            else:
+                piece.pending[:R].copy_(rn.ops.as_tensor(p))
+        return logits
+
+
+class _Piece:
+    """A run of consecutive items of the step: one captured graph, or eager code."""
+    __slots__ = ("safe", "items", "graph", "resid", "pending", "logits")
+
+    def __init__(self, safe: bool, items: list):
+        self.safe, self.items = safe, items
+        self.graph = self.resid = self.pending = self.logits = None
 
 
 def graph_buckets(max_seqs: int) -> list[int]:

@@ -80,9 +80,9 @@ class ModelRunner:
             if group is not None:
                 k, v = self.cache.kv_tensors(cache_id)
             self._calls.append((cache_id, writes, group, k, v, self.cache.state_tensors.get(cache_id)))
-        # decode-only steps replay a HIP graph if every part of the model can be captured
+        # decode-only steps replay HIP graphs of the pieces of the model that can be captured
         self._graphs = {}
-        self._graph_buckets = graph_buckets(max_seqs) if (self.use_graphs and model.graph_safe()) else []
+        self._graph_buckets = graph_buckets(max_seqs) if (self.use_graphs and model.graph_pieces()) else []
 
     # ---- requests --------------------------------------------------------
     def add_request(self, req) -> int:

@@ -108,11 +108,36 @@ class DecoderModel:
 
     def graph_safe(self) -> bool:
         """True if every part launches only kernels that read the step's sizes
-        from device tables, so a decode step can be captured in a HIP graph."""
-        parts = [p for _, p in self._weighted_parts()]
-        for block in self.blocks:
-            parts.extend(p for _, p in _leaves("", block, {}))
+        from device tables, so a whole decode step can be captured in one HIP graph."""
+        pieces = self.graph_pieces()
+        return pieces is not None and len(pieces) == 1
+
+    def _item_graph_safe(self, item) -> bool:
+        if item == "embed":
+            parts = [self.embedding]
+        elif item == "finish":
+            parts = [self.final_norm, self.head]
+        else:
+            parts = [p for _, p in _leaves("", self.blocks[self.schedule[item].layer], {})]
         return all(getattr(p, "graph_safe", False) for p in parts)
+
+    def graph_pieces(self):
+        """The step as a list of pieces ``(capturable, items)``: items are "embed", the
+        indices of the run order, and "finish" (final norm and head), in order; consecutive
+        items that can all be captured in a HIP graph (or that all cannot: a part that loops
+        on the host over the step's entries) form a piece.  None when nothing is gained:
+        the embedding cannot be captured, or no layer call can."""
+        items = ["embed"] + list(range(len(self.schedule))) + ["finish"]
+        if not self._item_graph_safe("embed") or not any(self._item_graph_safe(i) for i in items[1:-1]):
+            return None
+        pieces = []
+        for it in items:
+            safe = self._item_graph_safe(it)
+            if pieces and pieces[-1][0] == safe:
+                pieces[-1][1].append(it)
+            else:
+                pieces.append((safe, [it]))
+        return pieces
 
     # ---- cache needs -----------------------------------------------------
     def call_requirements(self):
@@ -128,12 +153,27 @@ class DecoderModel:
     def forward(self, ctx) -> torch.Tensor:
         """Runs the tokens of ``ctx.batch`` and returns float32 logits
         [len(logit_rows), vocab]."""
+        items = ["embed"] + list(range(len(self.schedule))) + ["finish"]
+        _, _, logits = self.run_items(ctx, items, None, None)
+        return logits
+
+    def run_items(self, ctx, items, resid, pending):
+        """Runs some consecutive items of the step (see ``graph_pieces``) and returns
+        (residual stream, pending term, logits or None).  The residual stream is one float32
+        tensor from the embedding on, added to in place; the pending term is what the last
+        block returned for the next norm to add."""
         b = ctx.batch
-        resid = self.embedding.forward(ctx, b.token_ids)
-        pending = None
-        for idx, call in enumerate(self.schedule):
-            pending = self.blocks[call.layer].forward(ctx.for_call(idx), resid, pending)
-        if b.num_logit_rows == 0:
-            return torch.empty(0, self.config.vocab_size, dtype=torch.float32, device=resid.device)
-        y = self.final_norm.forward(ctx, resid, pending, rows=b.logit_rows)
-        return self.head.forward(ctx, y)
+        logits = None
+        for it in items:
+            if it == "embed":
+                resid, pending = self.embedding.forward(ctx, b.token_ids), None
+            elif it == "finish":
+                if b.num_logit_rows == 0:
+                    logits = torch.empty(0, self.config.vocab_size, dtype=torch.float32, device=resid.device)
+                else:
+                    y = self.final_norm.forward(ctx, resid, pending, rows=b.logit_rows)
+                    logits = self.head.forward(ctx, y)
+            else:
+                call = self.schedule[it]
+                pending = self.blocks[call.layer].forward(ctx.for_call(it), resid, pending)
+        return resid, pending, logits

@@ -77,7 +77,7 @@ class GQAttention(Mixer):
         ops, kv, b = ctx.ops, ctx.kv, ctx.batch
         nq, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
         qkv = ops.linear(x, self.w_qkv)
-        table = self.position.table(ctx.max_positions, x.device) if self.position is not None else None
+        table = self.position.cached_table(ctx.max_positions, x.device) if self.position is not None else None
         pairing = 1 if (self.position is not None and self.position.pairing == "interleaved") else 0
         o = ops.qkv_attention(qkv, nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0,
                               table, pairing, kv, b, self.window, self.scale)

@@ -83,6 +83,17 @@ class PositionEncoding(Part):
         for an encoding that leaves q and k as they are."""
         raise NotImplementedError
 
+    def cached_table(self, max_positions: int, device) -> torch.Tensor | None:
+        """``table`` asked for once per (positions, device) and kept for as long as the
+        encoding lives: the mixers call this, so that a subclass's ``table`` may build its
+        tensor on the host each time it is called, and so that a captured decode graph,
+        which holds the table's address, never sees it go."""
+        cache = self.__dict__.setdefault("_table_cache", {})
+        key = (int(max_positions), str(torch.device(device)))
+        if key not in cache:
+            cache[key] = self.table(max_positions, device)
+        return cache[key]
+
 
 class Norm(Part):
     def forward(self, ctx, resid: torch.Tensor, delta: torch.Tensor | None,
