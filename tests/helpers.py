@@ -78,7 +78,7 @@ def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
 # (relative step 2^-8).  One wrong page among a request's five moves the logits of these models
 # by 7e-2 and more.
 _TOL = {
-    "float32": {"A": 1e-6, "B": 2.5e-6, "C": 3e-6, "D": 2e-6, "mid": 1.2e-5},
+    "float32": {"A": 1e-6, "B": 2.5e-6, "C": 3e-6, "D": 2e-6, "mid": 1.2e-5, "large": 1.2e-5},
     "bfloat16": {"A": 1e-2, "B": 2e-2, "C": 1.8e-2, "D": 1.6e-2, "mid": 2.6e-2, "large": 2e-2},
 }
 

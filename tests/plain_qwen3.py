@@ -289,15 +289,16 @@ def fast_forward(cfg: dict, raw: dict, token_ids) -> torch.Tensor:
     eps = cfg.get("rms_norm_eps", 1e-6)
     theta = cfg.get("rope_theta", 10000.0)
     G = nq // nkv
-    ids = torch.as_tensor(list(token_ids), dtype=torch.long)
-    T = ids.numel()
     E = raw["model.embed_tokens.weight"]
+    where = E.device      # the weights may sit on a GPU, for the widths of the large models
+    ids = torch.as_tensor(list(token_ids), dtype=torch.long, device=where)
+    T = ids.numel()
     x = E[ids]
     dt = x.dtype
     pos = torch.arange(T, dtype=torch.float64)
     inv = torch.exp(-(2.0 * torch.arange(d // 2, dtype=torch.float64)) / d * math.log(theta))
     ang = pos[:, None] * inv[None, :]
-    cos, sin = torch.cos(ang).to(dt)[:, None, :], torch.sin(ang).to(dt)[:, None, :]
+    cos, sin = torch.cos(ang).to(dt)[:, None, :].to(where), torch.sin(ang).to(dt)[:, None, :].to(where)
 
     def norm(a, w):
         return a * torch.rsqrt((a * a).mean(-1, keepdim=True) + eps) * w
@@ -307,7 +308,7 @@ def fast_forward(cfg: dict, raw: dict, token_ids) -> torch.Tensor:
         return torch.cat([lo * cos - hi * sin, lo * sin + hi * cos], -1)
 
     wins = layer_windows(cfg)
-    ii = torch.arange(T)
+    ii = torch.arange(T, device=where)
     for i in range(cfg["num_hidden_layers"]):
         lw = _layer_weights(raw, i)
         h = norm(x, lw["input_layernorm"])

@@ -210,26 +210,43 @@ LARGE_SHAPES = {
 
 
 @pytest.mark.parametrize("shape", ["14b", "32b"])
-def test_bfloat16_against_float32_at_large_layer_sizes(shape):
+def test_large_layer_sizes_against_the_plain_implementation(shape, tmp_path):
     """One layer with the widths of the 14B and 32B models (inner sizes that are no power of
-    two, 5 and 8 query heads to a key head): the bfloat16 kernels against the engine's own
-    float32 path (which the small configurations pin to the plain implementation), for a
-    prompt in portions beside another request, then steps of two decoding requests."""
+    two, 5 and 8 query heads to a key head), weights from a folder: the float32 engine and the
+    bfloat16 engine against the plain implementation (in float64; its matrix products run on
+    the GPU here, the widths being what they are), for a prompt in portions beside another
+    request, then steps of two decoding requests.  The kernels that only these widths reach
+    (tiles that split K, the streaming product's other shapes) are thus pinned to the plain
+    implementation directly, not only to the engine's other precision."""
+    from plain_qwen3 import fast_forward, load_plain_model
     from tffinfer_amd.engine.batch import StepEntry
     from tffinfer_amd.engine.runner import ModelRunner
-    from tffinfer_amd.models import build_model_skeleton, config_from_dict
+    from tffinfer_amd.models import load_model
+    from tffinfer_amd.weights import write_random_model
     cfg = dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=1, vocab_size=5003,
                max_position_embeddings=2048, rms_norm_eps=1e-6, rope_theta=1000000.0,
                tie_word_embeddings=False, **LARGE_SHAPES[shape])
     V = cfg["vocab_size"]
+    d = write_random_model(str(tmp_path / shape), cfg, seed=11)
     a, b = random_tokens(712, V, 5), random_tokens(47, V, 6)
     steps = [[("a", a[:512], [0, 100, 511])], [("a", a[512:700], [187]), ("b", b[:40], [39])]]
     steps += [[("a", [a[700 + i]], [0]), ("b", [b[40 + i]], [0])] for i in range(7)]
     steps += [[("a", a[707:712], [0, 4])]]
+    # the plain logits at the places the steps ask for, in their order
+    pcfg, raw = load_plain_model(d, torch.float64)
+    raw = {k: v.cuda() for k, v in raw.items()}
+    full = {"a": fast_forward(pcfg, raw, a).cpu(), "b": fast_forward(pcfg, raw, b).cpu()}
+    del raw
+    torch.cuda.empty_cache()
+    want, done = [], {"a": 0, "b": 0}
+    for st in steps:
+        for r, t, w in st:
+            want += [full[r][done[r] + i] for i in w]
+            done[r] += len(t)
+    want = torch.stack(want)
     out = {}
     for dtype in (torch.float32, torch.bfloat16):
-        model = build_model_skeleton(config_from_dict(cfg))
-        model.init_random(11, dtype, "cuda:0", on_device=True)
+        model = load_model(d, dtype, "cuda:0")
         runner = ModelRunner(model, page_size=16, num_pages=64, max_seqs=2)
         runner.add_request("a")
         runner.add_request("b")
@@ -239,7 +256,9 @@ def test_bfloat16_against_float32_at_large_layer_sizes(shape):
         out[dtype] = torch.cat(rows)
         del runner, model
         torch.cuda.empty_cache()
-    assert out[torch.float32].shape[0] == 3 + 2 + 14 + 2
-    worst = rel_err(out[torch.bfloat16], out[torch.float32])
-    print(f"{shape}: bfloat16 against float32, worst rel. error {worst:.3e}")
-    assert worst <= tol("bfloat16", "large")
+    assert out[torch.float32].shape[0] == 3 + 2 + 14 + 2 == want.shape[0]
+    e32, e16 = rel_err(out[torch.float32], want), rel_err(out[torch.bfloat16], want)
+    print(f"{shape}: against the plain implementation, float32 {e32:.3e}, bfloat16 {e16:.3e}; "
+          f"bfloat16 against float32 {rel_err(out[torch.bfloat16], out[torch.float32]):.3e}")
+    assert e32 <= tol("float32", "large")
+    assert e16 <= tol("bfloat16", "large")
