@@ -771,6 +771,27 @@ def test_attention_mfma_portions_beside_decoding_requests(nq, nkv, d, ps, window
         _close(out.reshape(T, nq, d)[mine], ref, 1.5e-2, f"request {r}")
 
 
+@pytest.mark.parametrize("nq,nkv,d,ps,window", [(32, 8, 128, 16, 0), (8, 2, 32, 8, 300), (40, 2, 96, 8, 0)])
+def test_attention_mfma_short_portions_beside_decoding_requests(nq, nkv, d, ps, window):
+    """Portions of a few tokens (a wave of their own per 16 columns) beside requests that bring
+    one token with a long context: those go to the split-key kernel here too, not to a single
+    wave that walks all their keys."""
+    ops = _ops()
+    entries = [(900, 1), (0, 3), (1500, 1), (44, 2), (300, 1), (9, 1)]
+    batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=nq + d + 1)
+    assert batch.max_new_tokens * (nq // nkv) <= 64
+    T = batch.num_tokens
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(T, nq, d, generator=g).to(torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale)
+    assert "single_rows" in batch._attn_work, "the decoding requests did not get the split-key launch"
+    for r in range(len(entries)):
+        sel = (token_req == r).nonzero().flatten()
+        ref = _attn_ref(q[sel], ks[r], vs[r], positions[sel], window, scale)
+        _close(out.reshape(T, nq, d)[sel], ref, 1.5e-2, f"request {r}")
+
+
 @pytest.mark.parametrize("splits", [1, 2, 5])
 def test_attention_mfma_decode_more_pages_than_the_wave_keeps(splits):
     """A wave keeps 1024 page numbers at hand; with more pages in its run of keys it works

@@ -81,7 +81,9 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_async_kernel(
     static_assert((STAGES - 2) * LPW < 64, "vmcnt has 6 bits");
     __shared__ __attribute__((aligned(1024))) bf16_t smem[STAGES * FR * 512];
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    // (the wave's index as a scalar: what follows from it, the fragments it copies and where they
+    // land in LDS, is then worked out by the scalar unit)
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
     const int fr = lane & 15, fg = lane >> 4;
     // Blocks are handed to the eight XCDs in turn, and each XCD has an L2 of its own: block b

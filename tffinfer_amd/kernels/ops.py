@@ -600,9 +600,10 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
     cols = 128 if batch.max_new_tokens * G > 64 else 16
     which = "all"
     single = _entries(batch, "single")
-    if cols == 128 and single and batch.max_context >= 256:
+    if single and batch.max_context >= 256:
         # Requests that decode beside the portions have one token each and possibly long
-        # contexts: they get the split-key kernel of their own rather than one block each.
+        # contexts: they get the split-key kernel of their own rather than one block, or one
+        # wave, each for all their keys.
         which = "multi"
         work = _attention_work(batch, G, 16, q.device, "single")
         cache = batch._attn_work
@@ -616,7 +617,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
             batch, G, nkv, int(window), q.device, bins=block_bins, which=which, key_groups=key_groups, head_dim=d)
         launch(work, work.shape[0], block_items, num_blocks, 1, 128, 1, groups=groups)
     else:
-        work = _attention_work(batch, G, cols, q.device)
+        work = _attention_work(batch, G, cols, q.device, which)
         launch(work, work.shape[0], None, 0, 1, cols, 1)
     return out
 
