@@ -631,6 +631,56 @@ def test_attention_mfma_long_portions(nq, nkv, d, ps, window, bins, groups):
             _close(out.reshape(T, nq, d)[mine], ref, 1.5e-2, f"block attention, request {r}")
 
 
+@pytest.mark.parametrize("bins", [None, 3, 1])
+@pytest.mark.parametrize("nq,nkv,d,ps,window", [
+    (32, 8, 128, 16, 0), (8, 2, 32, 8, 300), (6, 3, 48, 8, 0), (5, 1, 128, 32, 0), (40, 2, 96, 8, 77),
+    (4, 2, 16, 16, 0), (7, 7, 112, 16, 130)])
+def test_attention_mfma_blocks_of_256_columns(nq, nkv, d, ps, window, bins):
+    """The blocks for long prompts, whose waves take two column tiles each, forced here on
+    portions of a few hundred tokens: requests whose columns end inside a wave's first or
+    second tile, a cached prefix, windows, one query head to a key head and twenty."""
+    ops = _ops()
+    entries = [(0, 700), (333, 200), (5, 1), (1000, 130), (64, 37)]
+    batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=nq * 5 + d)
+    T = batch.num_tokens
+    g = torch.Generator().manual_seed(14)
+    q = torch.randn(T, nq, d, generator=g).to(torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale, block_bins=bins,
+                             block_cols=256)
+    gen = ops.attention_generic(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv.k_cache, kv.v_cache, kv.block_tables,
+                                batch.token_req, batch.positions, window, scale)
+    _close(out, gen.double(), 1.5e-2, "blocks of 256 columns against the general kernel")
+    sel = torch.tensor([0, 1, 31, 32, 63, 64, 127, 128, 699, 700, 899, 900, 901, 1030, 1031, T - 1])
+    for r in range(len(entries)):
+        mine = sel[(token_req[sel] == r)]
+        if len(mine):
+            ref = _attn_ref(q[mine], ks[r], vs[r], positions[mine], window, scale)
+            _close(out.reshape(T, nq, d)[mine], ref, 1.5e-2, f"blocks of 256 columns, request {r}")
+
+
+def test_attention_mfma_picks_its_blocks_by_the_work():
+    """A prompt of 2,048 tokens goes to the blocks of 128 columns, one of 6,000 tokens to those
+    of 256 (and gives the same as the general kernel); head sizes beyond 128 never do."""
+    from types import SimpleNamespace
+    ops = _ops()
+    nq, nkv, d, ps = 32, 8, 128, 16
+    G = nq // nkv
+    for T, want in ((2048, 128), (6000, 256)):
+        b = SimpleNamespace(host_cu_tokens=[0, T], host_start_pos=[0])
+        assert ops._pick_block_cols(b, G, nkv, 0, DEV, "all", 128) == want
+        assert ops._pick_block_cols(SimpleNamespace(host_cu_tokens=[0, T], host_start_pos=[0]), G, nkv, 0, DEV, "all", 256) == 128
+    entries = [(0, 6000)]
+    batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=3)
+    T = batch.num_tokens
+    q = torch.randn(T, nq, d, generator=torch.Generator().manual_seed(15)).to(torch.bfloat16)
+    out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, 0, 1 / math.sqrt(d))
+    assert ("blocks", G, nkv, 256, 0, _ops()._num_cus(DEV) // nkv, "all", 1, d, None) in batch._attn_work
+    gen = ops.attention_generic(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv.k_cache, kv.v_cache, kv.block_tables,
+                                batch.token_req, batch.positions, 0, 1 / math.sqrt(d))
+    _close(out, gen.double(), 1.5e-2, "a long prompt against the general kernel")
+
+
 @pytest.mark.parametrize("nq,nkv,d,ps,window,splits", [
     (32, 8, 128, 16, 0, None), (32, 8, 128, 16, 0, 1), (32, 8, 128, 16, 0, 7), (4, 2, 16, 16, 0, 3),
     (8, 2, 32, 8, 24, 4), (40, 2, 96, 8, 0, 5), (6, 3, 48, 8, 100, None), (16, 1, 64, 32, 0, 64),

@@ -595,7 +595,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
     __shared__ __attribute__((aligned(1024))) bf16_t smem[STAGES * FRT * 512];
     __shared__ int32_t pages[ATTN_BT_LDS];
     static_assert(ATTN_STAGES >= 3, "the barrier between reads and MFMAs needs the copies one slice further ahead");
-    static_assert(KGRP == 1 || (size_t)STAGES * FRT * 1024 >= (size_t)NW * (DT * 1024 + 512),
+    static_assert(KGRP == 1 || (size_t)STAGES * FRT * 1024 >= (size_t)NW * NQT * (DT * 1024 + 512),
                   "the merge of the key groups borrows the stages");
     const int tid = threadIdx.x, lane = tid & 63, wave_all = tid >> 6;
     const int wave = wave_all % NW, kgi = wave_all / NW;     // column tile(s) and key group of this wave
@@ -846,31 +846,39 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
     if constexpr (KGRP > 1) {
         // The second key group hands its maxima, sums and accumulators to the first through the
         // stages (all copies have landed and all slices are read after the barrier).
-        static_assert(KGRP == 2 && NQT == 1, "the merge is written for two groups of single tiles");
-        float* mo = reinterpret_cast<float*>(smem) + wave * (DT * 256 + 128);
+        static_assert(KGRP == 2, "the merge is written for two groups");
+        float* mo = reinterpret_cast<float*>(smem) + wave * NQT * (DT * 256 + 128);
         __syncthreads();
         if (kgi == 1) {
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-                *reinterpret_cast<float4*>(mo + dt * 256 + lane * 4) =
-                    make_float4(oacc[0][dt][0], oacc[0][dt][1], oacc[0][dt][2], oacc[0][dt][3]);
-            mo[DT * 256 + lane * 2] = m_run[0];
-            mo[DT * 256 + lane * 2 + 1] = l_run[0];
+            for (int t = 0; t < NQT; ++t) {
+                float* mt = mo + t * (DT * 256 + 128);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    *reinterpret_cast<float4*>(mt + dt * 256 + lane * 4) =
+                        make_float4(oacc[t][dt][0], oacc[t][dt][1], oacc[t][dt][2], oacc[t][dt][3]);
+                mt[DT * 256 + lane * 2] = m_run[t];
+                mt[DT * 256 + lane * 2 + 1] = l_run[t];
+            }
         }
         __syncthreads();
         if (kgi == 1) continue;   // the next item, if any
-        const float m2 = mo[DT * 256 + lane * 2], l2 = mo[DT * 256 + lane * 2 + 1];
-        const float m = fmaxf(m_run[0], m2);
-        const float a1 = m_run[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m_run[0] - m) * sl2);
-        const float a2 = m2 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m2 - m) * sl2);
-        l_run[0] = l_run[0] * a1 + l2 * a2;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const float4 o2 = *reinterpret_cast<const float4*>(mo + dt * 256 + lane * 4);
-            oacc[0][dt][0] = oacc[0][dt][0] * a1 + o2.x * a2;
-            oacc[0][dt][1] = oacc[0][dt][1] * a1 + o2.y * a2;
-            oacc[0][dt][2] = oacc[0][dt][2] * a1 + o2.z * a2;
-            oacc[0][dt][3] = oacc[0][dt][3] * a1 + o2.w * a2;
+        for (int t = 0; t < NQT; ++t) {
+            const float* mt = mo + t * (DT * 256 + 128);
+            const float m2 = mt[DT * 256 + lane * 2], l2 = mt[DT * 256 + lane * 2 + 1];
+            const float m = fmaxf(m_run[t], m2);
+            const float a1 = m_run[t] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m_run[t] - m) * sl2);
+            const float a2 = m2 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m2 - m) * sl2);
+            l_run[t] = l_run[t] * a1 + l2 * a2;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const float4 o2 = *reinterpret_cast<const float4*>(mt + dt * 256 + lane * 4);
+                oacc[t][dt][0] = oacc[t][dt][0] * a1 + o2.x * a2;
+                oacc[t][dt][1] = oacc[t][dt][1] * a1 + o2.y * a2;
+                oacc[t][dt][2] = oacc[t][dt][2] * a1 + o2.z * a2;
+                oacc[t][dt][3] = oacc[t][dt][3] * a1 + o2.w * a2;
+            }
         }
     }
 
@@ -902,6 +910,19 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
                        int T_total, hipStream_t s, const AttnFuse* fuse = nullptr, int key_groups = 2) {
     int page_shift = 0;   // the page size is a power of two (tff_attention_mfma_supported)
     while ((1 << page_shift) < page_size) ++page_shift;
+    if (cols_per_wave == 256) {
+        // Eight waves of two column tiles each, one block a CU (a wave has 256 registers): every
+        // key and value fragment read from LDS feeds two MFMAs, half the LDS traffic per flop of
+        // the blocks below.  For prompts long enough to give every block several items.
+        if constexpr (DT <= 8) {
+            attn_mfma_block_kernel<DT, 2, 8, 1><<<dim3(num_blocks, nkv), 512, 0, s>>>(
+                q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
+                block_items, nq, nkv, page_size, page_shift, window, scale);
+            return tff_check_launch("attention_mfma_block256");
+        } else {
+            return tff_fail("attention_mfma: blocks of 256 columns take head sizes up to 128");
+        }
+    }
     if (cols_per_wave == 128) {   // blocks of eight waves that share their keys through LDS
         // Two groups of eight waves that take every other slice, where LDS holds their stages:
         // half as many slices one after the other for a block, which is what counts when there
@@ -970,11 +991,12 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
     TFF_REQUIRE((long)nkv * page_size * d < (1L << 31), "attention_mfma: a page of %d x %d x %d elements is too large", nkv, page_size, d);
     TFF_REQUIRE(q_stride >= nq * d && q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0,
                 "attention_mfma: query rows must be 16-byte aligned (stride %d)", q_stride);
-    TFF_REQUIRE(cols_per_wave == 16 || cols_per_wave == 128,
+    TFF_REQUIRE(cols_per_wave == 16 || cols_per_wave == 128 || cols_per_wave == 256,
                 "attention_mfma: bad tile width %d", cols_per_wave);
-    TFF_REQUIRE(cols_per_wave != 128 || (work && splits == 1),
-                "attention_mfma: blocks of 128 columns take a work table and no key split");
-    if (cols_per_wave == 128) {
+    TFF_REQUIRE(cols_per_wave < 128 || (work && splits == 1),
+                "attention_mfma: blocks of 128 or 256 columns take a work table and no key split");
+    TFF_REQUIRE(cols_per_wave != 256 || d <= 128, "attention_mfma: blocks of 256 columns take head sizes up to 128, not %d", d);
+    if (cols_per_wave >= 128) {
         if (!block_items) num_blocks = num_work;
         TFF_REQUIRE(num_blocks >= 0 && num_blocks <= num_work,
                     "attention_mfma: %d blocks for %d work items", num_blocks, num_work);

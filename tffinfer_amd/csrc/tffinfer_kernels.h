@@ -120,7 +120,9 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out,
 // are runs of 128 columns for a block of eight waves that stages keys and
 // values in LDS; block b works through items block_items[b] ..
 // block_items[b + 1] of the work table (block_items null: item b); key_groups 2 (head sizes
-// up to 128): a block is two groups of eight waves that take every other slice, 1: one group.  Head sizes 16..128 in steps of
+// up to 128): a block is two groups of eight waves that take every other slice, 1: one group.
+// cols_per_wave 256 (head sizes up to 128): the same with work items of 256 columns for blocks of eight waves of two
+// column tiles each, one block a CU, half the LDS reads per flop: for long prompts.  Head sizes 16..128 in steps of
 // 16, 192 and 256; pages of a power of two of tokens, at least 8; values transposed in their pages.
 TFF_API int tff_attention_mfma_supported(int d, int page_size);
 TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* part_o, float* part_ml,

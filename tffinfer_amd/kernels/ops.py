@@ -533,6 +533,35 @@ def _attention_block_work(batch, G: int, nkv: int, window: int, device, cols: in
     return cache[key]
 
 
+def _pick_block_cols(batch, G: int, nkv: int, window: int, device, which: str, head_dim: int) -> int:
+    """128 or 256 columns to a block of the prompt attention.  Blocks of 256 columns (two
+    column tiles a wave) read half as much from LDS per flop and run a quarter faster, but
+    there is one of them to a CU and each walks its items' slices alone: they pay once every
+    block has some 96 slices of 32 keys to go through (a prompt of about 3,500 tokens at four
+    query heads to a key head); below that the blocks of 128 columns, whose two groups of
+    waves share an item's slices, end sooner."""
+    if head_dim > 128:
+        return 128
+    cache = getattr(batch, "_attn_work", None)
+    if cache is None:
+        cache = batch._attn_work = {}
+    key = ("block_cols", G, nkv, window, which, head_dim)
+    if key not in cache:
+        cu, P = batch.host_cu_tokens, batch.host_start_pos
+        slices = 0
+        for r in _entries(batch, which):
+            ncols = (cu[r + 1] - cu[r]) * G
+            for c0 in range(0, ncols, 256):
+                first = P[r] + c0 // G
+                last = P[r] + (min(c0 + 256, ncols) - 1) // G
+                lo = max(0, first - window + 1) if window > 0 else 0
+                slices += last // 32 - lo // 32 + 1
+        num_cus = _num_cus(device) if torch.device(device).type == "cuda" else 256
+        per_cu = max(1, num_cus // max(1, nkv))
+        cache[key] = 256 if slices >= 96 * per_cu else 128
+    return cache[key]
+
+
 def pick_splits(waves: int, max_context: int) -> int:
     """Into how many runs the keys of a decoding request are split so that
     the launch has enough waves to pull on all of HBM: about 1024 waves, at
@@ -542,7 +571,8 @@ def pick_splits(waves: int, max_context: int) -> int:
 
 def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,
                    scale: float | None = None, splits: int | None = None,
-                   block_bins: int | None = None, key_groups: int | None = None) -> torch.Tensor:
+                   block_bins: int | None = None, key_groups: int | None = None,
+                   block_cols: int | None = None) -> torch.Tensor:
     """bfloat16 attention of the step's tokens on the matrix cores; decode-only
     steps split each request's keys over several waves and merge them.
     ``splits``, ``block_bins`` (blocks per kv head that share the work of
@@ -613,6 +643,16 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
         sp = splits if splits is not None else pick_splits(work.shape[0] * nkv, batch.max_context)
         launch(work, work.shape[0], None, 0, 1, 16, sp, cache["single_rows"])
     if cols == 128:
+        bcols = block_cols or _pick_block_cols(batch, G, nkv, int(window), q.device, which, d)
+        if bcols == 256:
+            # long prompts: items of 256 columns for blocks whose waves take two column tiles
+            # each (one block a CU, so one bin a CU and kv head)
+            per_cu = max(1, _num_cus(q.device) // max(1, nkv))
+            work, block_items, num_blocks, _ = _attention_block_work(
+                batch, G, nkv, int(window), q.device, cols=256, bins=block_bins or per_cu, which=which,
+                key_groups=1, head_dim=d)
+            launch(work, work.shape[0], block_items, num_blocks, 1, 256, 1, groups=1)
+            return out
         work, block_items, num_blocks, groups = _attention_block_work(
             batch, G, nkv, int(window), q.device, bins=block_bins, which=which, key_groups=key_groups, head_dim=d)
         launch(work, work.shape[0], block_items, num_blocks, 1, 128, 1, groups=groups)
