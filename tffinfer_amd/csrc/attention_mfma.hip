@@ -807,10 +807,16 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
             }
             float mt = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
                              fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-            mt = rows_max(mt);
-            const float m_new = fmaxf(m_run[t], mt);          // maxima are kept in raw score units
+            // The maximum over a column's four lanes and the rescale are needed only when some
+            // score of the slice exceeds a running maximum, which away from a prompt's first
+            // slices is rare: the same numbers either way (maxima are kept in raw score units).
+            float m_new = m_run[t], alpha = 1.f;
+            if (__any(mt > m_run[t])) {
+                mt = rows_max(mt);
+                m_new = fmaxf(m_run[t], mt);
+                alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((m_run[t] - m_new) * sl2);
+            }
             const float mb = m_new == -INFINITY ? 0.f : m_new * sl2;
-            const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((m_run[t] - m_new) * sl2);
             float ps = 0.f;
             bf16x8 pv;
 #pragma unroll
