@@ -660,13 +660,14 @@ def test_attention_mfma_blocks_of_256_columns(nq, nkv, d, ps, window, bins):
 
 
 def test_attention_mfma_picks_its_blocks_by_the_work():
-    """A prompt of 2,048 tokens goes to the blocks of 128 columns, one of 6,000 tokens to those
-    of 256 (and gives the same as the general kernel); head sizes beyond 128 never do."""
+    """A prompt of 2,048 tokens goes to the blocks of 128 columns, one of 32,768 tokens to those
+    of 256; head sizes beyond 128 never do.  A prompt of 6,000 tokens through either gives
+    what the general kernel gives."""
     from types import SimpleNamespace
     ops = _ops()
     nq, nkv, d, ps = 32, 8, 128, 16
     G = nq // nkv
-    for T, want in ((2048, 128), (6000, 256)):
+    for T, want in ((2048, 128), (6000, 128), (32768, 256)):
         b = SimpleNamespace(host_cu_tokens=[0, T], host_start_pos=[0])
         assert ops._pick_block_cols(b, G, nkv, 0, DEV, "all", 128) == want
         assert ops._pick_block_cols(SimpleNamespace(host_cu_tokens=[0, T], host_start_pos=[0]), G, nkv, 0, DEV, "all", 256) == 128
@@ -674,11 +675,12 @@ def test_attention_mfma_picks_its_blocks_by_the_work():
     batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=3)
     T = batch.num_tokens
     q = torch.randn(T, nq, d, generator=torch.Generator().manual_seed(15)).to(torch.bfloat16)
-    out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, 0, 1 / math.sqrt(d))
-    assert ("blocks", G, nkv, 256, 0, _ops()._num_cus(DEV) // nkv, "all", 1, d, None) in batch._attn_work
     gen = ops.attention_generic(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv.k_cache, kv.v_cache, kv.block_tables,
                                 batch.token_req, batch.positions, 0, 1 / math.sqrt(d))
-    _close(out, gen.double(), 1.5e-2, "a long prompt against the general kernel")
+    for cols in (None, 256):
+        out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, 0, 1 / math.sqrt(d), block_cols=cols)
+        _close(out, gen.double(), 1.5e-2, f"a long prompt against the general kernel (blocks: {cols})")
+    assert ("blocks", G, nkv, 256, 0, _ops()._num_cus(DEV) // nkv, "all", 1, d, None) in batch._attn_work
 
 
 @pytest.mark.parametrize("nq,nkv,d,ps,window,splits", [

@@ -731,6 +731,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
     // accumulators only when some column's maximum moved: away from the diagonal the vector
     // unit then has a fused multiply-add, an exponential and an addition per score to do.
     const float sl2 = scale * 1.44269504088896f;
+    const float slack = 8.0f / sl2;   // 8 in the exponent's units, as a raw score
     int t_min_pos[NQT], t_max_lo[NQT];
 #pragma unroll
     for (int t = 0; t < NQT; ++t) {
@@ -807,11 +808,15 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
             }
             float mt = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
                              fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-            // The maximum over a column's four lanes and the rescale are needed only when some
-            // score of the slice exceeds a running maximum, which away from a prompt's first
-            // slices is rare: the same numbers either way (maxima are kept in raw score units).
+            // m_run is the reference the exponentials are taken against: the largest score seen
+            // when it was last moved, in raw score units.  It is moved (the maximum over a
+            // column's four lanes, the accumulators rescaled) only when some score exceeds it by
+            // more than 8 in the exponent's units: until then p stays below 2^8, far from any
+            // overflow, and the quotient o / l does not depend on the reference.  Scores that
+            // creep up slice after slice, as they do towards the diagonal under a rotation,
+            // would otherwise rescale the accumulators in every slice.
             float m_new = m_run[t], alpha = 1.f;
-            if (__any(mt > m_run[t])) {
+            if (__any(mt > m_run[t] + slack)) {
                 mt = rows_max(mt);
                 m_new = fmaxf(m_run[t], mt);
                 alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((m_run[t] - m_new) * sl2);

@@ -535,11 +535,13 @@ def _attention_block_work(batch, G: int, nkv: int, window: int, device, cols: in
 
 def _pick_block_cols(batch, G: int, nkv: int, window: int, device, which: str, head_dim: int) -> int:
     """128 or 256 columns to a block of the prompt attention.  Blocks of 256 columns (two
-    column tiles a wave) read half as much from LDS per flop and run a quarter faster, but
-    there is one of them to a CU and each walks its items' slices alone: they pay once every
-    block has some 96 slices of 32 keys to go through (a prompt of about 3,500 tokens at four
-    query heads to a key head); below that the blocks of 128 columns, whose two groups of
-    waves share an item's slices, end sooner."""
+    column tiles a wave) read half as much from LDS and fetch half as many keys per flop.
+    Measured alone they are ahead from some 3,500 tokens on (a tenth at 32,768 tokens, a
+    quarter on the slower boxes of the pool); inside a whole prefill, between products that
+    hold the chip at its power limit, the two are within a percent or two of each other up to
+    16,384 tokens.  They are taken for the longest prompts only, where they were never behind:
+    4,096 slices of 32 keys a block and more (some 24,000 tokens at four query heads to a key
+    head)."""
     if head_dim > 128:
         return 128
     cache = getattr(batch, "_attn_work", None)
@@ -558,7 +560,7 @@ def _pick_block_cols(batch, G: int, nkv: int, window: int, device, which: str, h
                 slices += last // 32 - lo // 32 + 1
         num_cus = _num_cus(device) if torch.device(device).type == "cuda" else 256
         per_cu = max(1, num_cus // max(1, nkv))
-        cache[key] = 256 if slices >= 96 * per_cu else 128
+        cache[key] = 256 if slices >= 4096 * per_cu else 128
     return cache[key]
 
 
