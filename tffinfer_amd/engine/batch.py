@@ -74,10 +74,35 @@ def _pad4(n: int) -> int:
     return (n + 3) & ~3
 
 
-def build_step_batch(entries, cache, device, pinned=None) -> StepBatch:
+class PinnedTables:
+    """A pinned host buffer for the step's tables that is used again step after step: to pin
+    memory anew for every step costs more than the copy it speeds up.  The copy out of it is
+    asynchronous, so the next step waits for that copy (an event) before it writes."""
+
+    def __init__(self, ints: int = 1 << 16):
+        self._buf = torch.empty(int(ints), dtype=torch.int32, pin_memory=True)
+        self._copied = torch.cuda.Event()
+        self._busy = False
+
+    def take(self, ints: int) -> torch.Tensor:
+        if self._busy:
+            self._copied.synchronize()
+            self._busy = False
+        if ints > self._buf.numel():
+            self._buf = torch.empty(max(int(ints), 2 * self._buf.numel()), dtype=torch.int32, pin_memory=True)
+        return self._buf[:ints]
+
+    def copied(self) -> None:
+        """To be called right after the copy to the device was queued."""
+        self._copied.record()
+        self._busy = True
+
+
+def build_step_batch(entries, cache, device, pinned: PinnedTables | None = None) -> StepBatch:
     """Packs all tables of a step into one host buffer and sends it with one
     copy.  ``cache`` is the CacheManager; pages for the new tokens must have
-    been reserved."""
+    been reserved.  ``pinned``: the caller's reusable pinned buffer (else pageable
+    memory, and a copy that waits)."""
     b = StepBatch()
     R = len(entries)
     tok, pos, treq, cu, start, ctxl, slots, rows = [], [], [], [0], [], [], [], []
@@ -115,12 +140,14 @@ def build_step_batch(entries, cache, device, pinned=None) -> StepBatch:
     for s in sections:
         offs.append(total)
         total += _pad4(len(s))
-    host = torch.empty(max(total, 4), dtype=torch.int32, pin_memory=bool(pinned))
+    host = pinned.take(max(total, 4)) if pinned is not None else torch.empty(max(total, 4), dtype=torch.int32)
     hv = host.numpy()
     for s, o in zip(sections, offs):
         if s:
             hv[o:o + len(s)] = s
     dev = host.to(device, non_blocking=True)
+    if pinned is not None:
+        pinned.copied()
 
     def sl(i, n):
         return dev[offs[i]:offs[i] + n]
@@ -135,5 +162,4 @@ def build_step_batch(entries, cache, device, pinned=None) -> StepBatch:
         b.groups.append(GroupTables(bt, sl(si + 1, T), no_slot))
     b.host_cu_tokens, b.host_start_pos, b.host_state_slots = cu, start, slots
     b.reqs = [e.req for e in entries]
-    b._host_buffer = host  # keeps the pinned buffer alive until the copy is done
     return b

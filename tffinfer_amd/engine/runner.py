@@ -14,7 +14,7 @@ import torch
 from ..cache.block_pool import OutOfPages
 from ..cache.manager import CacheManager
 from ..kernels import ops as _ops
-from .batch import KVView, StepBatch, StepEntry, build_step_batch
+from .batch import KVView, PinnedTables, StepBatch, StepEntry, build_step_batch
 from .graphs import DecodeGraph, graph_buckets
 
 
@@ -80,6 +80,7 @@ class ModelRunner:
             if group is not None:
                 k, v = self.cache.kv_tensors(cache_id)
             self._calls.append((cache_id, writes, group, k, v, self.cache.state_tensors.get(cache_id)))
+        self._pinned = PinnedTables()     # the tables of steps that run eagerly leave through it
         # decode-only steps replay HIP graphs of the pieces of the model that can be captured
         self._graphs = {}
         self._graph_buckets = graph_buckets(max_seqs) if (self.use_graphs and model.graph_pieces()) else []
@@ -153,7 +154,7 @@ class ModelRunner:
                 and all(len(e.tokens) == 1 for e in entries):
             return self._step_graph(entries, token_source)
         with torch.cuda.device(self.device):
-            batch = build_step_batch(entries, self.cache, self.device)
+            batch = build_step_batch(entries, self.cache, self.device, self._pinned)
             if token_source is not None:
                 batch.token_ids[:len(entries)].copy_(token_source)
             ctx = StepContext(self.ops, self.act_dtype, batch, self.max_model_len, self._calls, self.cache)
