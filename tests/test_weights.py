@@ -92,6 +92,17 @@ def test_tied_model_ignores_a_stored_head(tmp_path):
     t["lm_head.weight"] = t["model.embed_tokens.weight"].clone()
     model = build_model_skeleton(config_from_dict(TINY_A))
     check_weights(model.expected_tensors(), t, {"lm_head.weight"})
+    # the model says so when it passes a stored copy over
+    import io
+    from tffinfer_amd import log
+    buf = io.StringIO()
+    level, app, stream = log.get_level(), log._State.app, log._State.stream
+    log.init("unit", "info", buf)
+    try:
+        model.load_tensors(t, torch.float32, "cpu", where=d)
+    finally:
+        log.init(app, level, stream)
+    assert "lm_head.weight" in buf.getvalue() and buf.getvalue().startswith("W")
 
 
 def test_broken_files(tmp_path):
@@ -117,6 +128,12 @@ def test_broken_files(tmp_path):
         load_file(str(tmp_path / "u.safetensors"))
     with pytest.raises(WeightFileError, match="neither"):
         load_model_dir(str(tmp_path / "empty_dir_that_is_missing"))
+    # a tensor named twice in the header (a JSON parser keeps the last without a word)
+    hdr = (b'{"w": {"dtype": "F32", "shape": [1], "data_offsets": [0, 4]}, '
+           b'"w": {"dtype": "F32", "shape": [1], "data_offsets": [4, 8]}}')
+    (tmp_path / "d.safetensors").write_bytes(struct.pack("<Q", len(hdr)) + hdr + b"\0" * 8)
+    with pytest.raises(WeightFileError, match="more than once"):
+        load_file(str(tmp_path / "d.safetensors"))
 
 
 def test_sharded_folder(tmp_path):

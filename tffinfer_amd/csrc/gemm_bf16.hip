@@ -624,7 +624,22 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
 // and 32B shapes at 96 .. 4,096 rows on an MI355X (156 cases, every tile with 1 .. 8 parts),
 // where its pick is within 7 % of the best candidate everywhere and 0.3 % from it on average.
 struct GemmPlan { int tile; int bn; int splits; };   // tile = rows of a block tile
+// Compute units of the current device (256 on an MI355X, which the rates below were fitted on; a
+// device with another count gets plans for its own number of blocks a round).  256 if it cannot
+// be asked.
+static int device_cus() {
+    static int cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
 static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
+    const double CUS = (double)device_cus();
     // Up to 16 rows: the streaming kernel, a block per 16 columns, unless those blocks go badly
     // round the 256 CUs (320 of them take as long as 512 would: N = 5120), the caller takes
     // partial sums anyway and the weight is large enough for the gain (three eighths of its
@@ -632,7 +647,7 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
     // its epilogue: then the tiles below, whose blocks split K as finely as it takes.
     if (M <= 16) {
         const int nb = (N + 15) / 16;
-        const double fill = (double)nb / (((nb + 255) / 256) * 256.0);
+        const double fill = (double)nb / (ceil(nb / CUS) * CUS);
         if (glu || !keep || fill >= 0.8 || (double)N * K < 40e6) return {0, 0, 1};
     }
     const int nk = (K + 63) / 64;
@@ -648,7 +663,7 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
         double best_t = 1e30;
         for (int S = 1; S <= 8; S *= 2) {
             if (S > 1 && nk / S < 4) break;
-            double t = ceil(blocks * S / 256.0) * ceil((double)nk / S) * 0.63 + ceil(blocks * S / 512.0) * 4.0 + 1.0;
+            double t = ceil(blocks * S / CUS) * ceil((double)nk / S) * 0.63 + ceil(blocks * S / (2.0 * CUS)) * 4.0 + 1.0;
             if (S > 1) t += keep ? (S - 1.0) * M * N * 4.0 / 4e6 : (double)S * M * N * 8.0 / 4e6 + 3.0;
             if (t < best_t) { best_t = t; best_s = S; }
         }
@@ -665,7 +680,7 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
             if (glu && c.bn == 192) break;   // gate and up groups come in pairs: an even number a wave
             if (S > 1 && nk / S < 8) break;
             const double blocks = (double)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * S;
-            const double rounds = ceil(blocks / (256.0 * c.slots));
+            const double rounds = ceil(blocks / (CUS * c.slots));
             // a round: the blocks' work at the tile's rate plus some 3 us to fill the pipeline and
             // store the tile; a last round that fills part of the machine takes as long as a full one
             const double round_us = 2.0 * c.bm * c.bn * ((double)K / S) * c.slots / c.rate + 3.0;

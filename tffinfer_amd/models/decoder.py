@@ -83,7 +83,12 @@ class DecoderModel:
         that is wrong) and hands every part its tensors."""
         ignorable = set(self.names.ignorable)
         if self.config.tie_word_embeddings:
-            ignorable.add(f"{self.names.head}.weight")  # a stored copy of the tied head is not used
+            head = f"{self.names.head}.weight"
+            ignorable.add(head)
+            if head in found:
+                from .. import log
+                log.warning("%s: '%s' is stored but the configuration ties the head to the embedding; "
+                            "the stored copy is not used", where or "weights", head)
         check_weights(self.expected_tensors(), found, ignorable, where)
         self.dtype, self.device = dtype, torch.device(device)
         for prefix, part in self._weighted_parts():

@@ -48,10 +48,23 @@ def read_header(path: str) -> tuple[dict, int]:
         if n <= 0 or 8 + n > size:
             raise WeightFileError(f"{path}: header length {n} does not fit the file of {size} bytes")
         raw = f.read(n)
+    twice = []
+
+    def pairs(items):
+        # a name that stands twice in an object: json.loads would keep the last without a word
+        seen = {}
+        for k, v in items:
+            if k in seen:
+                twice.append(k)
+            seen[k] = v
+        return seen
+
     try:
-        header = json.loads(raw.decode("utf-8"))
+        header = json.loads(raw.decode("utf-8"), object_pairs_hook=pairs)
     except (UnicodeDecodeError, ValueError) as e:
         raise WeightFileError(f"{path}: header is not JSON: {e}") from None
+    if twice:
+        raise WeightFileError(f"{path}: the header names {sorted(set(twice))} more than once")
     if not isinstance(header, dict):
         raise WeightFileError(f"{path}: header is not a JSON object")
     return header, 8 + n
