@@ -183,3 +183,64 @@ def test_steps_launched_ahead_against_the_plain_implementation(model_dirs, dtype
         check_choices(d, r, dtype, sc[i])
     assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
     assert eng.runner.cache.slots.num_free == 4
+
+
+@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("name,dtype", [("B", "float32"), ("D", "bfloat16"), ("D", "float32"), ("A", "bfloat16")])
+def test_random_workloads_on_small_pools(model_dirs, name, dtype, seed):
+    """Random workloads (lengths, arrival steps, sampling, stop lengths, an abort) on pools that
+    hold about half of what the requests need together, with decode graphs and steps launched
+    ahead: whatever the schedule turns out to be (admissions, portions, preemptions, windows that
+    give pages back, rows that change hands), every kept row of logits matches the plain logits
+    of the request's own sequence and every token is the plain sampler's choice."""
+    import random
+    from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
+    rng = random.Random(1000 * seed + 17 * ord(name) + (7 if dtype == "float32" else 0))
+    d = model_dirs[name]
+    cfg = read_config(d)
+    V, limit = cfg["vocab_size"], min(cfg["max_position_embeddings"], 160)
+    n = rng.randrange(3, 7)
+    ps = rng.choice([8, 16])
+    reqs, need = [], 0
+    for i in range(n):
+        plen, new = rng.randrange(1, 60), rng.randrange(2, 45)
+        new = min(new, limit - plen - 1)
+        sc = SamplingConfig("random", temperature=rng.choice([0.6, 1.0, 1.3]), seed=rng.randrange(1 << 20)) \
+            if rng.random() < 0.5 else SamplingConfig()
+        reqs.append(dict(prompt_ids=random_tokens(plen, V, 7000 + 31 * seed + i), sampling=sc, max_new_tokens=new,
+                         ignore_eos=True, request_id=i))
+        need += -(-(plen + new) // ps)
+    biggest = max(-(-(len(r["prompt_ids"]) + r["max_new_tokens"]) // ps) for r in reqs)
+    pages = max(biggest + 1, need // 2)
+    slots = rng.randrange(2, 5)
+    opt = EngineOptions(dtype=dtype, page_size=ps, num_pages=pages, max_num_seqs=slots,
+                        max_num_batched_tokens=rng.choice([16, 32, 64]), prefill_chunk=rng.choice([8, 16, 24]),
+                        max_model_len=limit, use_graphs=True, run_ahead=True)
+    eng = LLMEngine.from_model_dir(d, opt)
+    eng.keep_logits = True
+    arrivals = {}
+    for r in reqs:
+        arrivals.setdefault(rng.randrange(0, 40), []).append(r)
+    victim = rng.randrange(n) if rng.random() < 0.5 else None
+    state = {}
+
+    def on_step(step):
+        r = eng._requests.get(victim)
+        if victim is not None and "done" not in state and r is not None and r.status == "running" and len(r.output) >= 2:
+            eng.abort(victim)
+            state["done"] = True
+
+    drive(eng, arrivals, on_step)
+    st = eng.scheduler.stats
+    print(f"{name} {dtype} seed {seed}: {n} requests, {pages} pages of {ps}, {slots} slots: {st.steps} steps, "
+          f"{st.preemptions} preemptions, {eng.steps_ahead} steps launched ahead, {len(eng.runner._graphs)} graphs")
+    for r in reqs:
+        res = eng.pop_result(r["request_id"])
+        if res.finish_reason == "abort":
+            assert r["request_id"] == victim
+        else:
+            assert res.finish_reason == "length" and len(res.output) == r["max_new_tokens"]
+        assert len(res.logits) == len(res.output)
+        check_choices(d, res, dtype, r["sampling"])
+    assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
+    assert eng.runner.cache.slots.num_free == slots
