@@ -917,6 +917,58 @@ def test_attention_mfma_far_key_and_window_edge():
             assert hit == sees, f"n={n} window={window}: far key {'missed' if sees else 'seen'}"
 
 
+@pytest.mark.parametrize("cols", [128, 256])
+def test_attention_mfma_blocks_far_key_and_window_edge(cols):
+    """The same for the kernels whose blocks share keys through LDS (a portion of 40 tokens,
+    blocks of 128 and of 256 columns): every token's query points at one key far back, whose
+    score towers over all others (the softmax's reference has to jump to it and stay), and each
+    token's window either just holds that key or has just passed it."""
+    ops = _ops()
+    nq, nkv, d, ps = 8, 2, 64, 16
+    P, n, far = 900, 40, 517
+    entries = [(P, n)]
+    batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=19)
+    q = torch.randn(1, nq, d).to(torch.bfloat16).repeat(n, 1, 1)
+    for gidx in range(nkv):
+        q[:, gidx * 4:(gidx + 1) * 4] = q[:, gidx * 4:gidx * 4 + 1]
+        kfar = (40 * q[0, gidx * 4].float() / q[0, gidx * 4].float().norm()).to(torch.bfloat16)
+        page = int(kv.block_tables[0, far // ps])
+        kv.k_cache[page, gidx, far % ps] = kfar.to(DEV)
+        ks[0][far, gidx] = kfar
+    # token t is at position P + t: a window of P - far + 1 + t0 holds the far key for t <= t0 only
+    for window, last_seeing in ((0, n - 1), (P - far + 1 + 17, 17), (P - far + 1, 0), (P - far, -1)):
+        ref = _attn_ref(q, ks[0], vs[0], positions, window, 1 / math.sqrt(d))
+        out = ops.attention_mfma(q.reshape(n, nq * d).to(DEV), nq, nkv, d, kv, batch, window, 1 / math.sqrt(d),
+                                 block_cols=cols)
+        _close(out.reshape(n, nq, d), ref, 1.5e-2, f"window={window}")
+        for t in range(n):
+            hit = torch.allclose(out.reshape(n, nq, d)[t, 0].float().cpu(), vs[0][far, 0].float(), atol=5e-2)
+            assert hit == (t <= last_seeing), f"window={window}, token {t}: far key {'missed' if t <= last_seeing else 'seen'}"
+
+
+def test_attention_mfma_blocks_scores_that_creep_up():
+    """Keys whose scores rise a little with every slice, by less than the slack the softmax's
+    reference is given, for hundreds of keys, then by a lot: what the kernel sums against a
+    reference that lags behind must equal the float64 softmax."""
+    ops = _ops()
+    nq, nkv, d, ps = 4, 1, 64, 16
+    P, n = 0, 600
+    batch, kv, ks, vs, positions, token_req = _fake_step([(P, n)], ps, nkv, d, torch.bfloat16, seed=29)
+    u = torch.zeros(d)
+    u[0] = 1.0
+    q = (8.0 * u).to(torch.bfloat16).repeat(n, nq, 1)            # every query: 8 along the first axis
+    for j in range(n):
+        rise = 0.02 * j if j < 500 else 10.0 + 0.5 * (j - 500)    # scaled score = rise (d = 64: 8 * k0 / 8)
+        k = torch.zeros(d)
+        k[0] = rise
+        ks[0][j, 0] = k.to(torch.bfloat16)
+        kv.k_cache[int(kv.block_tables[0, j // ps]), 0, j % ps] = k.to(torch.bfloat16).to(DEV)
+    ref = _attn_ref(q, ks[0], vs[0], positions, 0, 1 / math.sqrt(d))
+    for cols in (128, 256):
+        out = ops.attention_mfma(q.reshape(n, nq * d).to(DEV), nq, nkv, d, kv, batch, 0, 1 / math.sqrt(d), block_cols=cols)
+        _close(out.reshape(n, nq, d), ref, 1.5e-2, f"creeping scores, blocks of {cols}")
+
+
 @pytest.mark.parametrize("M", [1, 8, 20, 50, 200])
 @pytest.mark.parametrize("I,K", [(200, 96), (64, 64), (1000, 256), (12288, 512), (8200, 104)])
 def test_linear_with_gated_epilogue(M, I, K):
