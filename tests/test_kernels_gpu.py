@@ -192,27 +192,30 @@ def test_norm_taken_into_the_products_on_either_side(M, H, K, N2, glu):
     assert isinstance(z3, torch.Tensor) and torch.equal(z3, z) and torch.equal(r3, r2)
 
 
-@pytest.mark.parametrize("M,N,K,glu", [(2000, 8100, 328, False), (1500, 8000, 1096, False), (2048, 4096, 12288, False),
+def _gemm_plan(M, N, K, glu=0, keep=0):
+    import ctypes
+    from tffinfer_amd.kernels import lib
+    r, c, s = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    assert lib.load().tff_gemm_plan(M, N, K, glu, keep, ctypes.byref(r), ctypes.byref(c), ctypes.byref(s)) == 0
+    return r.value, c.value, s.value
+
+
+@pytest.mark.parametrize("M,N,K,glu", [(2000, 8100, 328, False), (1500, 8000, 1096, False), (2048, 4096, 12296, False),
                                          (2000, 16160, 328, True), (1024, 16000, 328, False),
                                          (2048, 6144, 520, False), (2000, 6100, 328, False)])
 def test_linear_on_the_largest_tile(M, N, K, glu):
-    """Shapes for which the plan takes 256 x 256 or 256 x 192 tiles: an odd number of
-    32-k steps, a last step that is not whole, rows and columns that do not fill the tiles, K
-    split over blocks with the partial sums added or handed on.  The float32 product of the
-    same (bfloat16) numbers is the yardstick."""
-    import ctypes
-    from tffinfer_amd.kernels import lib
+    """Shapes for which the plan takes the sixteen-wave 256 x 256 or 256 x 192 tiles (K no
+    multiple of 64): an odd number of 32-k steps, a last step that is not whole, rows and columns
+    that do not fill the tiles, K split over blocks with the partial sums added or handed on.  The
+    float32 product of the same (bfloat16) numbers is the yardstick."""
     ops = _ops()
-    L = lib.load()
     g = torch.Generator().manual_seed(N)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
-    r, c, sp = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     if glu:
         I = N // 2
         gate = (torch.randn(I, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
         up = (torch.randn(I, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
-        assert L.tff_gemm_plan(M, 2 * I, K, 1, 0, ctypes.byref(r), ctypes.byref(c), ctypes.byref(sp)) == 0
-        assert (r.value, c.value) == (256, 256)
+        assert _gemm_plan(M, 2 * I, K, 1)[:2] == (256, 256)
         y = ops.linear(x, ops.pack_gate_up(gate, up), out_dtype=torch.float32)
         a, b = ops.linear(x.float(), gate.float()), ops.linear(x.float(), up.float())
         ref = a / (1 + torch.exp(-a)) * b
@@ -222,15 +225,73 @@ def test_linear_on_the_largest_tile(M, N, K, glu):
     pw = ops.pack_weight(w)
     ref = ops.linear(x.float(), w.float())
     for keep in (0, 1):
-        assert L.tff_gemm_plan(M, N, K, 0, keep, ctypes.byref(r), ctypes.byref(c), ctypes.byref(sp)) == 0
+        r, c, sp = _gemm_plan(M, N, K, 0, keep)
         if K < 12288 or keep:       # (the long K runs on this tile when its two halves are handed on)
-            assert r.value == 256 and c.value in ((192,) if N in (6144, 6100) else (192, 256)), (r.value, c.value, sp.value)
+            assert r == 256 and c in ((192,) if N in (6144, 6100) else (192, 256)), (r, c, sp)
         y = ops.linear(x, pw, out_dtype=torch.float32, partials=bool(keep))
-        if keep and sp.value > 1:
-            assert y.dim() == 3 and y.shape[0] == sp.value
-        _close(ops.as_tensor(y), ref, 3e-5, f"product (keep={keep}, {sp.value} parts)")
+        if keep and sp > 1:
+            assert y.dim() == 3 and y.shape[0] == sp
+        _close(ops.as_tensor(y), ref, 3e-5, f"product (keep={keep}, {sp} parts)")
     yb = ops.linear(x, pw)       # bfloat16 result
     _close(yb, ref, 8e-3, "bfloat16 result")
+
+
+FOUR_WAVE_CASES = [
+    # M, N, K, gated: K in units of 64, so tiles of 256 rows are the four-wave kernel's
+    (2048, 6144, 256, False),      # 256 x 192, whole tiles
+    (2000, 8100, 320, False),      # 256 x 256, ragged rows and columns, an odd number of units
+    (2304, 2100, 64, False),       # 256 x 128, nine row tiles (a last group of one), a single unit of K
+    (1999, 4100, 2048, False),     # 256 x 192, a last column tile of a few columns
+    (2048, 4096, 1024, False),     # 256 x 128
+    (1024, 4096, 12288, False),    # K split over blocks: added up, and handed on
+    (700, 4096, 2048, False),      # three row tiles and K split, when the sums are handed on (smaller tiles otherwise)
+    (3000, 12288, 64, False),      # twelve row tiles: a full group of eight and one of four
+    (2048, 16384, 128, True),      # gated, 256 x 256
+    (1100, 12288, 192, True),      # gated, ragged rows
+    (2048, 24576, 4096, True),     # gated, 256 x 192: pairs of groups within a wave's six
+]
+
+
+@pytest.mark.parametrize("M,N,K,glu", FOUR_WAVE_CASES)
+def test_linear_on_four_wave_tiles(M, N, K, glu):
+    """The four-wave kernel (tiles of 256 rows, K in units of 64, A fetched as whole cache lines and
+    read back through a swizzle): every tile width, gated or not, ragged edges, more than eight row
+    tiles, a row stride beyond K, K split over blocks with the sums added or handed on."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(N + K)
+    wide = torch.randn(M, K + 72, generator=g).to(torch.bfloat16).to(DEV)
+    x = wide[:, :K].contiguous()
+    if glu:
+        I = N // 2
+        gate = (torch.randn(I, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+        up = (torch.randn(I, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+        assert _gemm_plan(M, 2 * I, K, 1)[0] == 256
+        a, b = ops.linear(x.float(), gate.float()), ops.linear(x.float(), up.float())
+        ref = a / (1 + torch.exp(-a)) * b
+        pw = ops.pack_gate_up(gate, up)
+        _close(ops.linear(x, pw, out_dtype=torch.float32), ref, 3e-5, "gated product")
+        _close(ops.linear(wide[:, :K], pw), ref, 8e-3, "gated product, strided rows, bfloat16 result")
+        return
+    w = (torch.randn(N, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+    pw = ops.pack_weight(w)
+    ref = ops.linear(x.float(), w.float())
+    seen = set()
+    for keep in (0, 1):
+        r, c, sp = _gemm_plan(M, N, K, 0, keep)
+        assert r == 256 or (M, keep) == (700, 0), (r, c, sp)
+        seen.add(sp)
+        y = ops.linear(x, pw, out_dtype=torch.float32, partials=bool(keep))
+        if keep and sp > 1:
+            assert y.dim() == 3 and y.shape[0] == sp
+        _close(ops.as_tensor(y), ref, 3e-5, f"product (keep={keep}, {c} columns, {sp} parts)")
+    if K >= 2048 and M <= 1024:
+        assert max(seen) > 1, "a case meant to split K"
+    _close(ops.linear(wide[:, :K], pw), ref, 8e-3, "strided rows, bfloat16 result")
+
+
+def test_four_wave_cases_cover_every_tile_width():
+    widths = {(_gemm_plan(M, N, K, int(glu))[1], glu) for M, N, K, glu in FOUR_WAVE_CASES}
+    assert {(128, False), (192, False), (256, False), (192, True), (256, True)} <= widths, widths
 
 
 @pytest.mark.parametrize("M,N,K", [(2600, 6144, 264), (4500, 520, 200), (1100, 300, 96), (9000, 130, 64),
@@ -266,11 +327,13 @@ def test_gemm_plan():
     assert plan(8, 4096, 12288, keep=1) == (0, 0, 1)
     assert plan(64, 4096, 12288) == (64, 128, 8)
     assert plan(64, 151936, 4096) == (64, 128, 1)
-    assert plan(2048, 24576, 4096, 1) == (256, 256, 1)
+    assert plan(2048, 24576, 4096, 1)[0] == 256 and plan(2048, 24576, 4096, 1)[2] == 1
+    assert plan(2048, 24584, 4104, 1) == (256, 256, 1)  # K no multiple of 64: the sixteen-wave tiles, gated on 256 columns only
     assert plan(4096, 4096, 4096) == (256, 256, 1)
     assert plan(2048, 6144, 4096) == (256, 192, 1)     # 8 x 32 tiles are one block a CU; 8 x 24 leave a quarter idle
+    assert plan(2048, 4096, 4096) == (256, 128, 1)     # 8 x 32 again, where 192 columns would leave a third of the CUs idle
     r, c, s = plan(1024, 4096, 12288)
-    assert r >= 128 and c >= 192 and s >= 2           # few tiles, long K: split
+    assert r >= 128 and s >= 2                        # few tiles, long K: split
     r, c, s = plan(256, 4096, 4096)
     assert r <= 128 and s >= 2
     for M, N, K in ((100, 203, 2048), (520, 264, 1544), (300, 1000, 64), (2000, 64, 8)):

@@ -324,6 +324,282 @@ static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int
     return 0;
 }
 
+// ------------------------------------------- four waves, whole cache lines ---
+// Block tile 256 x (32 WTN) on 2 x 2 waves, one to a SIMD, each wave 8 x WTN MFMA tiles: half the
+// LDS reads per MFMA of sixteen waves of 64 x 64.  With one wave to a SIMD nothing overlaps unless
+// the wave interleaves it itself: the fragments of k-tile t + 1 are read from LDS into a second set
+// of registers, and the copies of later tiles are issued, between the MFMAs of k-tile t.
+//
+// What bounds this product is the number of requests to L2, not their bytes: a row-major A read 32 k
+// at a time is 64 bytes a row, half a cache line a request.  So A is copied 64 k at a time, eight
+// rows x 128 bytes a copy (a unit of two k-tiles, NA = 3 of them in LDS), W 32 k at a time as it is
+// packed (NWS k-tiles in LDS).  Within a copy's 1 KB lane i lands at byte 16 i; it fetches row
+// i / 8, 16-byte chunk (i % 8) ^ (i / 8), so that the sixteen rows an MFMA operand is made of are
+// read back from different banks.
+// In k-tile t (32 k) a wave issues, if t is even, its copies of A unit t / 2 + 2, and its copies of W
+// tile t + NWS - 1; at the start of t it needs W tile t + 1 and the A unit of t + 1, issued in tile
+// t - NWS + 2 at the latest.  Copies complete in the order issued, so the wait is by count.
+// K a multiple of 64; a split of K takes whole units.
+__device__ __forceinline__ void mfma_acc(floatx4& c, const bf16x8& a, const bf16x8& b) {
+    // accumulate in place, in the accumulation registers, as the instruction itself says it: through
+    // the builtin the register allocator moves accumulators between the two files around every MFMA
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void copy16_to_lds_sbase(unsigned long long base, unsigned lane_off, unsigned lds_wave_addr) {
+    // the address is a uniform base and a 32-bit offset per lane: walking k is scalar work
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_wave_addr), "v"(lane_off), "s"(base)
+                 : "memory", "m0");
+}
+
+template <int WTN, int NWS, bool GLU, typename TC>
+__global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
+    int K, int lda, int KB, int n_out, float* __restrict__ part) {
+    constexpr int NW = 4, WTM = 8, NA = 3;
+    constexpr int BM = 2 * WTM * 16, BN = 2 * WTN * 16;
+    constexpr int WF = BN / 16;                       // W fragments a k-tile, 1 KB each
+    constexpr int ACP = BM / 8;                       // A copies a unit, 1 KB each
+    constexpr int LPA = ACP / NW, LPW = (WF + NW - 1) / NW;
+    constexpr int NMF = WTM * WTN;                    // MFMAs a k-tile
+    constexpr int RPM = NMF / (WTM + WTN);            // a read after every RPM MFMAs
+    constexpr int CPM = NMF / (LPA + LPW);            // a copy after every CPM MFMAs
+    constexpr int D = NWS - 1;                        // W is copied D tiles ahead
+    static_assert(D == 3 || D == 4, "the waits below are written for three or four tiles ahead");
+    static_assert(RPM >= 1 && CPM >= 1, "not enough MFMAs to hide the reads and copies");
+    constexpr unsigned A_UNIT = ACP * 1024u, W_TILE = WF * 1024u, W_BASE = NA * A_UNIT;
+    static_assert(W_BASE + NWS * W_TILE <= 160 * 1024, "LDS");
+    __shared__ __attribute__((aligned(1024))) char smem[W_BASE + NWS * W_TILE];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int fr = lane & 15, fg = lane >> 4;
+    const int TM = (M + BM - 1) / BM, TN = (N + BN - 1) / BN;
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int full = (TM >> 3) * TN;
+    int grp, grp_rows, j;
+    if (seq < full) {
+        grp = seq / TN;
+        grp_rows = 8;
+        j = xcd * TN + (seq - grp * TN);
+    } else {
+        grp = TM >> 3;
+        grp_rows = TM & 7;
+        const int per = (grp_rows * TN + 7) >> 3;
+        j = xcd * per + (seq - full);
+        if (seq - full >= per || j >= grp_rows * TN) return;
+    }
+    const int tn = j / grp_rows, tm = grp * 8 + j % grp_rows;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int NB = (N + 15) / 16;
+    const int nu = KB / 2;                            // units of 64 k
+    const int u_per = (nu + (int)gridDim.z - 1) / (int)gridDim.z;
+    const int u0 = (int)blockIdx.z * u_per;
+    const int u1 = min(nu, u0 + u_per);
+    const int kt0 = 2 * u0, kt1 = 2 * u1;
+
+    floatx4 acc[WTN][WTM];
+#pragma unroll
+    for (int i = 0; i < WTN; ++i)
+#pragma unroll
+        for (int jj = 0; jj < WTM; ++jj) acc[i][jj] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // this wave's copies: of an A unit the copies wave + 4 c, of a W tile the fragments wave + 4 c
+    unsigned long long abase[LPA], wbase[LPW];
+    unsigned aoff[LPA];
+    unsigned wlds[LPW];
+    const unsigned woff = lane * 16;
+#pragma unroll
+    for (int c = 0; c < LPA; ++c) {
+        const int cp = wave + NW * c;
+        const int row0 = min(m0 + cp * 8, M - 1);
+        const int row = min(m0 + cp * 8 + (lane >> 3), M - 1);
+        abase[c] = (unsigned long long)(A + (size_t)row0 * lda + (size_t)kt0 * 32);
+        aoff[c] = (unsigned)(row - row0) * (unsigned)lda * 2u + (unsigned)(((lane & 7) ^ (lane >> 3)) * 16);
+    }
+#pragma unroll
+    for (int c = 0; c < LPW; ++c) {
+        const int f = min(wave + NW * c, WF - 1);     // the last waves copy the last fragment once more
+        const int nb = min(n0 / 16 + f, NB - 1);
+        wbase[c] = (unsigned long long)(Wp + ((size_t)nb * KB + kt0) * 512);
+        wlds[c] = W_BASE + (unsigned)f * 1024u;
+    }
+    const unsigned smem_addr = (unsigned)(size_t)(lds_ptr_t)smem;
+    // copies past the end repeat the last unit or tile, so that the counts in flight stay the same
+    int a_next = u0, w_next = kt0;                    // the next unit and tile to copy
+    unsigned a_ws = 0, w_ws = 0;                      // where they go: byte offsets of the slots
+#define W4_COPY_A(c)                                                                                \
+    {                                                                                               \
+        copy16_to_lds_sbase(abase[c], aoff[c], smem_addr + a_ws + (unsigned)(wave + NW * (c)) * 1024u); \
+        abase[c] += a_next + 1 < u1 ? 128ull : 0ull;                                                \
+    }
+#define W4_A_ISSUED()                                                                               \
+    {                                                                                               \
+        a_next += a_next + 1 < u1 ? 1 : 0;                                                          \
+        a_ws = a_ws + A_UNIT == NA * A_UNIT ? 0u : a_ws + A_UNIT;                                   \
+    }
+#define W4_COPY_W(c)                                                                                \
+    {                                                                                               \
+        copy16_to_lds_sbase(wbase[c], woff, smem_addr + w_ws + wlds[c]);                            \
+        wbase[c] += w_next + 1 < kt1 ? 1024ull : 0ull;                                              \
+    }
+#define W4_W_ISSUED()                                                                               \
+    {                                                                                               \
+        w_next += w_next + 1 < kt1 ? 1 : 0;                                                         \
+        w_ws = w_ws + W_TILE == NWS * W_TILE ? 0u : w_ws + W_TILE;                                  \
+    }
+    if (u0 < u1) {   // (a part of a split K that holds no unit only stores its zeros)
+        // the tiles before the first, in the order of the loop: t = -4 .. -1
+#pragma unroll
+        for (int t = -4; t < 0; ++t) {
+            if ((t & 1) == 0) {
+#pragma unroll
+                for (int c = 0; c < LPA; ++c) W4_COPY_A(c)
+                W4_A_ISSUED()
+            }
+            if (t + D >= 0) {
+#pragma unroll
+                for (int c = 0; c < LPW; ++c) W4_COPY_W(c)
+                W4_W_ISSUED()
+            }
+        }
+        // what may still be in flight at the start of tile t: the copies of tiles t - D + 2 .. t - 1
+        constexpr int EVEN = LPA + LPW, ODD = LPW;
+        constexpr int FLY_E = D == 4 ? EVEN + ODD : ODD;  // t even: t - 1 is odd
+        constexpr int FLY_O = D == 4 ? EVEN + ODD : EVEN;
+        // a lane's 16 bytes of an A operand: row fr of 16, chunk h * 4 + fg of the row's 8
+        unsigned a_rd[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            a_rd[h] = (unsigned)(wm * WTM * 2 + (fr >> 3)) * 1024u + (unsigned)(((fr & 7) * 8 + ((h * 4 + fg) ^ (fr & 7))) * 16);
+        const unsigned w_rd = W_BASE + (unsigned)(wn * WTN) * 1024u + lane * 16;
+        unsigned a_rs = 0, w_rs = W_TILE;                 // slots of the tile whose fragments are read next (kt0 + 1)
+        // before the first tile: A unit u0 and W tile kt0, issued in tile -4 and tile -D
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(D == 4 ? LPA + 3 * LPW : LPA + 2 * LPW));
+        __syncthreads();
+        bf16x8 fw[2][WTN], fa[2][WTM];
+#pragma unroll
+        for (int i = 0; i < WTN; ++i) fw[0][i] = *reinterpret_cast<const bf16x8*>(smem + w_rd + i * 1024);
+#pragma unroll
+        for (int jj = 0; jj < WTM; ++jj) fa[0][jj] = *reinterpret_cast<const bf16x8*>(smem + a_rd[0] + jj * 2048);
+
+        // a k-tile's MFMAs with the LDS reads of the next tile and the copies of later ones between them
+#define W4_TILE(h)                                                                                  \
+        {                                                                                           \
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((h) ? FLY_O : FLY_E));                             \
+            asm volatile("s_barrier" ::: "memory");                                                 \
+            const char* na = smem + a_rs + a_rd[(h) ^ 1];                                           \
+            const char* nw = smem + w_rs + w_rd;                                                    \
+            _Pragma("unroll") for (int i = 0; i < WTN; ++i)                                         \
+                _Pragma("unroll") for (int jj = 0; jj < WTM; ++jj) {                                \
+                    const int q = i * WTM + jj;                                                     \
+                    mfma_acc(acc[i][jj], fw[h][i], fa[h][jj]);                                      \
+                    if (q % RPM == RPM - 1 && q / RPM < WTN + WTM) {                                \
+                        const int rd = q / RPM;                                                     \
+                        if (rd < WTM) fa[(h) ^ 1][rd < WTM ? rd : 0] = *reinterpret_cast<const bf16x8*>(na + rd * 2048); \
+                        else fw[(h) ^ 1][rd >= WTM ? rd - WTM : 0] = *reinterpret_cast<const bf16x8*>(nw + (rd - WTM) * 1024); \
+                    }                                                                               \
+                    if (q % CPM == CPM - 1) {                                                       \
+                        const int cp = q / CPM;                                                     \
+                        if ((h) == 0) {                                                             \
+                            if (cp < LPA) W4_COPY_A(cp < LPA ? cp : 0)                              \
+                            else if (cp < LPA + LPW) W4_COPY_W(cp >= LPA && cp < LPA + LPW ? cp - LPA : 0) \
+                        } else if (cp < LPW) W4_COPY_W(cp < LPW ? cp : 0)                           \
+                    }                                                                               \
+                }                                                                                   \
+            if ((h) == 0) W4_A_ISSUED()                                                             \
+            W4_W_ISSUED()                                                                           \
+            if ((h) == 0) a_rs = a_rs + A_UNIT == NA * A_UNIT ? 0u : a_rs + A_UNIT;                 \
+            w_rs = w_rs + W_TILE == NWS * W_TILE ? 0u : w_rs + W_TILE;                              \
+        }
+        // tile 2 u reads its successor from its own unit, tile 2 u + 1 from the next: a_rs moves on after an even tile
+        for (int kt = kt0; kt < kt1; kt += 2) {
+            W4_TILE(0)
+            W4_TILE(1)
+        }
+    }
+#undef W4_TILE
+#undef W4_COPY_A
+#undef W4_COPY_W
+#undef W4_A_ISSUED
+#undef W4_W_ISSUED
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written their accumulators
+
+    if (part) {
+        float* P = part + (size_t)blockIdx.z * M * N;
+        const bool vec = (N % 4) == 0;
+#pragma unroll
+        for (int i = 0; i < WTN; ++i) {
+            const int n = n0 + (wn * WTN + i) * 16 + fg * 4;
+#pragma unroll
+            for (int jj = 0; jj < WTM; ++jj) {
+                const int m = m0 + (wm * WTM + jj) * 16 + fr;
+                if (m < M && n < N) store4<float>(P + (size_t)m * N + n, acc[i][jj], n, N, vec);
+            }
+        }
+        return;
+    }
+    if constexpr (GLU) {
+        static_assert(WTN % 2 == 0, "gate and up groups come in pairs");
+        const bool vec = (n_out % 4) == 0;
+#pragma unroll
+        for (int i = 0; i < WTN; i += 2) {
+            const int n = (n0 + (wn * WTN + i) * 16) / 2 + fg * 4;
+#pragma unroll
+            for (int jj = 0; jj < WTM; ++jj) {
+                const int m = m0 + (wm * WTM + jj) * 16 + fr;
+                if (m < M && n < n_out)
+                    store4<TC>(C + (size_t)m * n_out + n, silu_mul(acc[i][jj], acc[i + 1][jj]), n, n_out, vec);
+            }
+        }
+    } else {
+        const bool vec = (N % 4) == 0;
+#pragma unroll
+        for (int i = 0; i < WTN; ++i) {
+            const int n = n0 + (wn * WTN + i) * 16 + fg * 4;
+#pragma unroll
+            for (int jj = 0; jj < WTM; ++jj) {
+                const int m = m0 + (wm * WTM + jj) * 16 + fr;
+                if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, acc[i][jj], n, N, vec);
+            }
+        }
+    }
+}
+
+// splits > 1: the blocks of a tile split K among them in units of 64; part holds splits * M * N floats
+template <int WTN, int NWS, bool GLU = false>
+static int launch_w4(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda, int c_dtype,
+                     int n_out, hipStream_t s, int splits = 1, float* part = nullptr, bool reduce = true) {
+    TFF_REQUIRE(K % 64 == 0, "gemm: the four-wave tiles take K in units of 64, not K=%d", K);
+    const int KB = K / 32;
+    constexpr int BM = 256, BN = 2 * WTN * 16;
+    if (splits <= 1 || !part) { splits = 1; part = nullptr; }
+    TFF_REQUIRE(splits <= KB / 2, "gemm: %d parts of %d units of K", splits, KB / 2);
+    const long TM = (M + BM - 1) / BM, TN = (N + BN - 1) / BN;
+    const long tiles = 8 * ((TM / 8) * TN + ((TM % 8) * TN + 7) / 8);   // eight equal shares, see the kernel
+    TFF_REQUIRE(tiles < (1L << 31), "gemm: too many tiles for M=%d N=%d", M, N);
+    TFF_REQUIRE((size_t)15 * lda * 2 + 128 < (1ull << 32), "gemm: row stride %d too large", lda);
+    const dim3 grid((unsigned)tiles, 1, splits);
+    if (c_dtype == TFF_F32)
+        gemm_bf16_w4_kernel<WTN, NWS, GLU, float><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out, part);
+    else
+        gemm_bf16_w4_kernel<WTN, NWS, GLU, bf16_t><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out, part);
+    if (int rc = tff_check_launch("gemm_bf16_w4")) return rc;
+    if (splits > 1 && reduce) {
+        const int No = GLU ? n_out : N;
+        const long threads = (long)M * ((No + 3) / 4);
+        const int blocks = (int)((threads + 255) / 256);
+        if (c_dtype == TFF_F32)
+            gemm_splitk_reduce_kernel<GLU, float><<<blocks, 256, 0, s>>>(part, splits, M, N, (float*)C, No);
+        else
+            gemm_splitk_reduce_kernel<GLU, bf16_t><<<blocks, 256, 0, s>>>(part, splits, M, N, (bf16_t*)C, No);
+        return tff_check_launch("gemm_splitk_reduce");
+    }
+    return 0;
+}
+
 // ------------------------------------------------------------- skinny M ---
 // For a few rows of A (decoding: M = number of live requests) the product is
 // a stream of W from HBM; what counts is bytes in flight, not LDS tiling.
@@ -616,13 +892,13 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
 
 // The tiled product's plan for M > 16: which tile, and into how many parts the blocks of a
 // tile split K.  Up to 64 rows: 64 x 128 tiles (two blocks to a CU), K split so that the most
-// loaded CU has the least to stream.  Beyond: the cheapest of 256 x 256, 256 x 192, 128 x 256,
-// 128 x 128 and 64 x 128 tiles with 1 .. 8 parts by a small cost model: rounds of blocks over
+// loaded CU has the least to stream.  Beyond: the cheapest of 256 x 256, 256 x 192, 256 x 128 (on
+// four waves, K in units of 64), 128 x 256, 128 x 128 and 64 x 128 tiles with 1 .. 8 parts by a small cost model: rounds of blocks over
 // the CUs times a block's work at the tile's measured rate (large tiles read fewer bytes of
 // LDS per flop), plus the traffic of the partial sums (less where the caller takes them as
 // they are).  Its constants were fitted to measurements of the four products of the 8B, 14B
-// and 32B shapes at 96 .. 4,096 rows on an MI355X (156 cases, every tile with 1 .. 8 parts),
-// where its pick is within 7 % of the best candidate everywhere and 0.3 % from it on average.
+// and 32B shapes at 96 .. 4,096 rows on an MI355X (144 cases, every tile with 1 .. 8 parts),
+// where its pick is within 11 % of the best candidate everywhere and 0.7 % from it on average.
 struct GemmPlan { int tile; int bn; int splits; };   // tile = rows of a block tile
 // Compute units of the current device (256 on an MI355X, which the rates below were fitted on; a
 // device with another count gets plans for its own number of blocks a round).  256 if it cannot
@@ -669,15 +945,22 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
         }
         return {64, 128, best_s};
     }
-    // rate: flops a microsecond that a CU sustains on blocks of this tile; slots: blocks a CU holds
+    // rate: flops a microsecond that a CU sustains on blocks of this tile; slots: blocks a CU holds.
+    // With K in units of 64 the tiles of 256 rows are those of the four-wave kernel (256, 192 or 128
+    // columns, gated or not); otherwise those of the sixteen-wave kernel.
     struct Cand { int bm, bn, slots; double rate; };
-    static const Cand cands[5] = {{256, 256, 1, 5.2e6}, {256, 192, 1, 4.4e6}, {128, 256, 1, 3.6e6},
-                                  {128, 128, 1, 2.6e6}, {64, 128, 2, 2.2e6}};
+    static const Cand cands_w4[6] = {{256, 256, 1, 5.6e6}, {256, 192, 1, 5.7e6}, {256, 128, 1, 5.0e6},
+                                     {128, 256, 1, 3.3e6}, {128, 128, 1, 2.8e6}, {64, 128, 2, 2.4e6}};
+    static const Cand cands_w16[6] = {{256, 256, 1, 5.2e6}, {256, 192, 1, 4.4e6}, {128, 256, 1, 3.6e6},
+                                      {128, 128, 1, 2.6e6}, {64, 128, 2, 2.2e6}, {0, 0, 0, 0.0}};
+    const bool w4 = K % 64 == 0;
     GemmPlan best = {256, 256, 1};
     double best_t = 1e30;
-    for (const Cand& c : cands)
+    for (const Cand& c : (w4 ? cands_w4 : cands_w16)) {
+        if (c.bm == 0) break;
         for (int S = 1; S <= (glu ? 2 : 8); S *= 2) {
-            if (glu && c.bn == 192) break;   // gate and up groups come in pairs: an even number a wave
+            // gate and up groups come in pairs, an even number a wave: three a wave of the sixteen do not do
+            if (glu && c.bn == 192 && !w4) break;
             if (S > 1 && nk / S < 8) break;
             const double blocks = (double)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * S;
             const double rounds = ceil(blocks / (CUS * c.slots));
@@ -687,9 +970,10 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
             double t = round_us * rounds + 3.0;
             // the partial sums: written, read and added by a second kernel, or (kept) read by the
             // consumer in place of one plane
-            if (S > 1) t += keep ? (S - 1.0) * M * N * 4.0 / 4e6 : (double)S * M * N * 4.0 / 3e6 + 3.0;
+            if (S > 1) t += keep ? (S - 1.0) * M * N * 4.0 / 4e6 : (double)S * M * N * 4.0 / (w4 ? 2.7e6 : 3e6) + 3.0;
             if (t < best_t) { best_t = t; best = {c.bm, c.bn, S}; }
         }
+    }
     return best;
 }
 
@@ -761,6 +1045,11 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
             return launch_async_g<2, 2, 4, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         if (plan.tile == 128)
             return launch_async_g<2, 4, 4, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+        if (K % 64 == 0) {
+            if (plan.bn == 128) return launch_w4<4, 5, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+            if (plan.bn == 192) return launch_w4<6, 5, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+            return launch_w4<8, 4, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+        }
         return launch_async_g<4, 4, 4, 4, 5, true, 1, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
     }
     if (plan.tile == 0) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, nullptr);
@@ -777,6 +1066,11 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
         return launch_async_g<2, 2, 4, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     if (plan.tile == 128)
         return launch_async_g<2, 4, 4, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+    if (K % 64 == 0) {
+        if (plan.bn == 128) return launch_w4<4, 5>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+        if (plan.bn == 192) return launch_w4<6, 5>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+        return launch_w4<8, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+    }
     if (plan.bn == 192)
         return launch_async_g<4, 4, 4, 3, 5, false, 1, true>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     return launch_async_g<4, 4, 4, 4, 5, false, 1, true>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
