@@ -353,10 +353,91 @@ __device__ __forceinline__ void copy16_to_lds_sbase(unsigned long long base, uns
                  : "memory", "m0");
 }
 
+// The lane's index, taken where it is asked for: what the epilogue works out from it is then worked out
+// after the main loop, where there are registers for it, instead of before it and kept (or spilled) across.
+__device__ __forceinline__ int w4_lane() {
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    return lane;
+}
+
+// A wave's 128 rows x OW column groups of results go out through LDS, so that a store instruction
+// writes whole rows instead of 16 rows x 8 or 16 bytes: a lane leaves its four columns of a row in
+// the wave's own region of LDS (rows padded by 16 bytes against bank conflicts) and takes 16 bytes
+// of a row back.  Only this wave touches the region, LDS works through a wave's accesses in order,
+// so no barrier is needed within; RC of the 8 row groups go through at a time, as many as the
+// region holds.  A store instruction takes 64 / LPR rows, LPR lanes to a row (the power of two that
+// holds a row's 16-byte pieces; the lanes beyond them idle), so that the address of a lane's store
+// is that of its last one plus a constant.  vec: the rows of the result are a multiple of 16 bytes
+// long, the 16 bytes are one store; otherwise they go out element by element (slow, and rare: a
+// width that is no multiple of 8).  This is the kernel's only way out for its results on purpose:
+// with a second one beside it the compiler converts accumulators for both before the branch, runs
+// out of registers and spills, and a kernel that uses scratch memory pays some 15 us at its launch.
+template <int OW, int REGION, typename TO, typename F>
+__device__ __forceinline__ void w4_store_rows(char* region, F val, TO* out, size_t ld, int m_base, int n_base,
+                                              int M, int ncols, int lane, bool vec) {
+    constexpr int E = 16 / (int)sizeof(TO);           // columns in 16 bytes
+    constexpr int RB = OW * 16 * (int)sizeof(TO), RBP = RB + 16, CPR = RB / 16;
+    constexpr int LPR = CPR <= 4 ? 4 : CPR <= 8 ? 8 : CPR <= 16 ? 16 : 32;   // lanes a row
+    static_assert(CPR <= LPR, "a row's pieces fit its lanes");
+    constexpr int RPI = 64 / LPR;                     // rows a store instruction
+    constexpr int RC = 8 * 16 * RBP <= REGION ? 8 : 4;
+    static_assert(RC * 16 * RBP <= REGION, "the wave's region of LDS holds four row groups at least");
+    const int fr = lane & 15, fg = lane >> 4;
+    const int srow = lane / LPR, sch = lane % LPR;    // this lane's row of an instruction's, and its piece
+    const int n = n_base + sch * E;
+    const bool mine = sch < CPR && n < ncols;
+    const char* src = region + srow * RBP + sch * 16;
+#pragma unroll
+    for (int p = 0; p < 8 / RC; ++p) {
+#pragma unroll
+        for (int jj = 0; jj < RC; ++jj) {
+            __builtin_amdgcn_sched_barrier(0);   // a row group at a time: all accumulators converted at once do not fit the registers
+#pragma unroll
+            for (int i = 0; i < OW; ++i) {
+                const floatx4 v = val(i, p * RC + jj);
+                char* dst = region + (jj * 16 + fr) * RBP + (i * 16 + fg * 4) * (int)sizeof(TO);
+                if constexpr (sizeof(TO) == 4) {
+                    *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+                    union { bf16_t h[4]; uint2 u; } pk;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) pk.h[e] = (bf16_t)v[e];
+                    *reinterpret_cast<uint2*>(dst) = pk.u;
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        int m = m_base + p * RC * 16 + srow;
+        TO* dst = out + (size_t)m * ld + n;
+        if (vec) {   // (the branch outside the loop: its reads of LDS are then issued together, not one per store)
+#pragma unroll
+            for (int t = 0; t < RC * 16 / RPI; ++t) {
+                const uint4 v = *reinterpret_cast<const uint4*>(src + t * RPI * RBP);
+                if (mine && m < M) *reinterpret_cast<uint4*>(dst) = v;
+                m += RPI;
+                dst += (size_t)RPI * ld;
+            }
+        } else {
+            for (int t = 0; t < RC * 16 / RPI; ++t) {
+                union { uint4 u; TO e[E]; } v;
+                v.u = *reinterpret_cast<const uint4*>(src + t * RPI * RBP);
+                if (mine && m < M) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e)
+                        if (n + e < ncols) dst[e] = v.e[e];
+                }
+                m += RPI;
+                dst += (size_t)RPI * ld;
+            }
+        }
+    }
+}
+
 template <int WTN, int NWS, bool GLU, typename TC>
 __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
-    int K, int lda, int KB, int n_out, float* __restrict__ part) {
+    int K, int lda, int KB, int n_out) {
     constexpr int NW = 4, WTM = 8, NA = 3;
     constexpr int BM = 2 * WTM * 16, BN = 2 * WTN * 16;
     constexpr int WF = BN / 16;                       // W fragments a k-tile, 1 KB each
@@ -524,47 +605,25 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(
 #undef W4_COPY_W
 #undef W4_A_ISSUED
 #undef W4_W_ISSUED
+    // every copy has landed and every read of LDS has come back, in every wave: LDS is free for the results
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written their accumulators
-
-    if (part) {
-        float* P = part + (size_t)blockIdx.z * M * N;
-        const bool vec = (N % 4) == 0;
-#pragma unroll
-        for (int i = 0; i < WTN; ++i) {
-            const int n = n0 + (wn * WTN + i) * 16 + fg * 4;
-#pragma unroll
-            for (int jj = 0; jj < WTM; ++jj) {
-                const int m = m0 + (wm * WTM + jj) * 16 + fr;
-                if (m < M && n < N) store4<float>(P + (size_t)m * N + n, acc[i][jj], n, N, vec);
-            }
-        }
-        return;
-    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");   // (and the last MFMAs have written their accumulators)
+    __syncthreads();
+    constexpr int REGION = (int)((W_BASE + NWS * W_TILE) / 4) & ~1023;
+    char* region = smem + wave * REGION;
+    const int mw = m0 + wm * WTM * 16;                // the wave's first row
+    constexpr int E = 16 / (int)sizeof(TC);
+    const int lane_out = w4_lane();
     if constexpr (GLU) {
         static_assert(WTN % 2 == 0, "gate and up groups come in pairs");
-        const bool vec = (n_out % 4) == 0;
-#pragma unroll
-        for (int i = 0; i < WTN; i += 2) {
-            const int n = (n0 + (wn * WTN + i) * 16) / 2 + fg * 4;
-#pragma unroll
-            for (int jj = 0; jj < WTM; ++jj) {
-                const int m = m0 + (wm * WTM + jj) * 16 + fr;
-                if (m < M && n < n_out)
-                    store4<TC>(C + (size_t)m * n_out + n, silu_mul(acc[i][jj], acc[i + 1][jj]), n, n_out, vec);
-            }
-        }
+        w4_store_rows<WTN / 2, REGION, TC>(region, [&](int i, int jj) { return silu_mul(acc[2 * i][jj], acc[2 * i + 1][jj]); },
+                                           C, (size_t)n_out, mw, (n0 + wn * WTN * 16) / 2, M, n_out, lane_out,
+                                           n_out % E == 0);
     } else {
-        const bool vec = (N % 4) == 0;
-#pragma unroll
-        for (int i = 0; i < WTN; ++i) {
-            const int n = n0 + (wn * WTN + i) * 16 + fg * 4;
-#pragma unroll
-            for (int jj = 0; jj < WTM; ++jj) {
-                const int m = m0 + (wm * WTM + jj) * 16 + fr;
-                if (m < M && n < N) store4<TC>(C + (size_t)m * N + n, acc[i][jj], n, N, vec);
-            }
-        }
+        // (partial sums of a split K: plane blockIdx.z of the launcher's float32 workspace, which it passes as C)
+        TC* out = C + (size_t)blockIdx.z * M * N;
+        w4_store_rows<WTN, REGION, TC>(region, [&](int i, int jj) { return acc[i][jj]; }, out, (size_t)N, mw,
+                                       n0 + wn * WTN * 16, M, N, lane_out, N % E == 0);
     }
 }
 
@@ -582,10 +641,13 @@ static int launch_w4(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, i
     TFF_REQUIRE(tiles < (1L << 31), "gemm: too many tiles for M=%d N=%d", M, N);
     TFF_REQUIRE((size_t)15 * lda * 2 + 128 < (1ull << 32), "gemm: row stride %d too large", lda);
     const dim3 grid((unsigned)tiles, 1, splits);
-    if (c_dtype == TFF_F32)
-        gemm_bf16_w4_kernel<WTN, NWS, GLU, float><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out, part);
+    // the blocks of a split K leave plain float32 sums, plane by plane; a gate is applied when they are added up
+    if (splits > 1)
+        gemm_bf16_w4_kernel<WTN, NWS, false, float><<<grid, 256, 0, s>>>(A, Wp, part, M, N, K, lda, KB, 0);
+    else if (c_dtype == TFF_F32)
+        gemm_bf16_w4_kernel<WTN, NWS, GLU, float><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
     else
-        gemm_bf16_w4_kernel<WTN, NWS, GLU, bf16_t><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out, part);
+        gemm_bf16_w4_kernel<WTN, NWS, GLU, bf16_t><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
     if (int rc = tff_check_launch("gemm_bf16_w4")) return rc;
     if (splits > 1 && reduce) {
         const int No = GLU ? n_out : N;
@@ -1003,7 +1065,8 @@ static int skinny_for(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, 
         if constexpr (EPI != 2) {
             if (N >= 16 * 1024)
                 return launch_skinny<1, 1, 8, 1, 2, true, true, EPI>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, fuse);
-            return launch_skinny<1, 1, 32, 4, 2, true, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, fuse);
+            // (with the norm's factor taken in, 32 k-steps in flight do not fit the registers: 24)
+            return launch_skinny<1, 1, (EPI == 1 ? 24 : 32), 4, 2, true, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, fuse);
         } else {
             return tff_fail("gemm: a gated product does not come before a norm");
         }
