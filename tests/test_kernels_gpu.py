@@ -249,7 +249,7 @@ FOUR_WAVE_CASES = [
     (2048, 16384, 128, True),      # gated, 256 x 256
     (1100, 12288, 192, True),      # gated, ragged rows
     (1100, 12280, 192, True),      # gated, a result whose rows are no multiple of 16 bytes: element by element
-    (2048, 24576, 4096, True),     # gated, 256 x 192: pairs of groups within a wave's six
+    (2048, 12288, 1024, True),     # gated, 256 x 192: pairs of groups within a wave's six
 ]
 
 

@@ -960,7 +960,7 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
 // LDS per flop), plus the traffic of the partial sums (less where the caller takes them as
 // they are).  Its constants were fitted to measurements of the four products of the 8B, 14B
 // and 32B shapes at 96 .. 4,096 rows on an MI355X (144 cases, every tile with 1 .. 8 parts),
-// where its pick is within 11 % of the best candidate everywhere and 0.7 % from it on average.
+// where its pick is within 9 % of the best candidate everywhere and 0.7 % from it on average.
 struct GemmPlan { int tile; int bn; int splits; };   // tile = rows of a block tile
 // Compute units of the current device (256 on an MI355X, which the rates below were fitted on; a
 // device with another count gets plans for its own number of blocks a round).  256 if it cannot
@@ -1011,8 +1011,8 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
     // With K in units of 64 the tiles of 256 rows are those of the four-wave kernel (256, 192 or 128
     // columns, gated or not); otherwise those of the sixteen-wave kernel.
     struct Cand { int bm, bn, slots; double rate; };
-    static const Cand cands_w4[6] = {{256, 256, 1, 5.6e6}, {256, 192, 1, 5.7e6}, {256, 128, 1, 5.0e6},
-                                     {128, 256, 1, 3.3e6}, {128, 128, 1, 2.8e6}, {64, 128, 2, 2.4e6}};
+    static const Cand cands_w4[6] = {{256, 256, 1, 5.7e6}, {256, 192, 1, 5.4e6}, {256, 128, 1, 5.1e6},
+                                     {128, 256, 1, 3.25e6}, {128, 128, 1, 2.7e6}, {64, 128, 2, 2.4e6}};
     static const Cand cands_w16[6] = {{256, 256, 1, 5.2e6}, {256, 192, 1, 4.4e6}, {128, 256, 1, 3.6e6},
                                       {128, 128, 1, 2.6e6}, {64, 128, 2, 2.2e6}, {0, 0, 0, 0.0}};
     const bool w4 = K % 64 == 0;
@@ -1032,7 +1032,7 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
             double t = round_us * rounds + 3.0;
             // the partial sums: written, read and added by a second kernel, or (kept) read by the
             // consumer in place of one plane
-            if (S > 1) t += keep ? (S - 1.0) * M * N * 4.0 / 4e6 : (double)S * M * N * 4.0 / (w4 ? 2.7e6 : 3e6) + 3.0;
+            if (S > 1) t += keep ? (S - 1.0) * M * N * 4.0 / 4e6 : (double)S * M * N * 4.0 / (w4 ? 2.6e6 : 3e6) + 3.0;
             if (t < best_t) { best_t = t; best = {c.bm, c.bn, S}; }
         }
     }
