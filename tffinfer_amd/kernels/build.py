@@ -24,6 +24,8 @@ from .. import log
 PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_NAME = "libtffinfer_hip.so"
+ENGINE_LIB_NAME = "libtffinfer_engine.so"     # the engine's C interface (csrc/tffinfer_engine.h)
+ENGINE_DEMO_NAME = "engine_demo"
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -173,6 +175,46 @@ def build(verbose: bool = True) -> str:
                     name, n)
     say(f"built {LIB_NAME} in {time.time() - t0:.0f} s")
     return os.path.join(out_dir, LIB_NAME)
+
+
+def build_engine_capi(out_dir: str | None = None, verbose: bool = True) -> str:
+    """Compiles the engine's C interface (csrc/engine_capi.c: an embedded interpreter around the
+    package's engine) and the example program that uses it; returns the library's path."""
+    import sysconfig
+    cc = os.environ.get("CC") or shutil.which("gcc") or shutil.which("cc")
+    if not cc:
+        raise BuildError("no C compiler was found for the engine's C interface (looked at $CC, gcc, cc)")
+    out_dir = out_dir or next((d for d in lib_dirs() if _writable(d)), None)
+    if out_dir is None:
+        raise BuildError("no writable folder for the engine library: " + ", ".join(lib_dirs()))
+    inc, libdir = sysconfig.get_config_var("INCLUDEPY"), sysconfig.get_config_var("LIBDIR")
+    pylib = "python" + (sysconfig.get_config_var("LDVERSION") or sysconfig.get_python_version())
+    if not inc or not os.path.exists(os.path.join(inc, "Python.h")):
+        raise BuildError(f"Python.h was not found in {inc}: the engine's C interface embeds the interpreter")
+    lib = os.path.join(out_dir, ENGINE_LIB_NAME)
+    cmd = [cc, "-O2", "-shared", "-fPIC", "-fvisibility=hidden", "-Wall", "-I", CSRC_DIR, "-I", inc,
+           os.path.join(CSRC_DIR, "engine_capi.c"), "-L", libdir, "-l" + pylib, "-ldl", "-o", lib]
+    p = subprocess.run(cmd, capture_output=True, text=True)
+    if p.returncode != 0:
+        raise BuildError(f"{cc} failed on engine_capi.c:\n{p.stderr[-4000:]}")
+    demo_src = os.path.join(os.path.dirname(PKG_DIR), "examples", "engine_demo.c")
+    if os.path.exists(demo_src):
+        cmd = [cc, "-O2", "-Wall", "-I", CSRC_DIR, demo_src, "-L", out_dir, "-ltffinfer_engine",
+               "-Wl,-rpath,$ORIGIN", "-o", os.path.join(out_dir, ENGINE_DEMO_NAME)]
+        p = subprocess.run(cmd, capture_output=True, text=True)
+        if p.returncode != 0:
+            raise BuildError(f"{cc} failed on engine_demo.c:\n{p.stderr[-4000:]}")
+    if verbose:
+        log.info("build: built %s", ENGINE_LIB_NAME)
+    return lib
+
+
+def find_engine_library() -> str | None:
+    for d in lib_dirs():
+        lib = os.path.join(d, ENGINE_LIB_NAME)
+        if os.path.exists(lib):
+            return lib
+    return None
 
 
 def ensure_built(verbose: bool = True) -> str:
