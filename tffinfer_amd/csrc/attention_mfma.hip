@@ -961,9 +961,9 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
         start_pos, work, tiles_per_entry, nq, nkv, page_size, page_shift, window, scale, T_total
     if (fuse) {
         if (splits > 1)
-            attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 2), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
+            attn_wave_kernel<DT, true, (DT <= 8 ? 4 : DT <= 12 ? 2 : 1), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
         else
-            attn_wave_kernel<DT, false, (DT <= 8 ? 4 : 2), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
+            attn_wave_kernel<DT, false, (DT <= 8 ? 4 : DT <= 12 ? 2 : 1), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
     } else if (splits > 1) {
         attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
     } else {
