@@ -769,7 +769,10 @@ def test_attention_mfma_decode_split_keys(nq, nkv, d, ps, window, splits):
 @pytest.mark.parametrize("nq,nkv,d,ps,window,splits,pairing", [
     (32, 8, 128, 16, 0, None, "half"), (32, 8, 128, 16, 0, 1, "interleaved"), (4, 2, 16, 16, 0, 3, "interleaved"),
     (8, 2, 32, 8, 24, 4, "interleaved"), (40, 2, 96, 8, 0, 5, "interleaved"), (6, 3, 48, 8, 100, None, "interleaved"),
-    (16, 1, 64, 32, 0, 64, "half"), (4, 2, 192, 16, 0, 3, "half"), (2, 1, 256, 8, 0, None, "half")])
+    (16, 1, 64, 32, 0, 64, "half"), (4, 2, 192, 16, 0, 3, "half"), (2, 1, 256, 8, 0, None, "half"),
+    # splits 0: a block of eight waves per entry and kv head, merged in LDS
+    (32, 8, 128, 16, 0, 0, "half"), (4, 2, 16, 16, 0, 0, "interleaved"), (8, 2, 32, 8, 24, 0, "interleaved"),
+    (40, 2, 96, 8, 0, 0, "interleaved"), (6, 3, 48, 8, 100, 0, "interleaved"), (16, 1, 112, 32, 0, 0, "interleaved")])
 def test_attention_decode_fused(nq, nkv, d, ps, window, splits, pairing, with_norm, with_rope):
     """Decode steps from the raw projection output: q/k norm, rotation, the token's key and value
     into its page and attention in one kernel, against each part's formula; the slot of the new
@@ -861,8 +864,58 @@ def test_attention_decode_fused(nq, nkv, d, ps, window, splits, pairing, with_no
     kv.k_cache, kv.v_cache = kc0.to(DEV), vc0.to(DEV)
     dq = qkv.to(DEV).clone()
     ops.qk_norm_rope_kv(dq, nq, nkv, d, w[0], w[1], eps, table, pr, batch.positions, slots, kv.k_cache, kv.v_cache)
-    out3 = ops.attention_mfma(dq, nq, nkv, d, kv, batch, window, scale, splits=splits)
+    out3 = ops.attention_mfma(dq, nq, nkv, d, kv, batch, window, scale, splits=splits or None)
     _close(out.reshape(R, nq, d), out3.reshape(R, nq, d).double().cpu(), 1.5e-2, "fused against two kernels")
+
+
+@pytest.mark.parametrize("d,ps,window", [(32, 8, 0), (128, 16, 0), (64, 8, 5000)])
+def test_attention_decode_fused_blocks_of_eight_waves_over_long_contexts(d, ps, window):
+    """A block of eight waves per entry and kv head: runs of keys of very different lengths in one
+    launch (a wave with more pages than it keeps at hand works through them in segments; short
+    entries leave most waves of their block without keys), one key far back made to dominate, the
+    token's own key and value from registers.  What the block picks by itself from the step's sizes
+    is the same kernel."""
+    ops = _ops()
+    nq, nkv = 8, 2
+    far = 77
+    entries = [(20000, 1), (40, 1), (0, 1), (95, 1), (96, 1), (3000, 1), (255, 1), (256, 1)]
+    batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=3 + d)
+    R = len(entries)
+    g = torch.Generator().manual_seed(7)
+    qkv = torch.randn(R, (nq + 2 * nkv) * d, generator=g).to(torch.bfloat16)
+    q = qkv[:, :nq * d].reshape(R, nq, d)
+    k_new = qkv[:, nq * d:(nq + nkv) * d].reshape(R, nkv, d)
+    v_new = qkv[:, (nq + nkv) * d:].reshape(R, nkv, d)
+    if window == 0:
+        kfar = (30 * q[0, 0].float() / q[0, 0].float().norm()).to(torch.bfloat16)
+        kv.k_cache[int(kv.block_tables[0, far // ps]), 0, far % ps] = kfar.to(DEV)
+        ks[0][far, 0] = kfar
+    scale = 1 / math.sqrt(d)
+    bt = kv.block_tables.cpu()
+    slots = torch.tensor([int(bt[r, P // ps]) * ps + P % ps for r, (P, _) in enumerate(entries)], dtype=torch.int32, device=DEV)
+    refs = []
+    for r, (P, _) in enumerate(entries):
+        k = torch.cat([ks[r][:P], k_new[r:r + 1]])
+        v = torch.cat([vs[r][:P], v_new[r:r + 1]])
+        refs.append(_attn_ref(q[r:r + 1], k, v, positions[r:r + 1], window, scale)[0])
+    ref = torch.stack(refs)
+    out = ops.attention_decode_fused(qkv.to(DEV), nq, nkv, d, None, None, 1e-6, None, 0, kv, batch, window, scale,
+                                     slot_mapping=slots, splits=0)
+    _close(out.reshape(R, nq, d), ref, 1.5e-2, "blocks of eight waves")
+    if window == 0:
+        assert torch.allclose(out.reshape(R, nq, d)[0, 0].float().cpu(), vs[0][far, 0].float(), atol=5e-2)
+    # with 256 pairs of entry and kv head and more, that is what a step gets unasked
+    assert ops.BLOCK_DECODE_MIN_PAIRS == 256
+    big = [(100 + 7 * i, 1) for i in range(128)]
+    batch2, kv2, ks2, vs2, pos2, _ = _fake_step(big, ps, nkv, d, torch.bfloat16, seed=11)
+    qkv2 = torch.randn(128, (nq + 2 * nkv) * d, generator=g).to(torch.bfloat16)
+    bt2 = kv2.block_tables.cpu()
+    slots2 = torch.tensor([int(bt2[r, P // ps]) * ps + P % ps for r, (P, _) in enumerate(big)], dtype=torch.int32, device=DEV)
+    a = ops.attention_decode_fused(qkv2.to(DEV), nq, nkv, d, None, None, 1e-6, None, 0, kv2, batch2, window, scale,
+                                   slot_mapping=slots2)
+    b = ops.attention_decode_fused(qkv2.to(DEV), nq, nkv, d, None, None, 1e-6, None, 0, kv2, batch2, window, scale,
+                                   slot_mapping=None, splits=0)
+    assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("nq,nkv,d,ps,window", [(32, 8, 128, 16, 0), (8, 2, 32, 8, 300), (40, 2, 96, 8, 0)])

@@ -143,8 +143,14 @@ __device__ __forceinline__ void norm_rope_fragments(bf16x8 (&f)[(DT * 16 + 31) /
 #pragma unroll
         for (int j = 0; j < 8; ++j) f[ks][j] = (bf16_t)x[ks][j];
 }
-template <int DT, bool SPLIT, int RING, bool FUSED = false>
-__global__ __launch_bounds__(64, 1) void attn_wave_kernel(
+// BW > 1 (entries of one token, FUSED): a block of BW waves per entry and kv head.  The waves
+// split the entry's keys among them (what blockIdx.z does for SPLIT), and their partial results
+// meet in LDS instead of global memory: no second kernel, no partial results written and read.
+// A wave alone streams some 16 GB/s, eight of them on a CU together as much as the CU takes
+// (≈ 100 GB/s), so this pays once there are entries x kv heads enough for the blocks to saturate
+// HBM between them (64 and more); with fewer, the keys are split over blocks as before.
+template <int DT, bool SPLIT, int RING, bool FUSED = false, int BW = 1>
+__global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int bt_stride,
@@ -153,9 +159,24 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
     int page_shift, int window, float scale, int T_total, AttnFuse fz) {
     constexpr int D = DT * 16;
     constexpr int KS = (D + 31) / 32;
-    __shared__ int32_t bt_lds[ATTN_WAVE_BT];
-    __shared__ __attribute__((aligned(16))) float fz_lds[FUSED ? 3 * D : 4];   // q weight, k weight, (cos, sin) pairs
-    const int lane = threadIdx.x, qc = lane & 15, kg = lane >> 4;
+    static_assert(BW == 1 || (FUSED && !SPLIT), "blocks of several waves are for fused decode steps, and merge in LDS");
+    constexpr int BT_LEN = BW == 1 ? ATTN_WAVE_BT : ATTN_WAVE_BT / 4;     // page numbers a wave keeps at a time
+    __shared__ int32_t bt_all[BW * BT_LEN];
+    __shared__ __attribute__((aligned(16))) float fz_all[BW * (FUSED ? 3 * D : 4)];   // q weight, k weight, (cos, sin) pairs
+    const int lane = threadIdx.x & 63, qc = lane & 15, kg = lane >> 4;
+    const int wv = BW == 1 ? 0 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int32_t* bt_lds = bt_all + wv * BT_LEN;
+    float* fz_lds = fz_all + wv * (FUSED ? 3 * D : 4);
+    // what a wave writes to its part of LDS only itself reads: with one wave a block the barrier is the
+    // fence; with several, a fence of the wave's own (LDS works through a wave's accesses in order)
+    auto wave_sync = [&]() {
+        if constexpr (BW == 1) {
+            __syncthreads();
+        } else {
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+            __builtin_amdgcn_wave_barrier();
+        }
+    };
     int r, col0;
     if (work) {
         r = work[2 * blockIdx.x];
@@ -188,6 +209,12 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
     const int kb0 = (kmin / 32) * 32;
     const int nsteps = (kmax - kb0) / 32 + 1;
     int s_begin = 0, s_end = nsteps;
+    if constexpr (BW > 1) {
+        // (never under 96 keys a wave, as below)
+        const int per = max((nsteps + BW - 1) / BW, min(3, nsteps));
+        s_begin = min(nsteps, wv * per);
+        s_end = min(nsteps, s_begin + per);
+    }
     if (SPLIT) {
         // The launch is sized for the longest context the engine allows; with shorter ones a run
         // of keys is not made shorter than 256 keys as long as some 512 waves are left with
@@ -213,7 +240,7 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
     // is a memory load, and to wait for it is to wait for every key and value load issued
     // before it, one round trip to HBM after the other.  Keys beyond what ATTN_WAVE_BT pages
     // hold are worked through in segments, each with its own page numbers in LDS.
-    const int seg_steps = max(1, ((ATTN_WAVE_BT - 1) * page_size) >> 5);
+    const int seg_steps = max(1, ((BT_LEN - 1) * page_size) >> 5);
     int pi0 = 0;
     auto fill_pages = [&](int seg0, int seg1, int from) {
         pi0 = page_index(kb0 + seg0 * 32, page_size, page_shift);
@@ -283,7 +310,7 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
     // the page numbers of the first segment: the first 64 came with the loads above
     if (lane < first_count) bt_lds[lane] = first_page;
     if (first_count > 64) fill_pages(s_begin, min(s_end, s_begin + seg_steps), 64);
-    __syncthreads();
+    wave_sync();
 
     floatx4 oacc[DT];
 #pragma unroll
@@ -333,6 +360,21 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
             _Pragma("unroll") for (int e = 0; e < 8; ++e)                                           \
                 if (e == at_) vf[buf][dt][e] = vnew[dt];                                            \
     }
+    // The softmax works on raw scores with the scale folded into the exponent,
+    //   p = 2^((s - m) * scale * log2 e),
+    // masks only the steps that touch a column's causal or window edge, and moves the reference m
+    // (and rescales the accumulators) only when some score exceeds it by more than 8 in the
+    // exponent's units: until then p stays below 2^8 and the quotient o / l does not depend on the
+    // reference.  A wave alone on its SIMD is bound by the instructions of a step, not by memory;
+    // rescaling 4 DT accumulator registers in every step was a quarter of them.
+    const float sl2 = scale * 1.44269504088896f;
+    const float slack = 8.0f / sl2;
+    int w_min_pos = c_ok ? c_pos : 0x7fffffff, w_max_lo = c_ok ? c_lo : 0;   // over the wave's columns
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        w_min_pos = min(w_min_pos, __shfl_xor(w_min_pos, o, 64));
+        w_max_lo = max(w_max_lo, __shfl_xor(w_max_lo, o, 64));
+    }
 #define TFF_WAVE_COMPUTE(buf, step)                                                                 \
     {                                                                                               \
         const int kb_ = kb0 + (step) * 32;                                                          \
@@ -342,30 +384,37 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
             _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                       \
                 sacc_[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[buf][kt][ks], qf[ks], sacc_[kt], 0, 0, 0); \
         float sv_[8];                                                                               \
-        float mt_ = -INFINITY;                                                                      \
-        _Pragma("unroll") for (int kt = 0; kt < 2; ++kt)                                            \
-            _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                         \
-                const int j = kb_ + kg * 8 + kt * 4 + i;                                            \
-                const bool vis = j >= c_lo && j <= c_pos;                                           \
-                const float x = vis ? sacc_[kt][i] * scale : -INFINITY;                             \
-                sv_[kt * 4 + i] = x;                                                                \
-                mt_ = fmaxf(mt_, x);                                                                \
+        _Pragma("unroll") for (int e = 0; e < 8; ++e) sv_[e] = sacc_[e >> 2][e & 3];                \
+        if (kb_ + 31 > w_min_pos || kb_ < w_max_lo) {   /* the step touches an edge of some column (a column */ \
+            /* that does not exist has a query of zeros and is masked with the others) */          \
+            _Pragma("unroll") for (int e = 0; e < 8; ++e) {                                         \
+                const int j = kb_ + kg * 8 + e;                                                     \
+                if (!(j >= c_lo && j <= c_pos)) sv_[e] = -INFINITY;                                 \
             }                                                                                       \
-        mt_ = rows_max(mt_);                                                                        \
-        const float m_new_ = fmaxf(m_run, mt_);                                                     \
-        const float alpha_ = m_new_ == -INFINITY ? 1.f : __expf(m_run - m_new_);                    \
+        }                                                                                           \
+        float mt_ = fmaxf(fmaxf(fmaxf(sv_[0], sv_[1]), fmaxf(sv_[2], sv_[3])),                      \
+                          fmaxf(fmaxf(sv_[4], sv_[5]), fmaxf(sv_[6], sv_[7])));                     \
+        float m_new_ = m_run, alpha_ = 1.f;                                                         \
+        if (__any(mt_ > m_run + slack)) {                                                           \
+            mt_ = rows_max(mt_);                                                                    \
+            m_new_ = fmaxf(m_run, mt_);                                                             \
+            alpha_ = m_new_ == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((m_run - m_new_) * sl2);    \
+        }                                                                                           \
+        const float mb_ = m_new_ == -INFINITY ? 0.f : m_new_ * sl2;                                 \
         float ps_ = 0.f;                                                                            \
         bf16x8 pv_;                                                                                 \
         _Pragma("unroll") for (int e = 0; e < 8; ++e) {                                             \
-            const float p = sv_[e] == -INFINITY ? 0.f : __expf(sv_[e] - m_new_);                    \
+            const float p = __builtin_amdgcn_exp2f(fmaf(sv_[e], sl2, -mb_));   /* 2^-inf = 0 for masked scores */ \
             ps_ += p;                                                                               \
             pv_[e] = (bf16_t)p;                                                                     \
         }                                                                                           \
         l_run = l_run * alpha_ + ps_;                                                               \
         m_run = m_new_;                                                                             \
-        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                         \
-            oacc[dt][0] *= alpha_; oacc[dt][1] *= alpha_;                                           \
-            oacc[dt][2] *= alpha_; oacc[dt][3] *= alpha_;                                           \
+        if (__any(alpha_ != 1.f)) {                                                                 \
+            _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                     \
+                oacc[dt][0] *= alpha_; oacc[dt][1] *= alpha_;                                       \
+                oacc[dt][2] *= alpha_; oacc[dt][3] *= alpha_;                                       \
+            }                                                                                       \
         }                                                                                           \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt)                                           \
             oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[buf][dt], pv_, oacc[dt], 0, 0, 0); \
@@ -374,9 +423,9 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
     for (int seg0 = s_begin; seg0 < s_end; seg0 += seg_steps) {
         const int seg1 = min(s_end, seg0 + seg_steps);
         if (seg0 > s_begin) {
-            __syncthreads();            // the segment before is read
+            wave_sync();            // the segment before is read
             fill_pages(seg0, seg1, 0);
-            __syncthreads();
+            wave_sync();
         }
         // steps past the end load the last step again and are not used
 #pragma unroll
@@ -392,7 +441,7 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
                         fz_lds[2 * D + i] = fz_cs[u];
                     }
                 }
-                __syncthreads();
+                wave_sync();
                 if (has_norm || has_rope) norm_rope_fragments<DT>(qf, has_norm, fz_lds, fz.eps, has_rope, fz_lds + 2 * D, fz.pairing, kg);
                 if (owns_new) {
                     norm_rope_fragments<DT>(knew, has_norm, fz_lds + D, fz.eps, has_rope, fz_lds + 2 * D, fz.pairing, kg);
@@ -440,6 +489,54 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
 
     float l = l_run;
     l = rows_sum(l);
+    if constexpr (BW > 1) {
+        // The waves' partial results meet in LDS: [wave][value tile][lane] four floats, and a
+        // maximum and a sum per wave and column.  Wave w then merges value tiles w, w + BW, ...:
+        //   m = max m_s, l = sum l_s e^(m_s - m), o = sum o_s e^(m_s - m) / l
+        // in the order of the waves, whatever their number of keys.
+        __shared__ __attribute__((aligned(16))) float mo[BW * DT * 256];
+        __shared__ float mml[BW * 32];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            *reinterpret_cast<float4*>(mo + ((wv * DT + dt) * 64 + lane) * 4) =
+                make_float4(oacc[dt][0], oacc[dt][1], oacc[dt][2], oacc[dt][3]);
+        if (kg == 0) {
+            mml[wv * 32 + qc * 2] = m_run * scale;   // (in the exponent's natural units)
+            mml[wv * 32 + qc * 2 + 1] = l;
+        }
+        __syncthreads();
+        if (!c_ok) return;
+        float m = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < BW; ++w) m = fmaxf(m, mml[w * 32 + qc * 2]);
+        float wgt[BW], lsum = 0.f;
+#pragma unroll
+        for (int w = 0; w < BW; ++w) {
+            const float ms = mml[w * 32 + qc * 2];
+            wgt[w] = ms == -INFINITY ? 0.f : __expf(ms - m);
+            lsum = fmaf(mml[w * 32 + qc * 2 + 1], wgt[w], lsum);
+        }
+        const float inv = 1.0f / lsum;
+        bf16_t* op = out + ((size_t)c_tok * nq + c_head) * D;
+        for (int dt = wv; dt < DT; dt += BW) {
+            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int w = 0; w < BW; ++w) {
+                const float4 o = *reinterpret_cast<const float4*>(mo + ((w * DT + dt) * 64 + lane) * 4);
+                acc.x = fmaf(o.x, wgt[w], acc.x);
+                acc.y = fmaf(o.y, wgt[w], acc.y);
+                acc.z = fmaf(o.z, wgt[w], acc.z);
+                acc.w = fmaf(o.w, wgt[w], acc.w);
+            }
+            union { bf16_t h[4]; uint2 u; } pk;
+            pk.h[0] = (bf16_t)(acc.x * inv);
+            pk.h[1] = (bf16_t)(acc.y * inv);
+            pk.h[2] = (bf16_t)(acc.z * inv);
+            pk.h[3] = (bf16_t)(acc.w * inv);
+            *reinterpret_cast<uint2*>(op + dt * 16 + kg * 4) = pk.u;
+        }
+        return;
+    }
     if (!c_ok) return;
     if (SPLIT) {
         // keys are split for entries of one token only: partial results are kept by entry
@@ -450,7 +547,7 @@ __global__ __launch_bounds__(64, 1) void attn_wave_kernel(
             *reinterpret_cast<float4*>(po + dt * 16 + kg * 4) =
                 make_float4(oacc[dt][0], oacc[dt][1], oacc[dt][2], oacc[dt][3]);
         if (kg == 0) {
-            part_ml[row * 2] = m_run;
+            part_ml[row * 2] = m_run * scale;   // (the merge works with e^(m_s - m): the reference in the exponent's natural units)
             part_ml[row * 2 + 1] = l;
         }
     } else {
@@ -954,16 +1051,25 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
                 block_items, nq, nkv, page_size, page_shift, window, scale);
         return tff_check_launch("attention_mfma_block");
     }
-    const dim3 grid(num_work, nkv, splits);
+    const dim3 grid(num_work, nkv, max(splits, 1));
     const AttnFuse fz = fuse ? *fuse : AttnFuse{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
 #define TFF_ATTN_ARGS                                                                              \
     q, q_stride, out, part_o, part_ml, k_cache, v_cache, block_tables, bt_stride, cu_tokens,       \
         start_pos, work, tiles_per_entry, nq, nkv, page_size, page_shift, window, scale, T_total
-    if (fuse) {
+    if (fuse && splits == 0) {
+        // a block of eight waves per entry and kv head: the keys split among its waves, merged in LDS
+        if constexpr (DT <= 8) {
+            // (two waves to a SIMD have 256 registers each: four steps of keys and values in flight a wave up to
+            // a head size of 64, two up to 96, one beyond; eight waves keep a CU's 100 GB/s busy either way)
+            attn_wave_kernel<DT, false, (DT <= 4 ? 4 : DT <= 6 ? 2 : 1), true, 8><<<dim3(num_work, nkv, 1), 512, 0, s>>>(TFF_ATTN_ARGS, fz);
+        } else {
+            return tff_fail("attention_decode_fused: blocks of eight waves take head sizes up to 128");
+        }
+    } else if (fuse) {
         if (splits > 1)
-            attn_wave_kernel<DT, true, (DT <= 8 ? 4 : DT <= 12 ? 2 : 1), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
+            attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 1), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
         else
-            attn_wave_kernel<DT, false, (DT <= 8 ? 4 : DT <= 12 ? 2 : 1), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
+            attn_wave_kernel<DT, false, (DT <= 8 ? 4 : 1), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
     } else if (splits > 1) {
         attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
     } else {
@@ -1070,8 +1176,11 @@ TFF_API int tff_attention_decode_fused(const void* qkv, int qkv_stride, void* ou
                 "attention_decode_fused: q and k norm weights must both be given or both be absent");
     TFF_REQUIRE(!cos_sin || ((pairing == 1 || (pairing == 0 && d % 64 == 0)) && max_pos > 0),
                 "attention_decode_fused: pairing %d with head size %d is not supported here", pairing, d);
-    TFF_REQUIRE(splits >= 1 && splits <= 256 && nkv <= 65535, "attention_decode_fused: bad split count %d", splits);
-    TFF_REQUIRE(splits == 1 || (part_o && part_ml), "attention_decode_fused: split keys need a workspace");
+    // splits 0: a block of eight waves per entry and kv head splits the keys among its waves and
+    // merges in LDS (head sizes up to 128; no workspace, no tff_attention_split_reduce afterwards)
+    TFF_REQUIRE(splits >= 0 && splits <= 256 && nkv <= 65535, "attention_decode_fused: bad split count %d", splits);
+    TFF_REQUIRE(splits != 0 || d <= 128, "attention_decode_fused: blocks of eight waves take head sizes up to 128, not %d", d);
+    TFF_REQUIRE(splits <= 1 || (part_o && part_ml), "attention_decode_fused: split keys need a workspace");
     TFF_REQUIRE(bt_stride > 0 && num_pages > 0 && window >= 0 && R >= 0, "attention_decode_fused: bad geometry");
     if (R == 0) return 0;
     const int tiles = (nq / nkv + 15) / 16;

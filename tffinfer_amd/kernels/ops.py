@@ -564,6 +564,12 @@ def _pick_block_cols(batch, G: int, nkv: int, window: int, device, which: str, h
     return cache[key]
 
 
+#: entries x kv heads from which a decode step gives every pair a block of eight waves: a CU
+#: with two waves to a SIMD streams some 45 GB/s (what bounds a wave is the instructions of a step of 32
+#: keys, not memory), 256 of them twice what HBM gives
+BLOCK_DECODE_MIN_PAIRS = 256
+
+
 def pick_splits(waves: int, max_context: int) -> int:
     """Into how many runs the keys of a decoding request are split so that
     the launch has enough waves to pull on all of HBM: about 1024 waves, at
@@ -721,7 +727,12 @@ def attention_decode_fused(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weigh
     if scale is None:
         scale = 1.0 / math.sqrt(d)
     if splits is None:
-        splits = getattr(batch, "attn_splits", None) or pick_splits(R * tiles * nkv, batch.max_context)
+        splits = getattr(batch, "attn_splits", None)
+        if splits is None:
+            # entries x kv heads enough for a block each to saturate HBM between them: the keys of
+            # an entry are split among the eight waves of its block and merged in LDS (splits 0)
+            splits = 0 if (R * nkv >= BLOCK_DECODE_MIN_PAIRS and tiles == 1 and d <= 128) else \
+                pick_splits(R * tiles * nkv, batch.max_context)
     out = torch.empty(R, nq * d, dtype=qkv.dtype, device=qkv.device)
     part_o = part_ml = None
     if splits > 1:
