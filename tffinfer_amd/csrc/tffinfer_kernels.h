@@ -141,7 +141,9 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
 // rotated; pairing 0 needs d to be a multiple of 64), the token's key and value written to
 // position start_pos[r] of the entry's pages where slot_mapping[r] >= 0 (negative, or
 // slot_mapping null: the pages hold them already), attention over the pages.  With
-// splits > 1 the partial results need tff_attention_split_reduce as there.
+// splits > 1 the partial results need tff_attention_split_reduce as there.  splits 0 (head sizes up to
+// 128): a block of eight waves per entry and kv head splits the keys among its waves and merges in LDS;
+// no workspace, no second call.  Worth it from some 256 pairs of entry and kv head on.
 TFF_API int tff_attention_decode_fused(const void* qkv, int qkv_stride, void* out, float* part_o,
                                        float* part_ml, void* k_cache, void* v_cache,
                                        const int32_t* block_tables, int bt_stride,
