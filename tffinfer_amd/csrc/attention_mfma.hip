@@ -592,7 +592,15 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __r
     const float m = block_max(ms, red);
     const float ws = ms == -INFINITY ? 0.f : __expf(ms - m);
     w[tid] = ws;
-    const float l = block_sum(ls * ws, red);   // its barriers also publish w
+    // A launch is sized for the longest context; the runs of keys past an entry's own are empty and
+    // come last: the splits up to the last one that weighs something are fetched, the rest not.
+    __shared__ int used_w[4];
+    {
+        const unsigned long long nz = __ballot(ws != 0.f);
+        if ((tid & 63) == 0) used_w[tid >> 6] = nz ? (tid & ~63) + 64 - __clzll((long long)nz) : 0;
+    }
+    const float l = block_sum(ls * ws, red);   // its barriers also publish w and used_w
+    const int used = max(max(used_w[0], used_w[1]), max(used_w[2], used_w[3]));
     const float inv = 1.0f / l;
     for (int e = tid; e < d; e += blockDim.x) {
         float acc = 0.f;
@@ -604,7 +612,7 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __r
             s0 = AHEAD;
         }
 #pragma unroll 8
-        for (int s = s0; s < splits; ++s)
+        for (int s = s0; s < used; ++s)
             acc = fmaf(part_o[(((size_t)s * R_total + r) * nq + h) * d + e], w[s], acc);
         out[((size_t)t * nq + h) * d + e] = (bf16_t)(acc * inv);
     }
