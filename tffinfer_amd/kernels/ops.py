@@ -572,9 +572,9 @@ BLOCK_DECODE_MIN_PAIRS = 256
 
 def pick_splits(waves: int, max_context: int) -> int:
     """Into how many runs the keys of a decoding request are split so that
-    the launch has enough waves to pull on all of HBM: about 1024 waves, at
-    least 128 keys per run."""
-    return max(1, min(-(-1024 // max(1, waves)), -(-max_context // 128), 256))
+    the launch has enough waves to pull on all of HBM: about 512 waves (a wave
+    alone on its SIMD streams some 30 GB/s), at least 128 keys per run."""
+    return max(1, min(-(-512 // max(1, waves)), -(-max_context // 128), 256))
 
 
 def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,
