@@ -583,6 +583,63 @@ def test_sample_distribution_and_draw(V):
         assert tok[r] == plain_inverse_cdf(ref, float(u[r]))
 
 
+def test_sample_ties_rows_off_alignment_and_batch_position():
+    """More equal logits at a threshold than the kernel keeps in LDS (it then goes through the row
+    again for the lower bits); ties at the top-k and top-p thresholds are all kept, as in the plain
+    implementation; rows of an odd vocabulary start off 16 bytes; a row's token does not depend on
+    where in the batch the row stands."""
+    from plain_qwen3 import plain_inverse_cdf, plain_probs
+    ops = _ops()
+    g = torch.Generator().manual_seed(5)
+    V = 20001
+    base = torch.randn(V, generator=g) * 2
+    tied = torch.randperm(V, generator=g)[:6000]
+    rows, params = [], []
+    for k, p in ((100, 1.0), (0, 0.6), (7000, 0.9)):
+        x = base.clone()
+        x[tied] = 1.5 if k else 3.5      # some 3,200 other logits above 1.5: the 100th largest is not a tie, the 7000th is
+        rows.append(x)
+        params.append((0.9, k, p, 0.0))
+    for V2 in (1, 3, 5, 67):
+        x = torch.full((V,), float("-inf"))
+        x[:V2] = torch.randn(V2, generator=g)
+        rows.append(x)
+        params.append((1.0, 0, 1.0, 0.0))
+    logits = torch.stack(rows)
+    R = len(rows)
+    temp = torch.tensor([q[0] for q in params])
+    top_k = torch.tensor([q[1] for q in params], dtype=torch.int32)
+    top_p = torch.tensor([q[2] for q in params])
+    min_p = torch.tensor([q[3] for q in params])
+    u = torch.linspace(0.05, 0.95, R)
+    tok, probs = ops.sample(logits.to(DEV), temp.to(DEV), u.to(DEV), top_k.to(DEV), top_p.to(DEV), min_p.to(DEV),
+                            return_probs=True)
+    tok, probs = tok.cpu(), probs.cpu()
+    for r in range(R):
+        ref = plain_probs(logits[r], *params[r])
+        assert int((ref > 0).sum()) == int((probs[r] > 0).sum()), f"row {r}: kept sets differ"
+        assert float((probs[r].double() - ref).abs().max()) < 1e-6
+        assert tok[r] == plain_inverse_cdf(ref, float(u[r])), f"row {r}"
+    assert int((probs[2] > 0).sum()) > 7000          # the ties at the 7000th were kept
+    # the same rows in another order, and alone
+    order = [3, 0, 6, 2, 5, 1, 4]
+    again = ops.sample(logits[order].to(DEV), temp[order].to(DEV), u[order].to(DEV), top_k[order].to(DEV),
+                       top_p[order].to(DEV), min_p[order].to(DEV)).cpu()
+    assert torch.equal(again, tok[order])
+    for r in (0, 2):
+        alone = ops.sample(logits[r:r + 1].to(DEV), temp[r:r + 1].to(DEV), u[r:r + 1].to(DEV), top_k[r:r + 1].to(DEV),
+                           top_p[r:r + 1].to(DEV), min_p[r:r + 1].to(DEV)).cpu()
+        assert alone[0] == tok[r]
+
+
+def test_sample_refuses_a_vocabulary_beyond_its_layout():
+    ops = _ops()
+    from tffinfer_amd.kernels.lib import KernelError
+    V = (1 << 20) + 1
+    with pytest.raises(KernelError, match="vocabulary"):
+        ops.sample(torch.zeros(1, V, device=DEV), torch.ones(1, device=DEV), torch.zeros(1, device=DEV))
+
+
 def test_repetition_penalty():
     from plain_qwen3 import plain_repetition_penalty
     ops = _ops()

@@ -199,7 +199,9 @@ TFF_API int tff_repetition_penalty(float* logits, int rows, int V, const int32_t
 
 // Draw from softmax(logits / temperature) restricted by top_k (0: off), top_p
 // (1: off) and min_p (0: off), by inverse CDF in index order with the given
-// uniform number per row.  temperature[r] <= 0 selects the argmax.
+// uniform number per row.  temperature[r] <= 0 selects the argmax.  Probabilities
+// are weighed in units of 2^-40 of the largest one (a token below that is never
+// drawn); V up to 1,048,576.
 TFF_API int tff_sample(const float* logits, int32_t* out, int rows, int V,
                        const float* temperature, const int32_t* top_k, const float* top_p,
                        const float* min_p, const float* uniform, float* probs_out,
