@@ -55,6 +55,10 @@ def parse_args():
     ap.add_argument("--ceilings", action="store_true",
                     help="measure streaming-read bandwidth, back-to-back MFMA rates and a large square product "
                          "on this machine and stop")
+    ap.add_argument("--sampling", default=None, metavar="K,P,T",
+                    help="with --only decode: every request draws from the top K tokens (0: off) that hold a share "
+                         "P of the probability (1: off) at temperature T, e.g. 50,0.95,0.8, instead of taking the "
+                         "most likely one")
     ap.add_argument("--no-large-points", action="store_true",
                     help="skip the two points at the larger shapes (32 mixed requests at the 14B shape; batch 16 "
                          "at 8,192 tokens of context at the 32B shape), which the default run adds to 'points'")
@@ -171,12 +175,21 @@ def main():
     if args.only != "decode":
         pre = M.measure_prefill(engine, gen, args.prefill_tokens, vocab)
     if args.only != "prefill":
-        dec = M.measure_decode(engine, gen, args.batch, args.context, args.steps, args.warmup, vocab)
+        sampling = None
+        if args.sampling:
+            if args.only != "decode":
+                raise SystemExit("--sampling goes with --only decode (the benchmark line is greedy decoding)")
+            from tffinfer_amd.sampling import SamplingConfig
+            k, p, t = args.sampling.split(",")
+            sampling = SamplingConfig(type="top_p", top_k=int(k), top_p=float(p), temperature=float(t), seed=args.seed)
+        dec = M.measure_decode(engine, gen, args.batch, args.context, args.steps, args.warmup, vocab, sampling)
     if args.only:
         part = ({"prefill_ms": round(1000 * pre["wall_s"], 3), "prefill_ms_device": round(1000 * pre["device_s"], 3)}
                 if pre else
                 {"decode_ms_per_step": round(1000 * dec["wall_s"] / args.steps, 4),
                  "decode_ms_per_step_median": round(1000 * dec["step_median_s"], 4)})
+        if args.sampling:
+            part["sampling"] = args.sampling
         print(json.dumps({"only": args.only, **part, "batch": args.batch, "context": args.context}))
         return
     points = {}

@@ -121,6 +121,34 @@ def test_sampling_filters_and_penalty_through_engine(model_dirs):
     assert plain != r.output, "a penalty of 5 was expected to change a tiny model's greedy loop"
 
 
+def test_sampler_parameters_go_round_the_pinned_ring():
+    """The sampler sends its per-row parameters through a ring of pinned buffers, one copy a
+    call: more calls in a row than the ring has buffers, batches of changing size (one of them
+    beyond a buffer's first size), penalties beside draws, every token against the plain
+    implementation."""
+    from tffinfer_amd.sampling import Sampler, SamplingConfig, uniform_at
+    from plain_qwen3 import plain_repetition_penalty
+    sampler = Sampler(torch.device("cuda:0"))
+    V = 300
+    g = torch.Generator().manual_seed(9)
+    for call, R in enumerate([3, 1, 7, 1500, 2, 5, 4, 6, 1, 3]):
+        logits = torch.randn(R, V, generator=g) * 2
+        configs = [SamplingConfig(type=["top_k", "top_p", "random", "greedy"][(r + call) % 4], temperature=0.5 + 0.1 * (r % 7),
+                                  top_k=[0, 5, 40][r % 3], top_p=[1.0, 0.9, 0.6][(r + call) % 3], min_p=[0.0, 0.02][r % 2],
+                                  repetition_penalty=1.0 if (r + call) % 5 else 1.3, seed=100 * call + r) for r in range(R)]
+        indices = [(7 * r + call) % 50 for r in range(R)]
+        seen = [[(r * 13 + j) % V for j in range(1 + r % 9)] for r in range(R)]
+        got = sampler.sample(logits.to("cuda:0"), configs, indices, seen)
+        for r in range(0, R, max(1, R // 12)):
+            c = configs[r]
+            x = plain_repetition_penalty(logits[r], seen[r], c.repetition_penalty) if c.repetition_penalty != 1.0 else logits[r]
+            if c.greedy:
+                assert got[r] == plain_greedy(x), (call, r)
+            else:
+                ref = plain_probs(x, c.temperature, c.top_k, c.top_p, c.min_p)
+                assert got[r] == plain_inverse_cdf(ref, uniform_at(c.seed, indices[r])), (call, r)
+
+
 def test_eos_stops(model_dirs):
     from tffinfer_amd import EngineOptions, LLMEngine
     d = model_dirs["A"]

@@ -1,6 +1,7 @@
 """Chooses the next token of each row of logits on the device."""
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from ..kernels import ops as _ops
@@ -23,10 +24,56 @@ def uniform_at(seed: int, index: int) -> float:
     return (x >> 40) / float(1 << 24)
 
 
+class _Staging:
+    """Per-row parameters on their way to the device: columns of 4-byte numbers packed into one
+    pinned buffer and sent with one asynchronous copy.  A copy from pageable memory makes the
+    host wait until the stream has reached it, that is until the step before has run, and a
+    host that waits cannot launch the next step ahead.  The buffers go round a ring, so that one
+    is written again only steps after its copy was queued (and then waits for that copy)."""
+
+    def __init__(self, device, ring: int = 4, ints: int = 4096):
+        self.device = device
+        self._bufs = [torch.empty(ints, dtype=torch.int32, pin_memory=True) for _ in range(ring)]
+        self._events = [None] * ring
+        self._next = 0
+
+    def send(self, columns: list) -> list[torch.Tensor]:
+        """``columns``: numpy arrays of int32 or float32.  Returns them as device tensors."""
+        offs, total = [], 0
+        for c in columns:
+            offs.append(total)
+            total += (c.size + 3) & ~3              # every column starts at a multiple of 16 bytes
+        i = self._next
+        self._next = (i + 1) % len(self._bufs)
+        if self._events[i] is not None:
+            self._events[i].synchronize()
+        if total > self._bufs[i].numel():
+            self._bufs[i] = torch.empty(max(total, 2 * self._bufs[i].numel()), dtype=torch.int32, pin_memory=True)
+        host = self._bufs[i][:max(total, 4)]
+        flat = host.numpy()
+        for c, o in zip(columns, offs):
+            flat[o:o + c.size] = c.view(np.int32)
+        dev = host.to(self.device, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._events[i] = ev
+        out = []
+        for c, o in zip(columns, offs):
+            t = dev[o:o + c.size]
+            out.append(t.view(torch.float32) if c.dtype == np.float32 else t)
+        return out
+
+
 class Sampler:
     def __init__(self, device, ops=_ops):
         self.device = device
         self.ops = ops
+        self._staging = None
+
+    def _send(self, columns: list) -> list[torch.Tensor]:
+        if self._staging is None:
+            self._staging = _Staging(self.device)
+        return self._staging.send(columns)
 
     def sample(self, logits: torch.Tensor, configs: list[SamplingConfig], indices: list[int],
                seen: list | None = None) -> list[int]:
@@ -50,19 +97,15 @@ class Sampler:
                 if c.repetition_penalty != 1.0 and seen is not None:
                     flat.extend(sorted(set(int(t) for t in seen[r])))
                 cu.append(len(flat))
-            dev = self.device
-            self.ops.repetition_penalty(
-                logits, torch.tensor(flat or [0], dtype=torch.int32, device=dev),
-                torch.tensor(cu, dtype=torch.int32, device=dev),
-                torch.tensor([c.repetition_penalty for c in configs], dtype=torch.float32, device=dev))
+            seen_d, cu_d, pen_d = self._send([
+                np.asarray(flat or [0], dtype=np.int32), np.asarray(cu, dtype=np.int32),
+                np.asarray([c.repetition_penalty for c in configs], dtype=np.float32)])
+            self.ops.repetition_penalty(logits, seen_d, cu_d, pen_d)
         if all(c.greedy for c in configs):
             return self.ops.argmax(logits)
         eff = [c.effective() for c in configs]
-        dev = self.device
-        temperature = torch.tensor([e[0] for e in eff], dtype=torch.float32, device=dev)
-        top_k = torch.tensor([e[1] for e in eff], dtype=torch.int32, device=dev)
-        top_p = torch.tensor([e[2] for e in eff], dtype=torch.float32, device=dev)
-        min_p = torch.tensor([e[3] for e in eff], dtype=torch.float32, device=dev)
-        u = torch.tensor([uniform_at(c.seed, i) for c, i in zip(configs, indices)],
-                         dtype=torch.float32, device=dev)
+        temperature, top_k, top_p, min_p, u = self._send([
+            np.asarray([e[0] for e in eff], dtype=np.float32), np.asarray([e[1] for e in eff], dtype=np.int32),
+            np.asarray([e[2] for e in eff], dtype=np.float32), np.asarray([e[3] for e in eff], dtype=np.float32),
+            np.asarray([uniform_at(c.seed, i) for c, i in zip(configs, indices)], dtype=np.float32)])
         return self.ops.sample(logits, temperature, u, top_k, top_p, min_p)
