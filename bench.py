@@ -55,10 +55,10 @@ def parse_args():
     ap.add_argument("--ceilings", action="store_true",
                     help="measure streaming-read bandwidth, back-to-back MFMA rates and a large square product "
                          "on this machine and stop")
-    ap.add_argument("--sampling", default=None, metavar="K,P,T",
+    ap.add_argument("--sampling", default=None, metavar="K,P,T[,R]",
                     help="with --only decode: every request draws from the top K tokens (0: off) that hold a share "
                          "P of the probability (1: off) at temperature T, e.g. 50,0.95,0.8, instead of taking the "
-                         "most likely one")
+                         "most likely one; R: a repetition penalty")
     ap.add_argument("--no-large-points", action="store_true",
                     help="skip the two points at the larger shapes (32 mixed requests at the 14B shape; batch 16 "
                          "at 8,192 tokens of context at the 32B shape), which the default run adds to 'points'")
@@ -180,8 +180,9 @@ def main():
             if args.only != "decode":
                 raise SystemExit("--sampling goes with --only decode (the benchmark line is greedy decoding)")
             from tffinfer_amd.sampling import SamplingConfig
-            k, p, t = args.sampling.split(",")
-            sampling = SamplingConfig(type="top_p", top_k=int(k), top_p=float(p), temperature=float(t), seed=args.seed)
+            k, p, t, *rest = args.sampling.split(",")
+            sampling = SamplingConfig(type="top_p", top_k=int(k), top_p=float(p), temperature=float(t), seed=args.seed,
+                                      repetition_penalty=float(rest[0]) if rest else 1.0)
         dec = M.measure_decode(engine, gen, args.batch, args.context, args.steps, args.warmup, vocab, sampling)
     if args.only:
         part = ({"prefill_ms": round(1000 * pre["wall_s"], 3), "prefill_ms_device": round(1000 * pre["device_s"], 3)}

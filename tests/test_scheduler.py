@@ -217,6 +217,24 @@ def test_stats_and_determinism():
     assert outs[0] == outs[1]
 
 
+def test_seen_tokens_keep_up_with_a_growing_sequence():
+    """The distinct tokens a repetition penalty needs, brought up to date token by token, are
+    those of the whole sequence at every length, each once."""
+    import random
+    import numpy as np
+    from tffinfer_amd.sampling import SeenTokens
+    rnd = random.Random(4)
+    seq = [rnd.randrange(40) for _ in range(30)]
+    seen = SeenTokens()
+    assert seen.update([]).size == 0
+    for n in (1, 2, 2, 9, 30):
+        got = seen.update(seq[:n])
+        assert got.dtype == np.int32 and sorted(got.tolist()) == sorted(set(seq[:n])) and len(set(got.tolist())) == got.size
+    for _ in range(700):              # beyond the first buffer
+        seq.append(rnd.randrange(5000))
+    assert sorted(seen.update(seq).tolist()) == sorted(set(seq))
+
+
 def test_sampling_config_validation():
     with pytest.raises(ValueError):
         SamplingConfig(type="unknown")

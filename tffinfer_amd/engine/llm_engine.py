@@ -12,7 +12,7 @@ from dataclasses import dataclass, field
 import torch
 
 from ..models import load_model
-from ..sampling import Sampler, SamplingConfig
+from ..sampling import Sampler, SamplingConfig, SeenTokens
 from .batch import StepEntry
 from .runner import ModelRunner
 from .scheduler import Request, Scheduler, SchedulerOptions
@@ -198,14 +198,25 @@ class LLMEngine:
             kept = torch.empty(logits.shape, dtype=torch.float32, pin_memory=True)
             kept.copy_(logits, non_blocking=True)
         ahead = 0 if token_source is None else 1      # outputs the host has not appended yet
+        seen = None
+        if any(r.sampling.repetition_penalty != 1.0 for r in rows):
+            seen = [self._seen_tokens(r) if r.sampling.repetition_penalty != 1.0 else None for r in rows]
         tokens = self.sampler.sample_on_device(
-            logits, [r.sampling for r in rows], [len(r.output) + ahead for r in rows],
-            [r.tokens for r in rows])
+            logits, [r.sampling for r in rows], [len(r.output) + ahead for r in rows], seen)
         host = torch.empty(len(rows), dtype=torch.int32, pin_memory=True)
         host.copy_(tokens, non_blocking=True)
         ready = torch.cuda.Event()
         ready.record()
         return _Launched(plan, rows, tokens, host, ready, kept)
+
+    @staticmethod
+    def _seen_tokens(req):
+        """The distinct tokens of the request's prompt and output, kept with the request and
+        brought up to date with the tokens it got since."""
+        tracker = getattr(req, "_seen_tokens", None)
+        if tracker is None:
+            tracker = req._seen_tokens = SeenTokens()
+        return tracker.update(req.tokens)
 
     def _complete(self, st: _Launched) -> list[tuple]:
         """Reads the step's tokens and tells the scheduler.  Requests that ended

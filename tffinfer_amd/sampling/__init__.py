@@ -1,2 +1,2 @@
 from .params import STRATEGIES, SamplingConfig
-from .sampler import Sampler, uniform_at
+from .sampler import Sampler, SeenTokens, uniform_at

@@ -24,6 +24,32 @@ def uniform_at(seed: int, index: int) -> float:
     return (x >> 40) / float(1 << 24)
 
 
+class SeenTokens:
+    """The distinct tokens of a sequence that only grows (a request's prompt and output), kept up
+    to date token by token: a repetition penalty needs them at every step, and to make a set of a
+    few thousand tokens anew for every request and step costs more than the step itself."""
+
+    def __init__(self):
+        self._set: set = set()
+        self._buf = np.empty(256, dtype=np.int32)
+        self._n = 0
+        self._consumed = 0
+
+    def update(self, tokens) -> np.ndarray:
+        """``tokens``: the sequence so far, longer than (or as long as) at the last call.
+        Returns its distinct tokens, int32, in the order of their first appearance."""
+        for t in tokens[self._consumed:]:
+            t = int(t)
+            if t not in self._set:
+                self._set.add(t)
+                if self._n == self._buf.size:
+                    self._buf = np.concatenate([self._buf, np.empty(self._buf.size, dtype=np.int32)])
+                self._buf[self._n] = t
+                self._n += 1
+        self._consumed = len(tokens)
+        return self._buf[:self._n]
+
+
 class _Staging:
     """Per-row parameters on their way to the device: columns of 4-byte numbers packed into one
     pinned buffer and sent with one asynchronous copy.  A copy from pageable memory makes the
@@ -79,7 +105,8 @@ class Sampler:
                seen: list | None = None) -> list[int]:
         """One token per row.  ``indices[r]`` is the number of the output token
         row r decides (the counter of its random draw); ``seen[r]`` the tokens
-        of its prompt and output so far (needed only with a repetition penalty).
+        of its prompt and output so far (needed only with a repetition penalty):
+        a sequence, or its distinct tokens as an int32 array (``SeenTokens``).
         ``logits`` may be changed in place by the penalty."""
         if logits.shape[0] == 0:
             return []
@@ -92,13 +119,19 @@ class Sampler:
         R = logits.shape[0]
         assert len(configs) == R and len(indices) == R
         if any(c.repetition_penalty != 1.0 for c in configs):
-            flat, cu = [], [0]
+            parts, cu = [], [0]
             for r, c in enumerate(configs):
                 if c.repetition_penalty != 1.0 and seen is not None:
-                    flat.extend(sorted(set(int(t) for t in seen[r])))
-                cu.append(len(flat))
+                    row = seen[r]
+                    if not isinstance(row, np.ndarray):      # a plain sequence: its distinct tokens
+                        row = np.unique(np.asarray(row, dtype=np.int32))
+                    parts.append(row)
+                    cu.append(cu[-1] + row.size)
+                else:
+                    cu.append(cu[-1])
+            flat = np.concatenate(parts) if parts and cu[-1] else np.zeros(1, dtype=np.int32)
             seen_d, cu_d, pen_d = self._send([
-                np.asarray(flat or [0], dtype=np.int32), np.asarray(cu, dtype=np.int32),
+                flat.astype(np.int32, copy=False), np.asarray(cu, dtype=np.int32),
                 np.asarray([c.repetition_penalty for c in configs], dtype=np.float32)])
             self.ops.repetition_penalty(logits, seen_d, cu_d, pen_d)
         if all(c.greedy for c in configs):
