@@ -79,10 +79,11 @@ def test_portions_budget_and_decode_first():
     def on_step(plan):
         total = sum(p.count for p in plan)
         assert total <= 40
-        assert all(p.count <= 24 for p in plan)
         ids = [p.request.id for p in plan]
         assert len(ids) == len(set(ids))
         decodes = [p for p in plan if p.request.num_pending == 1]
+        if any(p.start > 0 for p in decodes):       # somebody decodes: no portion beyond the chunk
+            assert all(p.count <= 24 for p in plan)
         if decodes:  # decodes come first in the plan and are never left out
             assert plan[:len(decodes)] == decodes
             running_decoding = [r for r in sched.running if r.num_pending == 1]
@@ -98,14 +99,40 @@ def test_portions_budget_and_decode_first():
     assert cache.groups[0].pool.num_used == 0 and cache.slots.num_free == 4
 
 
-def test_first_portion_of_first_request():
+def test_prompts_share_the_whole_budget_while_nobody_decodes():
+    """The chunk bounds a step's time for the sake of requests that decode in it.  A prompt alone
+    takes the whole budget; two prompts take a chunk each and the first what is left; beside a
+    request that decodes no portion is longer than the chunk."""
     cache, sched, runner = make(budget=64, chunk=24)
-    sched.add_request(Request("a", list(range(100)), max_new_tokens=2))
+    sched.add_request(Request("a", list(range(100)), max_new_tokens=3))
     plan = sched.schedule()
-    assert [(p.request.id, p.start, p.count, p.samples) for p in plan] == [("a", 0, 24, False)]
+    assert [(p.request.id, p.start, p.count, p.samples) for p in plan] == [("a", 0, 64, False)]
     sched.update(plan, runner.run(plan))
+    sched.add_request(Request("b", list(range(1, 81)), max_new_tokens=3))
+    plan = sched.schedule()          # 36 tokens of a are left: its chunk, b's chunk, the rest of a; 4 more for b
+    assert [(p.request.id, p.start, p.count, p.samples) for p in plan] == [("a", 64, 36, True), ("b", 0, 28, False)]
+    sched.update(plan, runner.run(plan))
+    plan = sched.schedule()          # a decodes now: b gets a chunk and no more
+    assert [(p.request.id, p.start, p.count, p.samples) for p in plan] == [("a", 100, 1, True), ("b", 28, 24, False)]
+    sched.update(plan, runner.run(plan))
+    run_all(sched, runner, cache)
+    assert cache.groups[0].pool.num_used == 0
+
+
+def test_leftover_budget_is_bounded_by_free_pages():
+    """What is left of the budget goes to a prompt only as far as pages are free."""
+    cache, sched, runner = make(num_pages=6, ps=8, budget=64, chunk=16, max_len=64)
+    sched.add_request(Request("a", list(range(47)), max_new_tokens=1))
     plan = sched.schedule()
-    assert (plan[0].start, plan[0].count) == (24, 24)
+    assert [(p.request.id, p.start, p.count, p.samples) for p in plan] == [("a", 0, 47, True)]
+    sched.update(plan, runner.run(plan))
+    cache2, sched2, runner2 = make(num_pages=6, ps=8, budget=64, chunk=16, max_len=64)
+    sched2.add_request(Request("x", list(range(30)), max_new_tokens=1))
+    sched2.add_request(Request("y", list(range(30)), max_new_tokens=1))
+    plan = sched2.schedule()         # six pages of eight: 30 tokens take four, 16 take two, nothing is left for more
+    assert [(p.request.id, p.count) for p in plan] == [("x", 30), ("y", 16)]
+    sched2.update(plan, runner2.run(plan))
+    cache2.check()
 
 
 def test_admission_in_arrival_order_and_slot_limit():

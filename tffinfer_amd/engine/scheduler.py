@@ -230,6 +230,18 @@ class Scheduler:
             self._take(req, n, free)
             plan.append(ScheduledPortion(req, req.num_computed, n, n == req.num_pending))
             budget -= n
+        # 4. prefill_chunk bounds the time of a step for the sake of the requests that decode in it.
+        #    In a step in which none does, what is left of the budget goes to the prompts, in their order.
+        if budget > 0 and plan and not any(p.samples and p.count == 1 and p.start > 0 for p in plan):
+            for i, p in enumerate(plan):
+                rest = p.request.num_pending - p.count
+                if rest <= 0 or budget <= 0:
+                    continue
+                n = self._fit(p.request, p.count + min(rest, budget), free)
+                if n > p.count:
+                    self._take(p.request, n, free)
+                    budget -= n - p.count
+                    plan[i] = ScheduledPortion(p.request, p.start, n, n == p.request.num_pending)
         return plan
 
     # ---- after the step --------------------------------------------------
