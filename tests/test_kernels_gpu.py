@@ -295,6 +295,59 @@ def test_four_wave_cases_cover_every_tile_width():
     assert {(128, False), (192, False), (256, False), (192, True), (256, True)} <= widths, widths
 
 
+ONE_BY_FOUR_CASES = [
+    # M, N, K, gated: few rows and K in units of 64, so tiles of 128 rows on four waves side by side
+    (100, 6150, 4096, False),      # 128 x 128, K split; rows of the result that are no multiple of 16 bytes
+    (120, 24576, 4096, True),      # 128 x 128, gated
+    (40, 51184, 1024, True),       # 128 x 256, gated, a last column tile of a few columns
+    (70, 40000, 512, False),       # 128 x 256
+    (36, 66752, 640, False),       # 128 x 384
+    (102, 73088, 1216, True),      # 128 x 384, gated
+    (100, 4096, 12288, False),     # 128 x 128, eight parts: added up, and handed on
+    (300, 34816, 320, False),      # three row tiles of 128, the last one ragged
+]
+
+
+@pytest.mark.parametrize("M,N,K,glu", ONE_BY_FOUR_CASES)
+def test_linear_on_tiles_of_128_rows(M, N, K, glu):
+    """The four-wave kernel with its waves side by side (tiles of 128 rows: products of few rows, whose
+    time is the weight's stream): every tile width, gated or not, ragged edges, a row stride beyond K,
+    K split over blocks with the sums added or handed on."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(N + K)
+    wide = torch.randn(M, K + 72, generator=g).to(torch.bfloat16).to(DEV)
+    x = wide[:, :K].contiguous()
+    if glu:
+        I = N // 2
+        gate = (torch.randn(I, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+        up = (torch.randn(I, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+        assert _gemm_plan(M, 2 * I, K, 1)[0] == 128
+        a, b = ops.linear(x.float(), gate.float()), ops.linear(x.float(), up.float())
+        ref = a / (1 + torch.exp(-a)) * b
+        pw = ops.pack_gate_up(gate, up)
+        _close(ops.linear(x, pw, out_dtype=torch.float32), ref, 3e-5, "gated product")
+        _close(ops.linear(wide[:, :K], pw), ref, 8e-3, "gated product, strided rows, bfloat16 result")
+        return
+    w = (torch.randn(N, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+    pw = ops.pack_weight(w)
+    ref = ops.linear(x.float(), w.float())
+    for keep in (0, 1):
+        r, c, sp = _gemm_plan(M, N, K, 0, keep)
+        assert r == 128, (r, c, sp)
+        y = ops.linear(x, pw, out_dtype=torch.float32, partials=bool(keep))
+        if keep and sp > 1:
+            assert y.dim() == 3 and y.shape[0] == sp
+        _close(ops.as_tensor(y), ref, 3e-5, f"product (keep={keep}, {c} columns, {sp} parts)")
+        if K >= 4096:
+            assert sp > 1, "a case meant to split K"
+    _close(ops.linear(wide[:, :K], pw), ref, 8e-3, "strided rows, bfloat16 result")
+
+
+def test_cases_of_128_rows_cover_every_tile_width():
+    widths = {(_gemm_plan(M, N, K, int(glu))[1], glu) for M, N, K, glu in ONE_BY_FOUR_CASES}
+    assert {(128, False), (256, False), (384, False), (128, True), (256, True), (384, True)} <= widths, widths
+
+
 @pytest.mark.parametrize("M,N,K", [(2600, 6144, 264), (4500, 520, 200), (1100, 300, 96), (9000, 130, 64),
                                    (2304, 2100, 72)])
 def test_linear_with_many_row_tiles(M, N, K):
@@ -323,11 +376,13 @@ def test_gemm_plan():
     assert plan(8, 4096, 4096) == (0, 0, 1)
     # a few rows, 320 column groups (two rounds for 64 CUs, one for the rest), partial sums wanted
     # anyway and a weight large enough: tiles that split K instead of the streaming kernel
-    assert plan(8, 5120, 8192, keep=1)[:2] == (64, 128) and plan(8, 5120, 8192, keep=1)[2] > 1
+    assert plan(8, 5120, 8192, keep=1)[0] in (64, 128) and plan(8, 5120, 8192, keep=1)[2] > 1
     assert plan(8, 5120, 8192) == (0, 0, 1) and plan(8, 5120, 5120, keep=1) == (0, 0, 1)
     assert plan(8, 4096, 12288, keep=1) == (0, 0, 1)
     assert plan(64, 4096, 12288) == (64, 128, 8)
-    assert plan(64, 151936, 4096) == (64, 128, 1)
+    assert plan(64, 151936, 4096)[0] in (64, 128) and plan(64, 151936, 4096)[2] == 1
+    assert plan(128, 24576, 4096, 1) == (128, 128, 1)    # few rows: tiles of 128 rows, as many blocks as the columns give
+    assert plan(32, 51200, 5120, 1)[:2] == (128, 256)
     assert plan(2048, 24576, 4096, 1)[0] == 256 and plan(2048, 24576, 4096, 1)[2] == 1
     assert plan(2048, 24584, 4104, 1) == (256, 256, 1)  # K no multiple of 64: the sixteen-wave tiles, gated on 256 columns only
     assert plan(4096, 4096, 4096) == (256, 256, 1)
@@ -339,7 +394,7 @@ def test_gemm_plan():
     assert r <= 128 and s >= 2
     for M, N, K in ((100, 203, 2048), (520, 264, 1544), (300, 1000, 64), (2000, 64, 8)):
         r, c, s = plan(M, N, K)
-        assert r in (64, 128, 256) and c in (128, 192, 256) and 1 <= s <= 8 and (s == 1 or (K + 63) // 64 // s >= 8)
+        assert r in (64, 128, 256) and c in (128, 192, 256, 384) and 1 <= s <= 8 and (s == 1 or (K + 63) // 64 // s >= 4)
         assert L.tff_gemm_workspace_bytes(M, N, K, 1, 0, 0) == (s * M * N * 4 if s > 1 else 0)
     assert plan(2048, 4096, 12288, keep=1)[2] >= plan(2048, 4096, 12288)[2]   # kept sums cost less
 

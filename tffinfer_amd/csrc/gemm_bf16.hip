@@ -325,8 +325,9 @@ static int launch_async_g(const bf16_t* A, const bf16_t* Wp, void* C, int M, int
 }
 
 // ------------------------------------------- four waves, whole cache lines ---
-// Block tile 256 x (32 WTN) on 2 x 2 waves, one to a SIMD, each wave 8 x WTN MFMA tiles: half the
-// LDS reads per MFMA of sixteen waves of 64 x 64.  With one wave to a SIMD nothing overlaps unless
+// Block tile 256 x (32 WTN) on 2 x 2 waves (or 128 x (64 WTN) on 1 x 4, for products of few rows,
+// whose time is the weight's stream: all four waves then read the same rows of A), one wave to a
+// SIMD, each wave 8 x WTN MFMA tiles: half the LDS reads per MFMA of sixteen waves of 64 x 64.  With one wave to a SIMD nothing overlaps unless
 // the wave interleaves it itself: the fragments of k-tile t + 1 are read from LDS into a second set
 // of registers, and the copies of later tiles are issued, between the MFMAs of k-tile t.
 //
@@ -434,12 +435,14 @@ __device__ __forceinline__ void w4_store_rows(char* region, F val, TO* out, size
     }
 }
 
-template <int WTN, int NWS, bool GLU, typename TC>
+template <int WTN, int NWS, bool GLU, typename TC, int WGM = 2>
 __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
     int K, int lda, int KB, int n_out) {
-    constexpr int NW = 4, WTM = 8, NA = 3;
-    constexpr int BM = 2 * WTM * 16, BN = 2 * WTN * 16;
+    // WGM: waves along the rows, 2 (a block tile of 256 rows, two waves side by side) or 1 (128 rows, four side by side)
+    constexpr int NW = 4, WTM = 8, NA = 3, WGN = NW / WGM;
+    static_assert(WGM == 1 || WGM == 2, "four waves as 2 x 2 or 1 x 4");
+    constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
     constexpr int WF = BN / 16;                       // W fragments a k-tile, 1 KB each
     constexpr int ACP = BM / 8;                       // A copies a unit, 1 KB each
     constexpr int LPA = ACP / NW, LPW = (WF + NW - 1) / NW;
@@ -454,7 +457,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(
     __shared__ __attribute__((aligned(1024))) char smem[W_BASE + NWS * W_TILE];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = WGM == 2 ? wave >> 1 : 0, wn = WGM == 2 ? wave & 1 : wave;
     const int fr = lane & 15, fg = lane >> 4;
     const int TM = (M + BM - 1) / BM, TN = (N + BN - 1) / BN;
     const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
@@ -628,12 +631,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(
 }
 
 // splits > 1: the blocks of a tile split K among them in units of 64; part holds splits * M * N floats
-template <int WTN, int NWS, bool GLU = false>
+template <int WTN, int NWS, bool GLU = false, int WGM = 2>
 static int launch_w4(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda, int c_dtype,
                      int n_out, hipStream_t s, int splits = 1, float* part = nullptr, bool reduce = true) {
     TFF_REQUIRE(K % 64 == 0, "gemm: the four-wave tiles take K in units of 64, not K=%d", K);
     const int KB = K / 32;
-    constexpr int BM = 256, BN = 2 * WTN * 16;
+    constexpr int BM = 128 * WGM, BN = (4 / WGM) * WTN * 16;
     if (splits <= 1 || !part) { splits = 1; part = nullptr; }
     TFF_REQUIRE(splits <= KB / 2, "gemm: %d parts of %d units of K", splits, KB / 2);
     const long TM = (M + BM - 1) / BM, TN = (N + BN - 1) / BN;
@@ -643,11 +646,11 @@ static int launch_w4(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, i
     const dim3 grid((unsigned)tiles, 1, splits);
     // the blocks of a split K leave plain float32 sums, plane by plane; a gate is applied when they are added up
     if (splits > 1)
-        gemm_bf16_w4_kernel<WTN, NWS, false, float><<<grid, 256, 0, s>>>(A, Wp, part, M, N, K, lda, KB, 0);
+        gemm_bf16_w4_kernel<WTN, NWS, false, float, WGM><<<grid, 256, 0, s>>>(A, Wp, part, M, N, K, lda, KB, 0);
     else if (c_dtype == TFF_F32)
-        gemm_bf16_w4_kernel<WTN, NWS, GLU, float><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
+        gemm_bf16_w4_kernel<WTN, NWS, GLU, float, WGM><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
     else
-        gemm_bf16_w4_kernel<WTN, NWS, GLU, bf16_t><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
+        gemm_bf16_w4_kernel<WTN, NWS, GLU, bf16_t, WGM><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
     if (int rc = tff_check_launch("gemm_bf16_w4")) return rc;
     if (splits > 1 && reduce) {
         const int No = GLU ? n_out : N;
@@ -953,14 +956,9 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
 }
 
 // The tiled product's plan for M > 16: which tile, and into how many parts the blocks of a
-// tile split K.  Up to 64 rows: 64 x 128 tiles (two blocks to a CU), K split so that the most
-// loaded CU has the least to stream.  Beyond: the cheapest of 256 x 256, 256 x 192, 256 x 128 (on
-// four waves, K in units of 64), 128 x 256, 128 x 128 and 64 x 128 tiles with 1 .. 8 parts by a small cost model: rounds of blocks over
-// the CUs times a block's work at the tile's measured rate (large tiles read fewer bytes of
-// LDS per flop), plus the traffic of the partial sums (less where the caller takes them as
-// they are).  Its constants were fitted to measurements of the four products of the 8B, 14B
-// and 32B shapes at 96 .. 4,096 rows on an MI355X (144 cases, every tile with 1 .. 8 parts),
-// where its pick is within 9 % of the best candidate everywhere and 0.7 % from it on average.
+// tile split K, by a small cost model (see plan_for).  With K in units of 64: the four-wave
+// kernel's tiles of 256 rows (256, 192 or 128 columns) and of 128 rows (384, 256 or 128 columns),
+// and the sixteen-wave kernel's 64 x 128; otherwise the sixteen-wave kernel's tiles.
 struct GemmPlan { int tile; int bn; int splits; };   // tile = rows of a block tile
 // Compute units of the current device (256 on an MI355X, which the rates below were fitted on; a
 // device with another count gets plans for its own number of blocks a round).  256 if it cannot
@@ -989,6 +987,40 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
         if (glu || !keep || fill >= 0.8 || (double)N * K < 40e6) return {0, 0, 1};
     }
     const int nk = (K + 63) / 64;
+    if (K % 64 == 0) {
+        // The four-wave kernel's tiles (256 rows on 2 x 2 waves, 128 rows on 1 x 4) and, up to 512 rows,
+        // the sixteen-wave kernel's 64 x 128, two blocks to a CU.  A block goes through its part of K in
+        // units of 64; a unit takes what its MFMAs take at the tile's rate or what its columns of W take
+        // to arrive, whichever is longer: a block's share of the HBM stream, at most what one CU pulls.
+        // Blocks go round the CUs; each round ends with the pipeline filled and the tile stored.  The
+        // constants were fitted to measurements of the four products of the 8B, 14B and 32B shapes at
+        // 17 .. 4,096 rows on an MI355X (weights in turn, so that none comes from a cache; every tile
+        // with 1 .. 8 parts, 204 cases): the pick is 0.3 % from the best candidate on average, 6 % at worst.
+        struct Cand { int bm, bn, slots; double rate; };
+        static const Cand cands[7] = {{256, 256, 1, 6.01e6}, {256, 192, 1, 5.45e6}, {256, 128, 1, 5.04e6},
+                                      {128, 384, 1, 3.24e6}, {128, 256, 1, 4.61e6}, {128, 128, 1, 3.45e6},
+                                      {64, 128, 2, 2.18e6}};
+        const double HBM = 7.72e6, CU_MAX = 6.0e4;       // bytes a microsecond: all CUs together, one alone
+        GemmPlan best = {128, 128, 1};
+        double best_t = 1e30;
+        for (const Cand& c : cands) {
+            if ((c.bm == 256 && M <= 64) || (c.bm == 64 && M > 512)) continue;
+            for (int S = 1; S <= ((glu && M > 64) ? 2 : 8); S *= 2) {
+                if (S > 1 && nk / S < 4) break;
+                const double blocks = (double)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * S;
+                const double rounds = ceil(blocks / (CUS * c.slots));
+                const double share = fmin((double)c.slots, ceil(blocks / CUS));   // blocks that share a CU's MFMAs
+                const double bw = fmin(CU_MAX, HBM / fmin(blocks, CUS * c.slots));
+                const double unit = fmax(2.0 * c.bm * c.bn * 64.0 * share / c.rate, c.bn * 128.0 / bw);
+                double t = rounds * ((double)nk / S * unit + 3.0) + 3.0;
+                // the partial sums: written, read and added by a second kernel, or (kept) read by the
+                // consumer in place of one plane
+                if (S > 1) t += keep ? (S - 1.0) * M * N * 4.0 / 4e6 : (double)S * M * N * 4.0 / 2.54e6 + 2.7;
+                if (t < best_t) { best_t = t; best = {c.bm, c.bn, S}; }
+            }
+        }
+        return best;
+    }
     if (M <= 64) {
         // A stream of W: a CU pulls a block's k-tile of 64 (16 KB) in some 0.63 us whatever else
         // runs, blocks go round the 256 CUs, and the most loaded CU sets the time.  Splitting K
@@ -1007,22 +1039,17 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
         }
         return {64, 128, best_s};
     }
-    // rate: flops a microsecond that a CU sustains on blocks of this tile; slots: blocks a CU holds.
-    // With K in units of 64 the tiles of 256 rows are those of the four-wave kernel (256, 192 or 128
-    // columns, gated or not); otherwise those of the sixteen-wave kernel.
+    // K in no units of 64, more than 64 rows: the sixteen-wave kernel's tiles.  rate: flops a microsecond
+    // that a CU sustains on blocks of this tile; slots: blocks a CU holds.
     struct Cand { int bm, bn, slots; double rate; };
-    static const Cand cands_w4[6] = {{256, 256, 1, 5.7e6}, {256, 192, 1, 5.4e6}, {256, 128, 1, 5.1e6},
-                                     {128, 256, 1, 3.25e6}, {128, 128, 1, 2.7e6}, {64, 128, 2, 2.4e6}};
-    static const Cand cands_w16[6] = {{256, 256, 1, 5.2e6}, {256, 192, 1, 4.4e6}, {128, 256, 1, 3.6e6},
-                                      {128, 128, 1, 2.6e6}, {64, 128, 2, 2.2e6}, {0, 0, 0, 0.0}};
-    const bool w4 = K % 64 == 0;
+    static const Cand cands_w16[5] = {{256, 256, 1, 5.2e6}, {256, 192, 1, 4.4e6}, {128, 256, 1, 3.6e6},
+                                      {128, 128, 1, 2.6e6}, {64, 128, 2, 2.2e6}};
     GemmPlan best = {256, 256, 1};
     double best_t = 1e30;
-    for (const Cand& c : (w4 ? cands_w4 : cands_w16)) {
-        if (c.bm == 0) break;
+    for (const Cand& c : cands_w16) {
         for (int S = 1; S <= (glu ? 2 : 8); S *= 2) {
             // gate and up groups come in pairs, an even number a wave: three a wave of the sixteen do not do
-            if (glu && c.bn == 192 && !w4) break;
+            if (glu && c.bn == 192) break;
             if (S > 1 && nk / S < 8) break;
             const double blocks = (double)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * S;
             const double rounds = ceil(blocks / (CUS * c.slots));
@@ -1032,7 +1059,7 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
             double t = round_us * rounds + 3.0;
             // the partial sums: written, read and added by a second kernel, or (kept) read by the
             // consumer in place of one plane
-            if (S > 1) t += keep ? (S - 1.0) * M * N * 4.0 / 4e6 : (double)S * M * N * 4.0 / (w4 ? 2.6e6 : 3e6) + 3.0;
+            if (S > 1) t += keep ? (S - 1.0) * M * N * 4.0 / 4e6 : (double)S * M * N * 4.0 / 3e6 + 3.0;
             if (t < best_t) { best_t = t; best = {c.bm, c.bn, S}; }
         }
     }
@@ -1104,15 +1131,20 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
         if (M <= 16) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, nullptr);
         if (plan.tile == 64)
             return launch_async_g<2, 2, 2, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
-        if (plan.tile == 128 && plan.bn == 128)
-            return launch_async_g<2, 2, 4, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
-        if (plan.tile == 128)
-            return launch_async_g<2, 4, 4, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         if (K % 64 == 0) {
+            if (plan.tile == 128) {
+                if (plan.bn == 128) return launch_w4<2, 5, true, 1>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+                if (plan.bn == 256) return launch_w4<4, 5, true, 1>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+                return launch_w4<6, 4, true, 1>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+            }
             if (plan.bn == 128) return launch_w4<4, 5, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
             if (plan.bn == 192) return launch_w4<6, 5, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
             return launch_w4<8, 4, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         }
+        if (plan.tile == 128 && plan.bn == 128)
+            return launch_async_g<2, 2, 4, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+        if (plan.tile == 128)
+            return launch_async_g<2, 4, 4, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         return launch_async_g<4, 4, 4, 4, 5, true, 1, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
     }
     if (plan.tile == 0) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, nullptr);
@@ -1125,15 +1157,20 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
         }
         return launch_async_g<2, 2, 2, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     }
-    if (plan.tile == 128 && plan.bn == 128)
-        return launch_async_g<2, 2, 4, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
-    if (plan.tile == 128)
-        return launch_async_g<2, 4, 4, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     if (K % 64 == 0) {
+        if (plan.tile == 128) {
+            if (plan.bn == 128) return launch_w4<2, 5, false, 1>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+            if (plan.bn == 256) return launch_w4<4, 5, false, 1>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+            return launch_w4<6, 4, false, 1>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+        }
         if (plan.bn == 128) return launch_w4<4, 5>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
         if (plan.bn == 192) return launch_w4<6, 5>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
         return launch_w4<8, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     }
+    if (plan.tile == 128 && plan.bn == 128)
+        return launch_async_g<2, 2, 4, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+    if (plan.tile == 128)
+        return launch_async_g<2, 4, 4, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     if (plan.bn == 192)
         return launch_async_g<4, 4, 4, 3, 5, false, 1, true>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     return launch_async_g<4, 4, 4, 4, 5, false, 1, true>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
