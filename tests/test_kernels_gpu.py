@@ -142,13 +142,16 @@ def test_linear_partial_sums_feed_the_norm(M, N, K):
 
 @pytest.mark.parametrize("glu", [False, True])
 @pytest.mark.parametrize("M,H,K,N2", [(1, 64, 64, 96), (8, 4096, 4096, 6144), (5, 320, 96, 200), (16, 200, 1000, 72),
-                                       (3, 1000, 256, 33000), (7, 4096, 12288, 24576), (16, 40, 8200, 136)])
+                                       (3, 1000, 256, 33000), (7, 4096, 12288, 24576), (16, 40, 8200, 136),
+                                       (16, 5120, 512, 51200), (11, 5120, 256, 49138), (2, 5120, 256, 51200)])
 def test_norm_taken_into_the_products_on_either_side(M, H, K, N2, glu):
     """Up to 16 rows: the product before a norm adds to the residual stream, writes (sum * norm
     weight) in bfloat16 and the sums of squares of its groups of 16 columns; the product after it
     multiplies by the row's factor.  Against the three steps done one after the other, in float64,
     with the norm's weights and a residual stream whose rows differ in size by orders of magnitude
-    (a factor applied to the wrong row, or a norm left out, would show)."""
+    (a factor applied to the wrong row, or a norm left out, would show).  The last three cases, gated:
+    a weight so large (or so many rows) that the product after the norm runs on tiles of 128 rows
+    of the four-wave kernel, which takes the rows' factors into its epilogue too."""
     ops = _ops()
     g = torch.Generator().manual_seed(M * 7 + H)
     eps = 1e-5
@@ -305,6 +308,8 @@ ONE_BY_FOUR_CASES = [
     (102, 73088, 1216, True),      # 128 x 384, gated
     (100, 4096, 12288, False),     # 128 x 128, eight parts: added up, and handed on
     (300, 34816, 320, False),      # three row tiles of 128, the last one ragged
+    (16, 51200, 5120, True),       # up to 16 rows, gated, a weight so large that the rows go on tiles, not the streaming kernel
+    (3, 49152, 5120, True),
 ]
 
 

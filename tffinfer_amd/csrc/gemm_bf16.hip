@@ -435,10 +435,18 @@ __device__ __forceinline__ void w4_store_rows(char* region, F val, TO* out, size
     }
 }
 
-template <int WTN, int NWS, bool GLU, typename TC, int WGM = 2>
+// SCALE: A's rows (up to 16 of them) still lack the factor of the RMS norm they went through; the
+// factor, rsqrt(sum of the row's sums of squares / dim + eps), is applied to the accumulators.
+struct W4Scale {
+    const float* ss;        // [16][stride] sums of squares, count of them a row
+    int stride, count;
+    float inv_dim, eps;
+};
+template <int WTN, int NWS, bool GLU, typename TC, int WGM = 2, bool SCALE = false>
 __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
-    int K, int lda, int KB, int n_out) {
+    int K, int lda, int KB, int n_out, W4Scale sc) {
+    static_assert(!SCALE || WGM == 1, "rows that lack their norm's factor: up to 16, one row tile");
     // WGM: waves along the rows, 2 (a block tile of 256 rows, two waves side by side) or 1 (128 rows, four side by side)
     constexpr int NW = 4, WTM = 8, NA = 3, WGN = NW / WGM;
     static_assert(WGM == 1 || WGM == 2, "four waves as 2 x 2 or 1 x 4");
@@ -488,6 +496,24 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(
     for (int i = 0; i < WTN; ++i)
 #pragma unroll
         for (int jj = 0; jj < WTM; ++jj) acc[i][jj] = floatx4{0.f, 0.f, 0.f, 0.f};
+    // (a lane's results are four columns of row fr of each row group: of row fr itself in the first,
+    // the only one that counts with up to 16 rows; the four lanes of a row share out its sums)
+    float row_ss = 0.f;
+    if constexpr (SCALE) {
+        // (16 bytes a load, eight loads asked for before the first is added: one trip to memory for rows of up to 8,192 elements)
+        const float* sp = sc.ss + (size_t)fr * sc.stride;
+        const int vec_end = sc.count & ~3;
+        for (int j0 = fg * 4; j0 < vec_end; j0 += 16 * 8) {
+            float4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                v[u] = j0 + 16 * u < vec_end ? *reinterpret_cast<const float4*>(sp + j0 + 16 * u) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) row_ss += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+        }
+        if (fg == 0)
+            for (int j = vec_end; j < sc.count; ++j) row_ss += sp[j];
+    }
 
     // this wave's copies: of an A unit the copies wave + 4 c, of a W tile the fragments wave + 4 c
     unsigned long long abase[LPA], wbase[LPW];
@@ -617,23 +643,36 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(
     const int mw = m0 + wm * WTM * 16;                // the wave's first row
     constexpr int E = 16 / (int)sizeof(TC);
     const int lane_out = w4_lane();
+    float rs = 1.f;
+    if constexpr (SCALE) {
+        row_ss += __shfl_xor(row_ss, 16, 64);
+        row_ss += __shfl_xor(row_ss, 32, 64);
+        rs = rsqrtf(row_ss * sc.inv_dim + sc.eps);
+    }
+    auto scaled = [&](const floatx4& v) {
+        if constexpr (SCALE) return floatx4{v[0] * rs, v[1] * rs, v[2] * rs, v[3] * rs};
+        else return v;
+    };
     if constexpr (GLU) {
         static_assert(WTN % 2 == 0, "gate and up groups come in pairs");
-        w4_store_rows<WTN / 2, REGION, TC>(region, [&](int i, int jj) { return silu_mul(acc[2 * i][jj], acc[2 * i + 1][jj]); },
+        w4_store_rows<WTN / 2, REGION, TC>(region, [&](int i, int jj) { return silu_mul(scaled(acc[2 * i][jj]), scaled(acc[2 * i + 1][jj])); },
                                            C, (size_t)n_out, mw, (n0 + wn * WTN * 16) / 2, M, n_out, lane_out,
                                            n_out % E == 0);
     } else {
         // (partial sums of a split K: plane blockIdx.z of the launcher's float32 workspace, which it passes as C)
         TC* out = C + (size_t)blockIdx.z * M * N;
-        w4_store_rows<WTN, REGION, TC>(region, [&](int i, int jj) { return acc[i][jj]; }, out, (size_t)N, mw,
+        w4_store_rows<WTN, REGION, TC>(region, [&](int i, int jj) { return scaled(acc[i][jj]); }, out, (size_t)N, mw,
                                        n0 + wn * WTN * 16, M, N, lane_out, N % E == 0);
     }
 }
 
 // splits > 1: the blocks of a tile split K among them in units of 64; part holds splits * M * N floats
-template <int WTN, int NWS, bool GLU = false, int WGM = 2>
+template <int WTN, int NWS, bool GLU = false, int WGM = 2, bool SCALE = false>
 static int launch_w4(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda, int c_dtype,
-                     int n_out, hipStream_t s, int splits = 1, float* part = nullptr, bool reduce = true) {
+                     int n_out, hipStream_t s, int splits = 1, float* part = nullptr, bool reduce = true,
+                     W4Scale sc = W4Scale{nullptr, 0, 0, 0.f, 0.f}) {
+    TFF_REQUIRE(!SCALE || (M <= 16 && sc.ss && (splits <= 1 || !part)),
+                "gemm: rows that lack their norm's factor: up to 16 of them and K in one part");
     TFF_REQUIRE(K % 64 == 0, "gemm: the four-wave tiles take K in units of 64, not K=%d", K);
     const int KB = K / 32;
     constexpr int BM = 128 * WGM, BN = (4 / WGM) * WTN * 16;
@@ -646,11 +685,11 @@ static int launch_w4(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, i
     const dim3 grid((unsigned)tiles, 1, splits);
     // the blocks of a split K leave plain float32 sums, plane by plane; a gate is applied when they are added up
     if (splits > 1)
-        gemm_bf16_w4_kernel<WTN, NWS, false, float, WGM><<<grid, 256, 0, s>>>(A, Wp, part, M, N, K, lda, KB, 0);
+        gemm_bf16_w4_kernel<WTN, NWS, false, float, WGM><<<grid, 256, 0, s>>>(A, Wp, part, M, N, K, lda, KB, 0, sc);
     else if (c_dtype == TFF_F32)
-        gemm_bf16_w4_kernel<WTN, NWS, GLU, float, WGM><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out);
+        gemm_bf16_w4_kernel<WTN, NWS, GLU, float, WGM, SCALE><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out, sc);
     else
-        gemm_bf16_w4_kernel<WTN, NWS, GLU, bf16_t, WGM><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out);
+        gemm_bf16_w4_kernel<WTN, NWS, GLU, bf16_t, WGM, SCALE><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out, sc);
     if (int rc = tff_check_launch("gemm_bf16_w4")) return rc;
     if (splits > 1 && reduce) {
         const int No = GLU ? n_out : N;
@@ -974,6 +1013,32 @@ static int device_cus() {
     }
     return cached[dev];
 }
+// Up to 16 rows, gated, a very large weight (the 32B shape's gate+up, 262M elements): the streaming
+// kernel's blocks each fetch all of A's rows, and with so many blocks that is traffic enough to show:
+// 94 us against 90 on tiles with one row, 115 against 90 with 16.  Then tiles of 128 rows of the
+// four-wave kernel, K in one part.  (At the 8B and 14B shapes' sizes tiles gain only with K in two
+// parts, which the rows' factors in the epilogue do not go with: the streaming kernel stays.)
+static bool few_rows_gated_on_tiles(int M, int N, int K) {
+    (void)M;
+    return K % 64 == 0 && (double)N * K >= 2.4e8;
+}
+// One row tile of 128 rows, K in one part: the width (128, 256 or 384 columns) that plan_for's model prices lowest.
+static int plan_rows128(int N, int K) {
+    const double CUS = (double)device_cus();
+    const int widths[3] = {128, 256, 384};
+    const double rates[3] = {3.45e6, 4.61e6, 3.24e6};
+    int best = 256;
+    double best_t = 1e30;
+    for (int i = 0; i < 3; ++i) {
+        const double blocks = (double)((N + widths[i] - 1) / widths[i]);
+        const double bw = fmin(6.0e4, 7.72e6 / fmin(blocks, CUS));
+        const double unit = fmax(2.0 * 128 * widths[i] * 64.0 / rates[i], widths[i] * 128.0 / bw);
+        const double t = ceil(blocks / CUS) * (K / 64.0 * unit + 3.0);
+        if (t < best_t) { best_t = t; best = widths[i]; }
+    }
+    return best;
+}
+
 static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
     const double CUS = (double)device_cus();
     // Up to 16 rows: the streaming kernel, a block per 16 columns, unless those blocks go badly
@@ -981,6 +1046,7 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
     // partial sums anyway and the weight is large enough for the gain (three eighths of its
     // stream) to pay for the norm's own kernel, which the streaming kernel would have taken into
     // its epilogue: then the tiles below, whose blocks split K as finely as it takes.
+    if (M <= 16 && glu && few_rows_gated_on_tiles(M, N, K)) return {128, plan_rows128(N, K), 1};
     if (M <= 16) {
         const int nb = (N + 15) / 16;
         const double fill = (double)nb / (ceil(nb / CUS) * CUS);
@@ -1128,7 +1194,7 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
     if (glu_out > 0) {
         TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
                     "gemm: a gated weight of %d rows does not fit %d output columns", N, glu_out);
-        if (M <= 16) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, nullptr);
+        if (plan.tile == 0) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, nullptr);
         if (plan.tile == 64)
             return launch_async_g<2, 2, 2, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         if (K % 64 == 0) {
@@ -1217,6 +1283,18 @@ TFF_API int tff_gemm_row_scaled(const void* A, const void* Wp, void* C, int M, i
     if (glu_out > 0)
         TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
                     "gemm_row_scaled: a gated weight of %d rows does not fit %d output columns", N, glu_out);
+    // (the four-wave kernel's tiles of 128 rows take the rows' factors into their epilogue too)
+    if (glu_out > 0 && few_rows_gated_on_tiles(M, N, K)) {
+        const W4Scale sc{ss, ss_stride, ss_count, 1.0f / (float)dim, eps};
+        const bf16_t* a = (const bf16_t*)A;
+        const bf16_t* w = (const bf16_t*)Wp;
+        hipStream_t s = (hipStream_t)stream;
+        switch (plan_rows128(N, K)) {
+            case 128: return launch_w4<2, 5, true, 1, true>(a, w, C, M, N, K, lda, c_dtype, glu_out, s, 1, nullptr, true, sc);
+            case 256: return launch_w4<4, 5, true, 1, true>(a, w, C, M, N, K, lda, c_dtype, glu_out, s, 1, nullptr, true, sc);
+            default: return launch_w4<6, 4, true, 1, true>(a, w, C, M, N, K, lda, c_dtype, glu_out, s, 1, nullptr, true, sc);
+        }
+    }
     SkinnyFuse fz{ss, ss_stride, ss_count, 1.0f / (float)dim, eps, nullptr, nullptr, nullptr, nullptr, 0};
     return skinny_for<1>((const bf16_t*)A, (const bf16_t*)Wp, C, M, N, K, lda, c_dtype, glu_out, (hipStream_t)stream, &fz);
 }
