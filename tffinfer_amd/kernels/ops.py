@@ -15,9 +15,11 @@ from __future__ import annotations
 import ctypes
 import math
 
+import numpy as np
 import torch
 
 from . import lib as _lib
+from . import staging as _staging
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
@@ -29,7 +31,15 @@ def dtype_code(dt: torch.dtype) -> int:
         raise _lib.KernelError(f"element type {dt} is not supported (float32 or bfloat16)") from None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """The current stream's handle.  Asked for at every launch (hundreds a step when a step is
+    launched kernel by kernel): through torch's C binding where there is one, which costs a
+    tenth of building a Stream object."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -460,7 +470,7 @@ def _attention_work(batch, G: int, cols: int, device, which: str = "all") -> tor
         for r in _entries(batch, which):
             for c0 in range(0, (cu[r + 1] - cu[r]) * G, cols):
                 flat.extend((r, c0))
-        cache[key] = torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(device)
+        cache[key] = _staging.send(device, [np.asarray(flat, dtype=np.int32).reshape(-1, 2)])[0]
     return cache[key]
 
 
@@ -528,8 +538,9 @@ def _attention_block_work(batch, G: int, nkv: int, window: int, device, cols: in
                 order.extend(lst)
                 starts.append(len(order))
         flat = [x for it in order for x in it[1:]]
-        cache[key] = (torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(device),
-                      torch.tensor(starts, dtype=torch.int32).to(device), len(starts) - 1, groups)
+        items_d, starts_d = _staging.send(device, [np.asarray(flat, dtype=np.int32).reshape(-1, 2),
+                                                   np.asarray(starts, dtype=np.int32)])
+        cache[key] = (items_d, starts_d, len(starts) - 1, groups)
     return cache[key]
 
 
@@ -647,7 +658,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
         cache = batch._attn_work
         if "single_rows" not in cache:
             cu = batch.host_cu_tokens
-            cache["single_rows"] = torch.tensor([(r, cu[r]) for r in single], dtype=torch.int32).to(q.device)
+            cache["single_rows"] = _staging.send(q.device, [np.asarray([(r, cu[r]) for r in single], dtype=np.int32)])[0]
         sp = splits if splits is not None else pick_splits(work.shape[0] * nkv, batch.max_context)
         launch(work, work.shape[0], None, 0, 1, 16, sp, cache["single_rows"])
     if cols == 128:

@@ -5,6 +5,7 @@ import numpy as np
 import torch
 
 from ..kernels import ops as _ops
+from ..kernels import staging as _staging
 from .params import SamplingConfig
 
 _M = (1 << 64) - 1
@@ -50,56 +51,15 @@ class SeenTokens:
         return self._buf[:self._n]
 
 
-class _Staging:
-    """Per-row parameters on their way to the device: columns of 4-byte numbers packed into one
-    pinned buffer and sent with one asynchronous copy.  A copy from pageable memory makes the
-    host wait until the stream has reached it, that is until the step before has run, and a
-    host that waits cannot launch the next step ahead.  The buffers go round a ring, so that one
-    is written again only steps after its copy was queued (and then waits for that copy)."""
-
-    def __init__(self, device, ring: int = 4, ints: int = 4096):
-        self.device = device
-        self._bufs = [torch.empty(ints, dtype=torch.int32, pin_memory=True) for _ in range(ring)]
-        self._events = [None] * ring
-        self._next = 0
-
-    def send(self, columns: list) -> list[torch.Tensor]:
-        """``columns``: numpy arrays of int32 or float32.  Returns them as device tensors."""
-        offs, total = [], 0
-        for c in columns:
-            offs.append(total)
-            total += (c.size + 3) & ~3              # every column starts at a multiple of 16 bytes
-        i = self._next
-        self._next = (i + 1) % len(self._bufs)
-        if self._events[i] is not None:
-            self._events[i].synchronize()
-        if total > self._bufs[i].numel():
-            self._bufs[i] = torch.empty(max(total, 2 * self._bufs[i].numel()), dtype=torch.int32, pin_memory=True)
-        host = self._bufs[i][:max(total, 4)]
-        flat = host.numpy()
-        for c, o in zip(columns, offs):
-            flat[o:o + c.size] = c.view(np.int32)
-        dev = host.to(self.device, non_blocking=True)
-        ev = torch.cuda.Event()
-        ev.record()
-        self._events[i] = ev
-        out = []
-        for c, o in zip(columns, offs):
-            t = dev[o:o + c.size]
-            out.append(t.view(torch.float32) if c.dtype == np.float32 else t)
-        return out
-
-
 class Sampler:
     def __init__(self, device, ops=_ops):
         self.device = device
         self.ops = ops
-        self._staging = None
 
     def _send(self, columns: list) -> list[torch.Tensor]:
-        if self._staging is None:
-            self._staging = _Staging(self.device)
-        return self._staging.send(columns)
+        # (a copy from pageable memory would make the host wait for the step in flight, and a host that
+        # waits cannot launch the next step ahead)
+        return _staging.send(self.device, columns)
 
     def sample(self, logits: torch.Tensor, configs: list[SamplingConfig], indices: list[int],
                seen: list | None = None) -> list[int]:
