@@ -618,7 +618,7 @@ def test_argmax_first_maximum():
     assert torch.equal(out[3:].long(), x[3:].argmax(-1))
 
 
-@pytest.mark.parametrize("V", [320, 5000, 151936])
+@pytest.mark.parametrize("V", [320, 5000, 151936, 600001])
 def test_sample_distribution_and_draw(V):
     from plain_qwen3 import plain_inverse_cdf, plain_probs
     ops = _ops()
