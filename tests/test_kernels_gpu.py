@@ -616,6 +616,17 @@ def test_argmax_first_maximum():
     out = ops.argmax(x.to(DEV)).cpu()
     assert out[0] == 77 and out[1] == 4999 and out[2] == 0
     assert torch.equal(out[3:].long(), x[3:].argmax(-1))
+    # few rows of a large vocabulary: a row cut into runs over several blocks, then the first of their maxima
+    V = 151937
+    y = torch.randn(5, V)
+    y[0, 100] = y[0, 100000] = 50.0          # equal maxima in different runs: the first one
+    y[1, V - 1] = 50.0                       # the last element of the last run
+    y[2, 4748] = y[2, 4749] = 50.0           # at a run's edge
+    y[3] = float("nan")                      # nothing compares: index 0
+    got = ops.argmax(y.to(DEV)).cpu()
+    assert got.tolist()[:4] == [100, V - 1, 4748, 0] and got[4] == y[4].argmax()
+    one = ops.argmax(y[4:5, 1:40000].contiguous().to(DEV)).cpu()     # rows off 16 bytes
+    assert one[0] == y[4, 1:40000].argmax()
 
 
 @pytest.mark.parametrize("V", [320, 5000, 151936, 600001])

@@ -189,7 +189,10 @@ TFF_API int tff_cast(const void* src, int src_dtype, void* dst, int dst_dtype, i
                      tff_stream_t stream);
 
 // out[r] = lowest index among the maxima of logits[r, :].
-TFF_API int tff_argmax(const float* logits, int32_t* out, int rows, int V, tff_stream_t stream);
+// workspace: tff_argmax_workspace_bytes(rows, V) bytes, 16-byte aligned (0: none needed), for the
+// form that cuts a row into runs over several blocks; null selects one block a row.
+TFF_API size_t tff_argmax_workspace_bytes(int rows, int V);
+TFF_API int tff_argmax(const float* logits, int32_t* out, int rows, int V, void* workspace, tff_stream_t stream);
 
 // logits[r, seen] is divided by penalty[r] if positive, multiplied otherwise,
 // for the distinct token ids seen[cu_seen[r] .. cu_seen[r+1]).

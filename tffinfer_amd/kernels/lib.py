@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 
 class KernelLibraryError(RuntimeError):
@@ -45,7 +45,8 @@ _SIGNATURES = {
     "tff_attention_split_reduce": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _P],
     "tff_swiglu": [_P, _P, _I, _I, _I, _P],
     "tff_cast": [_P, _I, _P, _I, c_int64, _P],
-    "tff_argmax": [_P, _P, _I, _I, _P],
+    "tff_argmax_workspace_bytes": [_I, _I],
+    "tff_argmax": [_P, _P, _I, _I, _P, _P],
     "tff_repetition_penalty": [_P, _I, _I, _P, _P, _P, _P],
     "tff_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
     "tff_probe_stream_read": [_P, _Z, _P, _I, _P],

@@ -818,7 +818,9 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     R, V = logits.shape
     out = torch.empty(R, dtype=torch.int32, device=logits.device)
     L = _lib.load()
-    _lib.check(L.tff_argmax(logits.data_ptr(), out.data_ptr(), R, V, _stream()))
+    ws_bytes = L.tff_argmax_workspace_bytes(R, V)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=logits.device) if ws_bytes else None
+    _lib.check(L.tff_argmax(logits.data_ptr(), out.data_ptr(), R, V, _ptr(ws), _stream()))
     return out
 
 
