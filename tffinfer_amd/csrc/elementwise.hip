@@ -383,6 +383,48 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_reg_kernel(
     }
 }
 
+// The values of 8 consecutive tokens and one kv head go to their (transposed) pages: where the 8
+// slots are consecutive and start at a multiple of 8 in a page, a thread writes one element's 8
+// tokens as one 16-byte run; else token by token.  (Blocks of qk_norm_rope_vec_kernel's grid.)
+__device__ __forceinline__ void v_page_write_block(
+    const bf16_t* __restrict__ qkv, int T, int nq, int nkv, int d, const int32_t* __restrict__ slot_mapping,
+    bf16_t* __restrict__ v_cache, int page_size, int t0, int head) {
+    __shared__ __attribute__((aligned(16))) bf16_t tile[8][QK_MAX_D];
+    __shared__ int32_t slots[8];
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    const int width = (nq + 2 * nkv) * d;
+    const int cpr = d / 8;   // 16-byte chunks per row
+    if (tid < 8) slots[tid] = t0 + tid < T ? slot_mapping[t0 + tid] : -1;
+    for (int i = tid; i < 8 * cpr; i += nthr) {
+        const int tk = i / cpr, c = i % cpr;
+        uint4 val = make_uint4(0, 0, 0, 0);
+        if (t0 + tk < T)
+            val = *reinterpret_cast<const uint4*>(qkv + (size_t)(t0 + tk) * width + (size_t)(nq + nkv + head) * d + c * 8);
+        *reinterpret_cast<uint4*>(&tile[tk][c * 8]) = val;
+    }
+    __syncthreads();
+    const int s0 = slots[0];
+    bool run = s0 >= 0 && (s0 & 7) == 0 && (s0 % page_size) + 8 <= page_size;
+#pragma unroll
+    for (int i = 1; i < 8; ++i) run = run && slots[i] == s0 + i;
+    if (run) {
+        bf16_t* vt = v_cache + ((size_t)(s0 / page_size) * nkv + head) * d * page_size + (s0 % page_size);
+        for (int e = tid; e < d; e += nthr) {
+            union { uint4 u; bf16_t h[8]; } pk;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pk.h[i] = tile[i][e];
+            *reinterpret_cast<uint4*>(vt + (size_t)e * page_size) = pk.u;
+        }
+    } else {
+        for (int i = 0; i < 8; ++i) {
+            const int slot = slots[i];
+            if (slot < 0) continue;
+            bf16_t* vt = v_cache + ((size_t)(slot / page_size) * nkv + head) * d * page_size + (slot % page_size);
+            for (int e = tid; e < d; e += nthr) vt[(size_t)e * page_size] = tile[i][e];
+        }
+    }
+}
+
 // bfloat16, head sizes 16 .. 256 that are powers of two, the whole head rotated (or none of it):
 // a lane has 8 consecutive elements of a head (one 16-byte access), LPH = d / 8 lanes a head,
 // 64 / LPH heads a wave.  The sum of squares goes over the head's lanes by shuffles; with pairs
@@ -392,8 +434,16 @@ __global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(
     bf16_t* __restrict__ qkv, int nq, int nkv, const float* __restrict__ qw,
     const float* __restrict__ kw, float eps, const float* __restrict__ cos_sin, int pairing,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slot_mapping,
-    bf16_t* __restrict__ k_cache, int page_size) {
+    bf16_t* __restrict__ k_cache, int page_size, int qk_rows, int T, bf16_t* __restrict__ v_cache) {
     constexpr int D = LPH * 8, HPW = 64 / LPH;
+    // The grid's rows beyond the q and k heads' are the values' way to their pages, 8 tokens and one kv
+    // head a block: one launch for both, and they run side by side.
+    if ((int)blockIdx.y >= qk_rows) {
+        const long item = (long)((int)blockIdx.y - qk_rows) * T + blockIdx.x;     // (8 tokens, kv head), heads fastest
+        if (item < (long)((T + 7) / 8) * nkv)
+            v_page_write_block(qkv, T, nq, nkv, D, slot_mapping, v_cache, page_size, (int)(item / nkv) * 8, (int)(item % nkv));
+        return;
+    }
     const int t = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l = lane % LPH;
@@ -475,55 +525,15 @@ __global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(
     }
 }
 
-// The values of 8 consecutive tokens and one kv head go to their (transposed) pages: where the 8
-// slots are consecutive and start at a multiple of 8 in a page, a thread writes one element's 8
-// tokens as one 16-byte run; else token by token.
-__global__ __launch_bounds__(128) void v_page_write_kernel(
-    const bf16_t* __restrict__ qkv, int T, int nq, int nkv, int d,
-    const int32_t* __restrict__ slot_mapping, bf16_t* __restrict__ v_cache, int page_size) {
-    __shared__ __attribute__((aligned(16))) bf16_t tile[8][QK_MAX_D];
-    __shared__ int32_t slots[8];
-    const int t0 = blockIdx.x * 8, head = blockIdx.y, tid = threadIdx.x;
-    const int width = (nq + 2 * nkv) * d;
-    const int cpr = d / 8;   // 16-byte chunks per row
-    if (tid < 8) slots[tid] = t0 + tid < T ? slot_mapping[t0 + tid] : -1;
-    for (int i = tid; i < 8 * cpr; i += 128) {
-        const int tk = i / cpr, c = i % cpr;
-        uint4 val = make_uint4(0, 0, 0, 0);
-        if (t0 + tk < T)
-            val = *reinterpret_cast<const uint4*>(qkv + (size_t)(t0 + tk) * width + (size_t)(nq + nkv + head) * d + c * 8);
-        *reinterpret_cast<uint4*>(&tile[tk][c * 8]) = val;
-    }
-    __syncthreads();
-    const int s0 = slots[0];
-    bool run = s0 >= 0 && (s0 & 7) == 0 && (s0 % page_size) + 8 <= page_size;
-#pragma unroll
-    for (int i = 1; i < 8; ++i) run = run && slots[i] == s0 + i;
-    if (run) {
-        bf16_t* vt = v_cache + ((size_t)(s0 / page_size) * nkv + head) * d * page_size + (s0 % page_size);
-        for (int e = tid; e < d; e += 128) {
-            union { uint4 u; bf16_t h[8]; } pk;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) pk.h[i] = tile[i][e];
-            *reinterpret_cast<uint4*>(vt + (size_t)e * page_size) = pk.u;
-        }
-    } else {
-        for (int i = 0; i < 8; ++i) {
-            const int slot = slots[i];
-            if (slot < 0) continue;
-            bf16_t* vt = v_cache + ((size_t)(slot / page_size) * nkv + head) * d * page_size + (slot % page_size);
-            for (int e = tid; e < d; e += 128) vt[(size_t)e * page_size] = tile[i][e];
-        }
-    }
-}
-
 template <int LPH>
 static void launch_qk_vec(bf16_t* qkv, int T, int nq, int nkv, const float* qw, const float* kw, float eps,
                           const float* cos_sin, int pairing, const int32_t* positions,
-                          const int32_t* slot_mapping, bf16_t* k_cache, int page_size, hipStream_t s) {
+                          const int32_t* slot_mapping, bf16_t* k_cache, bf16_t* v_cache, int page_size, hipStream_t s) {
     constexpr int HPB = 4 * (64 / LPH);
-    qk_norm_rope_vec_kernel<LPH><<<dim3(T, (nq + nkv + HPB - 1) / HPB), 256, 0, s>>>(
-        qkv, nq, nkv, qw, kw, eps, cos_sin, pairing, positions, slot_mapping, k_cache, page_size);
+    const int qk_rows = (nq + nkv + HPB - 1) / HPB;
+    const int v_rows = (int)(((long)((T + 7) / 8) * nkv + T - 1) / T);   // the values' blocks fill whole rows of the grid
+    qk_norm_rope_vec_kernel<LPH><<<dim3(T, qk_rows + v_rows), 256, 0, s>>>(
+        qkv, nq, nkv, qw, kw, eps, cos_sin, pairing, positions, slot_mapping, k_cache, page_size, qk_rows, T, v_cache);
 }
 
 TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d, const float* q_weight,
@@ -554,14 +564,14 @@ TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d, const 
     hipStream_t s = (hipStream_t)stream;
     TFF_REQUIRE(dtype == TFF_F32 || dtype == TFF_BF16, "qk_norm_rope_kv: unknown dtype %d", dtype);
     const bool pow2 = d >= 16 && d <= 256 && (d & (d - 1)) == 0;
-    // for prompt portions: two kernels with 16-byte accesses; a few tokens are done by one launch
+    // for prompt portions: 16-byte accesses, the q and k heads and the values in blocks of their own of one launch
     if (T >= 128 && dtype == TFF_BF16 && pow2 && (!cos_sin || rot_dim == d) && ((uintptr_t)qkv % 16) == 0 &&
         ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 16) == 0 &&
         (!q_weight || (((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0)) &&
         (!cos_sin || ((uintptr_t)cos_sin % 16) == 0)) {
 #define TFF_QK_VEC(L)                                                                               \
     launch_qk_vec<L>((bf16_t*)qkv, T, nq, nkv, q_weight, k_weight, eps, cos_sin, pairing, positions, \
-                     slot_mapping, (bf16_t*)k_cache, page_size, s)
+                     slot_mapping, (bf16_t*)k_cache, (bf16_t*)v_cache, page_size, s)
         switch (d) {
             case 16: TFF_QK_VEC(2); break;
             case 32: TFF_QK_VEC(4); break;
@@ -570,10 +580,7 @@ TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d, const 
             default: TFF_QK_VEC(32); break;
         }
 #undef TFF_QK_VEC
-        if (int rc = tff_check_launch("qk_norm_rope")) return rc;
-        v_page_write_kernel<<<dim3((T + 7) / 8, nkv), 128, 0, s>>>((const bf16_t*)qkv, T, nq, nkv, d, slot_mapping,
-                                                                 (bf16_t*)v_cache, page_size);
-        return tff_check_launch("v_page_write");
+        return tff_check_launch("qk_norm_rope");
     }
     if (!cos_sin || rot_dim == d) {
         dim3 grid4(T, (nq + 2 * nkv + 3) / 4);
