@@ -68,3 +68,19 @@ def test_key_groups_and_blocks_follow_the_amount_of_work():
     # a portion of 2,048 tokens late in a long context is plenty of work as well
     _, _, blocks, groups = _attention_block_work(_batch([(6144, 2048)]), 4, 8, 0, "cpu", num_cus=256)
     assert (blocks, groups) == (64, 1)
+
+
+def test_staged_tables_keep_shape_and_type_on_the_host():
+    """The staging module's host form (what the work lists' tests above go through): every
+    column comes back as a tensor of its own shape and element type, a copy of the array."""
+    import numpy as np
+    import torch
+    from tffinfer_amd.kernels import staging
+    a = np.arange(12, dtype=np.int32).reshape(-1, 2)
+    b = np.asarray([0.5, 1.5, -2.0], dtype=np.float32)
+    c = np.zeros((0, 2), dtype=np.int32)
+    ta, tb, tc = staging.send("cpu", [a, b, c])
+    assert ta.dtype == torch.int32 and tuple(ta.shape) == (6, 2) and ta.tolist() == a.tolist()
+    assert tb.dtype == torch.float32 and tb.tolist() == b.tolist() and tuple(tc.shape) == (0, 2)
+    a[0, 0] = 99
+    assert ta[0, 0] == 0
