@@ -199,6 +199,13 @@ def main():
             k = min(args.steps, 32)
             r = M.measure_decode(engine, gen, b, args.context, k, min(args.warmup, 4), vocab)
             points[key] = round(b * k / r["wall_s"], 1)
+        # the headline batch again with every request drawing from the top 50 tokens at top-p 0.95 and
+        # temperature 0.8 instead of taking the most likely one
+        from tffinfer_amd.sampling import SamplingConfig
+        k = min(args.steps, 32)
+        r = M.measure_decode(engine, gen, args.batch, args.context, k, min(args.warmup, 4), vocab,
+                             SamplingConfig(type="top_p", top_k=50, top_p=0.95, temperature=0.8, seed=args.seed))
+        points[f"decode_b{args.batch}_top_k50_top_p0.95"] = round(args.batch * k / r["wall_s"], 1)
     ceilings = M.quick_ceilings("cuda:0")
 
     t_decode, t_prefill = dec["wall_s"], pre["wall_s"]

@@ -46,4 +46,6 @@ def test_one_json_line_with_the_contract_keys():
     assert rec["prefill"]["tokens"] == 8200 and rec["prefill"]["ms"] > 0 and 0 < rec["prefill"]["frac"] < 1
     assert rec["roofline"]["bound"] == "hbm" and rec["roofline"]["peak"] == 8000.0
     assert rec["roofline"]["frac"] == pytest.approx(rec["roofline"]["achieved"] / 8000.0, abs=1e-3)
-    assert set(rec["points"]) == {"decode_b1", "decode_b64"} and all(v > 0 for v in rec["points"].values())
+    assert set(rec["points"]) == {"decode_b1", "decode_b64", "decode_b2_top_k50_top_p0.95"}
+    assert all(v > 0 for v in rec["points"].values())
+    assert rec["points"]["decode_b2_top_k50_top_p0.95"] < 1.05 * rec["value"]      # drawing costs something, not nothing
