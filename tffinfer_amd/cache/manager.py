@@ -137,13 +137,6 @@ class CacheManager:
     def block_table(self, group: int, req) -> list[int]:
         return self.groups[group].tables[req]
 
-    def bytes_per_token(self) -> int:
-        total = 0
-        for g in self.groups:
-            esz = g.kv.element_size() if g.kv is not None else 2
-            total += len(g.cache_ids) * 2 * g.spec.num_kv_heads * g.spec.head_dim * esz
-        return total
-
     # ---- life of a request ----------------------------------------------
     def add_request(self, req) -> int:
         if req in self.requests:
