@@ -13,7 +13,7 @@ import argparse
 import json
 import sys
 
-# layer sizes of the benchmark configuration (Qwen3-8B shape) and of the two larger shapes
+# layer sizes of the benchmark configuration (Qwen3-8B shape), of three smaller shapes and of two larger ones
 QWEN3_8B = dict(
     architectures=["Qwen3ForCausalLM"], hidden_size=4096, num_hidden_layers=36,
     num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288,
@@ -21,6 +21,11 @@ QWEN3_8B = dict(
     tie_word_embeddings=False,
 )
 SHAPES = {
+    "0.6b": ("Qwen3-0.6B shape", dict(QWEN3_8B, hidden_size=1024, num_hidden_layers=28, num_attention_heads=16,
+                                      intermediate_size=3072, tie_word_embeddings=True)),
+    "1.7b": ("Qwen3-1.7B shape", dict(QWEN3_8B, hidden_size=2048, num_hidden_layers=28, num_attention_heads=16,
+                                      intermediate_size=6144, tie_word_embeddings=True)),
+    "4b": ("Qwen3-4B shape", dict(QWEN3_8B, hidden_size=2560, intermediate_size=9728, tie_word_embeddings=True)),
     "8b": ("Qwen3-8B shape", QWEN3_8B),
     "14b": ("Qwen3-14B shape", dict(QWEN3_8B, hidden_size=5120, num_hidden_layers=40, num_attention_heads=40,
                                     intermediate_size=17408)),
@@ -37,7 +42,7 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048)
     ap.add_argument("--shape", choices=sorted(SHAPES), default="8b",
-                    help="layer sizes: the benchmark configuration (8b) or one of the larger shapes")
+                    help="layer sizes: the benchmark configuration (8b) or one of the smaller and larger shapes")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--prefill-tokens", type=int, default=2048)

@@ -1158,13 +1158,20 @@ static int skinny_for(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, 
         if constexpr (EPI != 2) {
             if (N >= 16 * 1024)
                 return launch_skinny<1, 1, 8, 1, 2, true, true, EPI>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, fuse);
-            // (with the norm's factor taken in, 32 k-steps in flight do not fit the registers: 24)
+            // A wave takes a quarter of K in groups of k-steps whose loads are issued together, and
+            // the steps that are left when a group is not full go one at a time: groups of eight
+            // where a quarter of K is fewer than 32 steps, of 32 (with the norm's factor taken in,
+            // which needs registers of its own, 24) otherwise.
+            if (K < 4096)
+                return launch_skinny<1, 1, 8, 4, 2, true, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, fuse);
             return launch_skinny<1, 1, (EPI == 1 ? 24 : 32), 4, 2, true, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, fuse);
         } else {
             return tff_fail("gemm: a gated product does not come before a norm");
         }
     }
-    if (N >= 32 * 1024) return launch_skinny<1, 1, 4, 8, 1, false, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, fuse);
+    // (K up to 1,024: sixteen waves would have two k-steps each, less than a group of four)
+    if (N >= 32 * 1024 || K <= 1024)
+        return launch_skinny<1, 1, 4, 8, 1, false, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, fuse);
     if (K >= 8192 || N <= 4096)
         return launch_skinny<1, 1, 4, 16, 1, false, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, fuse);
     return launch_skinny<1, 1, 8, 4, 1, false, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, fuse);

@@ -121,8 +121,40 @@ def _scratch_users(remarks: str) -> dict[str, int]:
     return out
 
 
-def build(verbose: bool = True) -> str:
-    """Compiles every source for gfx950 and links the library; returns its path."""
+def _masked_mfma(asm: str) -> dict[str, int]:
+    """Kernels of a device assembly listing in which an MFMA stands under a mask of lanes with no
+    branch round it: name -> number of such places.  Where the compiler takes a condition to
+    differ between lanes it may, for a short body, only narrow the mask of active lanes and run
+    the body (s_and_saveexec without an s_cbranch_execz).  An MFMA does not look at that mask: it
+    runs for the whole wave and accumulates what the condition was meant to keep out.  The cure is
+    a condition that is a scalar in the compiler's eyes (values derived from the wave's number
+    go through readfirstlane)."""
+    out: dict[str, int] = {}
+    name, masked = None, False
+    for ln in asm.splitlines():
+        m = re.match(r"^(\S+):\s+; @", ln)
+        if m:
+            name, masked = m.group(1), False
+            continue
+        t = ln.strip()
+        if name is None or not t:
+            continue
+        if re.match(r"s_\w+_saveexec_b64", t):
+            masked = True
+        elif masked:
+            if t.startswith("s_cbranch_exec") or re.match(r"s_\w+_b64 exec,", t):
+                masked = False      # the body is skipped when no lane is on, or the mask is restored
+            elif t.startswith("v_mfma") or t.startswith("v_smfma"):
+                out[name] = out.get(name, 0) + 1
+                masked = False
+    return out
+
+
+def build(verbose: bool = True, check_masks: bool = False) -> str:
+    """Compiles every source for gfx950 and links the library; returns its path.
+    check_masks: also lists the device assembly of the sources that use the matrix cores and
+    fails if an MFMA stands under a mask of lanes (see _masked_mfma); it runs beside the
+    compilation and takes as long as the longest source."""
     hipcc = _hipcc()
     out_dir = next((d for d in lib_dirs() if _writable(d)), None)
     if out_dir is None:
@@ -153,13 +185,35 @@ def build(verbose: bool = True) -> str:
         say(f"compiled {os.path.basename(src)} ({time.time() - t0:.0f} s)")
         return obj
 
+    masked: dict[str, int] = {}
+
+    def list_one(src):
+        flags = [f for f in HIPCC_FLAGS if not f.startswith("-Rpass")]
+        p = subprocess.run([hipcc, *flags, "-I", CSRC_DIR, "-S", "--cuda-device-only", src, "-o", "-"],
+                           capture_output=True, text=True)
+        if p.returncode != 0:
+            raise BuildError(f"hipcc -S failed on {os.path.basename(src)}:\n{p.stderr[-4000:]}")
+        masked.update(_masked_mfma(p.stdout))
+        say(f"checked the MFMAs of {os.path.basename(src)} ({time.time() - t0:.0f} s)")
+
+    def uses_mfma(src):
+        with open(src) as f:
+            return "mfma" in f.read()
+
     say(f"compiling {len(sources)} files for gfx950 into {out_dir}")
     th = threading.Thread(target=ticker, daemon=True)
     th.start()
     try:
-        workers = max(1, min(len(sources), int(os.environ.get("MAX_JOBS", "8")), 16))
+        listed = [s for s in sources if uses_mfma(s)] if check_masks else []
+        workers = max(1, min(len(sources) + len(listed), int(os.environ.get("MAX_JOBS", "8")), 16))
         with ThreadPoolExecutor(workers) as pool:
+            checks = [pool.submit(list_one, s) for s in listed]
             objs = list(pool.map(compile_one, sources))
+            for c in checks:
+                c.result()
+        if masked:
+            raise BuildError("an MFMA under a mask of lanes, which it does not look at (make its condition a "
+                             "scalar): " + ", ".join(f"{k} ({v})" for k, v in sorted(masked.items())))
         tmp_lib = os.path.join(out_dir, f".{LIB_NAME}.{os.getpid()}")
         cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp_lib]
         p = subprocess.run(cmd, capture_output=True, text=True)
@@ -167,7 +221,10 @@ def build(verbose: bool = True) -> str:
             raise BuildError(f"link failed:\n{p.stderr[-4000:]}")
         os.replace(tmp_lib, os.path.join(out_dir, LIB_NAME))
         with open(os.path.join(out_dir, "build_info.json"), "w") as f:
-            json.dump({"digest": source_digest(), "flags": HIPCC_FLAGS, "scratch_bytes_per_lane": scratch}, f, indent=1)
+            info = {"digest": source_digest(), "flags": HIPCC_FLAGS, "scratch_bytes_per_lane": scratch}
+            if check_masks:
+                info["mfma_under_lane_mask"] = masked
+            json.dump(info, f, indent=1)
     finally:
         done.set()
     for name, n in sorted(scratch.items()):
