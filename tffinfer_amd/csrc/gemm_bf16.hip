@@ -1148,15 +1148,15 @@ TFF_API int tff_gemm_plan(int M, int N, int K, int glu, int keep_partials, int* 
     return 0;
 }
 
-// Up to 16 rows: which streaming kernel.  Gated: with a thousand row groups and more a wave takes
-// a group's whole K through a ring.  Plain: more waves per block where there are few blocks
+// Up to 16 rows: which streaming kernel.  Gated: with 512 row groups and more a wave takes
+// a group's whole K through a ring (384 such waves, at N = 6,144, are too few: 3 % slower).  Plain: more waves per block where there are few blocks
 // (small N) or long rows (large K), fewer and deeper ones in between.
 template <int EPI>
 static int skinny_for(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda, int c_dtype,
                       int glu_out, hipStream_t s, const SkinnyFuse* fuse) {
     if (glu_out > 0) {
         if constexpr (EPI != 2) {
-            if (N >= 16 * 1024)
+            if (N >= 8 * 1024)
                 return launch_skinny<1, 1, 8, 1, 2, true, true, EPI>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, fuse);
             // A wave takes a quarter of K in groups of k-steps whose loads are issued together, and
             // the steps that are left when a group is not full go one at a time: groups of eight
