@@ -1215,7 +1215,7 @@ def test_attention_mfma_blocks_scores_that_creep_up():
 
 
 @pytest.mark.parametrize("M", [1, 8, 20, 50, 200])
-@pytest.mark.parametrize("I,K", [(200, 96), (64, 64), (1000, 256), (12288, 512), (8200, 104)])
+@pytest.mark.parametrize("I,K", [(200, 96), (64, 64), (1000, 256), (12288, 512), (8200, 104), (4100, 1000), (3000, 2080)])
 def test_linear_with_gated_epilogue(M, I, K):
     """Gate and up interleaved in one weight: the product yields silu(x Wg^T) * (x Wu^T)."""
     ops = _ops()
