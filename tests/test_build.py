@@ -67,7 +67,7 @@ def test_an_mfma_under_a_lane_mask_is_found_in_a_listing():
 
 
 def test_the_built_library_has_no_mfma_under_a_lane_mask():
-    """Of the library in the tree, if its build listed the assembly (the entry point's build does)."""
+    """Of the library in the tree, if its build listed the assembly (every build does unless told not to)."""
     import pytest
     lib = build.find_library()
     if lib is None:

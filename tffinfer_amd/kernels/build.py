@@ -150,10 +150,11 @@ def _masked_mfma(asm: str) -> dict[str, int]:
     return out
 
 
-def build(verbose: bool = True, check_masks: bool = False) -> str:
+def build(verbose: bool = True, check_masks: bool = True) -> str:
     """Compiles every source for gfx950 and links the library; returns its path.
     check_masks: also lists the device assembly of the sources that use the matrix cores and
-    fails if an MFMA stands under a mask of lanes (see _masked_mfma); it runs beside the
+    fails if an MFMA stands under a mask of lanes (see _masked_mfma): what the compiler makes of
+    a condition is its choice, and another version may choose otherwise.  It runs beside the
     compilation and takes as long as the longest source."""
     hipcc = _hipcc()
     out_dir = next((d for d in lib_dirs() if _writable(d)), None)
