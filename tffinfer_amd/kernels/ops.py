@@ -575,10 +575,13 @@ def _pick_block_cols(batch, G: int, nkv: int, window: int, device, which: str, h
     return cache[key]
 
 
-#: entries x kv heads from which a decode step gives every pair a block of eight waves: a CU
-#: with two waves to a SIMD streams some 45 GB/s (what bounds a wave is the instructions of a step of 32
-#: keys, not memory), 256 of them twice what HBM gives
-BLOCK_DECODE_MIN_PAIRS = 256
+#: entries x kv heads from which a decode step gives every pair a block of eight waves that
+#: split its keys and merge in LDS, instead of splitting the keys over blocks of one wave and
+#: merging in a second kernel.  A block a pair keeps only as many CUs busy as there are pairs, and
+#: eight waves do not pull a CU's share of HBM alone: measured at the 8B shape (eight kv heads),
+#: 128 pairs are 1 % (2,048 cached tokens) to 11 % (32,768) slower as blocks, 160 pairs and more
+#: 3 to 7 % faster at every length.
+BLOCK_DECODE_MIN_PAIRS = 160
 
 
 def pick_splits(waves: int, max_context: int) -> int:
