@@ -217,12 +217,14 @@ __global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
     }
     if (SPLIT) {
         // The launch is sized for the longest context the engine allows; with shorter ones a run
-        // of keys is not made shorter than 256 keys as long as some 512 waves are left with
-        // work (the other waves of the launch end at once; their partial results are empty):
-        // runs of 128 keys were 7 % slower at 8 requests of 2,048 tokens.
-        const int busy = (512 + (int)(gridDim.x * gridDim.y) - 1) / (int)(gridDim.x * gridDim.y);
+        // of keys is not made shorter than 256 keys as long as some 256 waves are left with
+        // work (the other waves of the launch end at once; their partial results are empty), and
+        // never shorter than 128: runs of 128 keys were 7 % slower at 8 requests of 2,048 tokens
+        // and 2 % at 4, and one request's 22 runs of 96 keys 2 % of the step slower than 16 of 128
+        // (up to 16 partial results the merge fetches in one go).
+        const int busy = (256 + (int)(gridDim.x * gridDim.y) - 1) / (int)(gridDim.x * gridDim.y);
         const int per = max(max((nsteps + (int)gridDim.z - 1) / (int)gridDim.z, min(8, (nsteps + busy - 1) / busy)),
-                            min(3, nsteps));   // (and never under 96 keys: more partial results cost more than they gain)
+                            min(4, nsteps));
         s_begin = min(nsteps, (int)blockIdx.z * per);
         s_end = min(nsteps, s_begin + per);
     }
