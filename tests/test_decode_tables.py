@@ -187,3 +187,27 @@ def test_lives_are_unique():
             seen.add(cache.life(rid))
         cache.release("x")
         cache.release("y")
+
+
+def test_half_way_buckets_wait_for_their_capture_until_they_are_popular():
+    """A decode step runs in the smallest bucket that holds it; where a graph of less than twice
+    that bucket's rows exists already, it stands in until the bucket has been wanted often."""
+    from types import SimpleNamespace
+    from tffinfer_amd.engine.runner import ModelRunner
+    assert graph_buckets(64) == [1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64]
+    assert graph_buckets(20) == [1, 2, 3, 4, 6, 8, 12, 16, 20] and graph_buckets(1) == [1]
+    r = SimpleNamespace(_graph_buckets=graph_buckets(64), _graphs={}, _graph_wanted={},
+                        CAPTURE_AFTER=ModelRunner.CAPTURE_AFTER)
+    pick = lambda n: ModelRunner._pick_bucket(r, n)
+    assert pick(32) == 32                      # nothing captured yet: its own bucket, now
+    r._graphs[32] = object()
+    assert pick(20) == 32 and pick(17) == 32   # 24 is wanted, 32 stands in
+    assert pick(16) == 16                      # 32 is twice 16: no stand-in
+    r._graphs[16] = object()
+    assert pick(12) == 16                      # 16 < 2 * 12 stands in for 12
+    assert pick(5) == 6                        # 16 and 32 are more than twice 6
+    for _ in range(ModelRunner.CAPTURE_AFTER - 3):
+        assert pick(24) == 32
+    assert pick(24) == 24                      # wanted often enough: captured now
+    r._graphs[24] = object()
+    assert pick(17) == 24 and r._graph_wanted[24] == ModelRunner.CAPTURE_AFTER

@@ -217,3 +217,32 @@ def test_command_line(model_dirs):
     p = subprocess.run([sys.executable, "-m", "tffinfer_amd", d, "--load-only"], capture_output=True, text=True,
                        timeout=300, cwd=ROOT)
     assert p.returncode == 0 and "loaded" in p.stderr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_warm_up_captures_every_decode_graph_beforehand(model_dirs, dtype):
+    """An engine that was warmed up has the graph of every batch size and captures none while it
+    works; its tokens are those of an engine that captures as it goes.  The latter lets a larger
+    graph stand in for a half-way bucket that is wanted only in passing."""
+    from tffinfer_amd import EngineOptions, LLMEngine
+    d = model_dirs["A"]
+    V = read_config(d)["vocab_size"]
+    prompts = [random_tokens(n, V, 400 + n) for n in (5, 9, 4, 12, 7, 3)]
+    lens = [20, 6, 14, 9, 17, 11]
+    outs = []
+    for warm in (False, True):
+        eng = LLMEngine.from_model_dir(d, EngineOptions(dtype=dtype, page_size=8, kv_tokens=512, max_num_seqs=6))
+        assert eng.runner._graph_buckets == [1, 2, 3, 4, 6]
+        if warm:
+            assert eng.warm_up() == 5 and eng.warm_up() == 0
+        for i, (p, n) in enumerate(zip(prompts, lens)):
+            eng.add_request(p, max_new_tokens=n, ignore_eos=True, request_id=i)
+        while eng.has_work:
+            eng.step()
+        outs.append([eng.pop_result(i).output for i in range(6)])
+        captured = sorted(eng.runner._graphs)
+        if warm:
+            assert captured == [1, 2, 3, 4, 6]
+        else:
+            assert captured == [1, 3, 6]      # 6 stood in for 4 and 3 for 2, which were wanted for a few steps only
+    assert outs[0] == outs[1]

@@ -77,6 +77,8 @@ def build_parser() -> argparse.ArgumentParser:
                    help="token budget of a step")
     g.add_argument("--prefill-chunk", type=int, default=512, help="longest portion of a prompt in a step")
     g.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
+    g.add_argument("--warm-up", action="store_true",
+                   help="capture the decode graphs of all batch sizes before the first request")
     g = ap.add_argument_group("output")
     g.add_argument("--json", action="store_true", help="print one JSON object per prompt")
     g.add_argument("--dump-logits", metavar="FILE",
@@ -122,7 +124,7 @@ def _bench(args, rt, cfg) -> int:
         kv_tokens, chunk = args.context + args.page_size, args.context
     opt = EngineOptions(dtype=model.dtype, page_size=args.page_size, max_num_seqs=max(1, args.batch),
                         max_num_batched_tokens=max(4096, args.batch, chunk), prefill_chunk=chunk,
-                        max_model_len=mc.max_position_embeddings, use_graphs=not args.no_graphs,
+                        max_model_len=mc.max_position_embeddings, use_graphs=not args.no_graphs, warm_up=args.warm_up,
                         kv_tokens=None if (args.num_pages or args.kv_bytes) else kv_tokens,
                         num_pages=args.num_pages, kv_bytes=args.kv_bytes)
     engine = LLMEngine(model, opt)
@@ -183,6 +185,7 @@ def main(argv=None) -> int:
     cfg._num_pages = args.num_pages
     cfg._kv_bytes = args.kv_bytes
     cfg._use_graphs = not args.no_graphs
+    cfg._warm_up = args.warm_up
     stype = args.sample_type
     if stype == "greedy" and (args.temperature != 1.0 or args.top_k or args.top_p < 1 or args.min_p > 0):
         stype = "random"   # sampling options without a type mean a random draw

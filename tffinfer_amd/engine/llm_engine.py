@@ -43,6 +43,9 @@ class EngineOptions:
     use_graphs: bool = True
     #: launch a decode step before the host has read the tokens of the one before it
     run_ahead: bool = True
+    #: capture the decode graphs of all batch sizes when the engine is made (some 50 ms each)
+    #: instead of at the first step that wants one
+    warm_up: bool = False
 
 
 @dataclass
@@ -105,6 +108,8 @@ class LLMEngine:
         self._requests: dict = {}
         self._ahead: _Launched | None = None   # a decode step launched ahead of its predecessor's tokens
         self.steps_ahead = 0                   # how many steps were launched that way
+        if opt.warm_up:
+            self.warm_up()
 
     @classmethod
     def from_model_dir(cls, model_dir: str, options: EngineOptions | None = None) -> "LLMEngine":
@@ -132,6 +137,11 @@ class LLMEngine:
             return max(1, num_pages)
         fit = int(free * opt.memory_fraction) // per_page
         return max(1, min(num_pages, fit))
+
+    def warm_up(self) -> int:
+        """What a server does before it takes requests: the decode graphs of all batch sizes are
+        captured now and not at the first step that wants one.  Returns the number of captures."""
+        return self.runner.capture_graphs()
 
     # ---- requests --------------------------------------------------------
     def add_request(self, prompt_ids, sampling: SamplingConfig | None = None, max_new_tokens: int = 64,

@@ -83,6 +83,7 @@ class ModelRunner:
         self._pinned = PinnedTables()     # the tables of steps that run eagerly leave through it
         # decode-only steps replay HIP graphs of the pieces of the model that can be captured
         self._graphs = {}
+        self._graph_wanted = {}         # bucket -> steps that would have run in it had it been captured
         self._graph_buckets = graph_buckets(max_seqs) if (self.use_graphs and model.graph_pieces()) else []
 
     # ---- requests --------------------------------------------------------
@@ -163,11 +164,43 @@ class ModelRunner:
             self.cache.commit(e.req, len(e.tokens))
         return logits
 
+    #: steps a bucket has to be wanted for before it is captured while a graph of less than twice
+    #: its rows can stand in: a capture holds the device up for some 60 ms, which the rows saved
+    #: (a few percent of a step) pay back over a few hundred steps
+    CAPTURE_AFTER = 64
+
+    def _pick_bucket(self, R: int) -> int:
+        """The bucket a decode step of R requests runs in: the smallest that holds it, if its
+        graph exists or no existing graph of less than twice its rows can stand in for it
+        (then it is captured now); otherwise that stand-in, until the smaller bucket has been
+        wanted often enough to be worth its capture.  A batch that shrinks request by request
+        passes through every size once and should not stop for a capture at each."""
+        want = next(b for b in self._graph_buckets if b >= R)
+        if want in self._graphs:
+            return want
+        have = min((b for b in self._graphs if want < b < 2 * want), default=None)
+        if have is None:
+            return want
+        n = self._graph_wanted[want] = self._graph_wanted.get(want, 0) + 1
+        return want if n >= self.CAPTURE_AFTER else have
+
+    def capture_graphs(self) -> int:
+        """Captures the decode graph of every bucket that has none yet (some 50 ms each), so that
+        no step stops for a capture later; returns how many it captured."""
+        n = 0
+        with torch.cuda.device(self.device):
+            for bucket in self._graph_buckets:
+                if bucket not in self._graphs:
+                    g = self._graphs[bucket] = DecodeGraph(self, bucket)
+                    g.capture()
+                    n += 1
+        return n
+
     def _step_graph(self, entries, token_source=None) -> torch.Tensor:
         """A decode-only step through the HIP graph of its batch size bucket.
         The logits live in a tensor the next such step overwrites."""
         R = len(entries)
-        bucket = next(b for b in self._graph_buckets if b >= R)
+        bucket = self._pick_bucket(R)
         with torch.cuda.device(self.device):
             g = self._graphs.get(bucket)
             if g is None:

@@ -125,6 +125,7 @@ def measure_mixed(engine, gen, requests: int, vocab: int, new_tokens: int = 256,
                   hi: int = 4096) -> dict:
     """Continuous batching: all requests arrive at once, the scheduler admits them as
     slots and pages allow, cuts prompts into portions and decodes the others beside them."""
+    engine.warm_up()      # (a server's start-up, not its work: the decode graphs of all batch sizes)
     lens = torch.randint(lo, hi + 1, (requests,), generator=gen).tolist()
     for n in lens:
         engine.add_request(random_prompt(gen, n, vocab), max_new_tokens=new_tokens, ignore_eos=True)

@@ -54,6 +54,7 @@ class ModelConfig:
     _num_pages: int | None = None      # pages per group of layers, or
     _kv_bytes: int | None = None       # bytes of device memory for keys and values
     _use_graphs: bool = True
+    _warm_up: bool = False
 
 
 class LLMInferRuntime:
@@ -130,7 +131,7 @@ class LLMInferRuntime:
         opt = EngineOptions(dtype=self._model.dtype, page_size=p._page_size, max_num_seqs=p._max_batches,
                             max_num_batched_tokens=p._max_batch_tokens, prefill_chunk=p._prefill_chunk,
                             max_model_len=p._n_ctx, kv_tokens=p._kv_tokens, num_pages=p._num_pages,
-                            kv_bytes=p._kv_bytes, use_graphs=p._use_graphs)
+                            kv_bytes=p._kv_bytes, use_graphs=p._use_graphs, warm_up=p._warm_up)
         self._engine = LLMEngine(self._model, opt)
         return True
 
