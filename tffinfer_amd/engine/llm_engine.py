@@ -9,8 +9,10 @@ from __future__ import annotations
 import itertools
 from dataclasses import dataclass, field
 
+import numpy as np
 import torch
 
+from ..kernels import staging as _staging
 from ..models import load_model
 from ..sampling import Sampler, SamplingConfig, SeenTokens
 from .batch import StepEntry
@@ -141,7 +143,21 @@ class LLMEngine:
     def warm_up(self) -> int:
         """What a server does before it takes requests: the decode graphs of all batch sizes are
         captured now and not at the first step that wants one.  Returns the number of captures."""
-        return self.runner.capture_graphs()
+        n = self.runner.capture_graphs()
+        # torch loads a kernel's code when it is first launched (the row selection below took
+        # 0.2 s once): the one torch kernel of the decode loop is launched here, on nothing
+        dev = self.model.device
+        if torch.device(dev).type == "cuda":
+            self._take_rows(torch.zeros(2, dtype=torch.int32, device=dev), np.zeros(1, dtype=np.int32))
+            torch.cuda.synchronize(dev)
+        return n
+
+    @staticmethod
+    def _take_rows(tokens: torch.Tensor, keep: np.ndarray) -> torch.Tensor:
+        """tokens[keep] on the device; the indices go through pinned memory without a wait (a copy
+        from pageable memory would hold the host until the step in flight has ended, and the
+        device idle for as long afterwards)."""
+        return torch.index_select(tokens, 0, _staging.send(tokens.device, [keep])[0])
 
     # ---- requests --------------------------------------------------------
     def add_request(self, prompt_ids, sampling: SamplingConfig | None = None, max_new_tokens: int = 64,
@@ -295,8 +311,9 @@ class LLMEngine:
         if nxt is not None:
             src = st.tokens
             if len(nxt) != len(st.rows):          # some requests end with the token in flight
-                keep = [i for i, r in enumerate(st.rows) if any(p.request is r for p in nxt)]
-                src = st.tokens[torch.tensor(keep, device=st.tokens.device)]
+                going = {id(p.request) for p in nxt}
+                src = self._take_rows(st.tokens, np.asarray([i for i, r in enumerate(st.rows) if id(r) in going],
+                                                            dtype=np.int32))
             self._ahead = self._launch(nxt, src)
             self.steps_ahead += 1
         return dropped + self._complete(st)
