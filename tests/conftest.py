@@ -27,3 +27,12 @@ def _seeded():
     import torch
     torch.manual_seed(1234)
     yield
+
+
+def pytest_terminal_summary(terminalreporter):
+    from helpers import WORST, _TOL
+    if WORST:
+        terminalreporter.write_line("worst error against the plain implementation / tolerance, per configuration:")
+        for (dtype, name), err in sorted(WORST.items()):
+            t = _TOL.get(dtype, {}).get(name)
+            terminalreporter.write_line(f"  {dtype:9s} {name:6s} {err:.2e}" + (f" / {t:.1e}" if t else ""))

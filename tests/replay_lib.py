@@ -10,7 +10,7 @@ import sys
 import numpy as np
 import torch
 
-from helpers import oracle_logits, rel_err
+from helpers import note_error, oracle_logits, rel_err
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CHUNK_CYCLE = [7, 2, 13, 3, 2, 24, 5, 2, 16, 9]
@@ -151,7 +151,7 @@ def run_steps_subprocess(model_dir, dtype, steps, out_dir, max_tokens, extra_arg
     return out
 
 
-def check_against_oracle(model_dir, requests, steps, results, tol) -> float:
+def check_against_oracle(model_dir, requests, steps, results, tol, dtype: str | None = None) -> float:
     """Every wanted row must match the plain implementation's logits at that
     request's position.  Returns the largest relative error; on a failure names
     the first wrong token."""
@@ -174,4 +174,6 @@ def check_against_oracle(model_dir, requests, steps, results, tol) -> float:
             done[rid] += len(e["tokens"])
         if s["step"] in results:
             assert row == results[s["step"]].shape[0]
+    if dtype is not None:
+        note_error(dtype, model_dir, worst)
     return worst

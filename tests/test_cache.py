@@ -166,3 +166,86 @@ def test_random_orders_keep_the_books(seed):
         c.release(r)
     c.check()
     assert all(g.pool.num_used == 0 for g in c.groups) and c.slots.num_free == 5
+
+
+def test_rollback_gives_back_what_no_commit_filled():
+    c = CacheManager([(0, True, FULL, None), (1, True, WIN, None)], 8, {FULL: 12, WIN: 8}, 2)
+    c.add_request("r")
+    c.reserve("r", 13)
+    c.commit("r", 13)
+    held = [list(c.block_table(g, "r")) for g in range(2)]
+    used = [g.pool.num_used for g in c.groups]
+    c.reserve("r", 30)                       # a step that then fails
+    assert c.groups[0].pool.num_used == 6
+    assert c.rollback("r") == 2 * 4
+    assert [list(c.block_table(g, "r")) for g in range(2)] == held
+    assert [g.pool.num_used for g in c.groups] == used and c.num_tokens("r") == 13
+    assert c.rollback("r") == 0              # nothing left to give back
+    c.check()
+    c.reserve("r", 3)                        # fits the page it has: nothing taken, nothing to roll back
+    assert c.rollback("r") == 0
+    c.commit("r", 3)
+    c.release("r")
+    c.check()
+
+
+def test_padding_slot_is_no_requests_slot():
+    c = CacheManager([(0, True, FULL, None), (1, True, None, StateSpec((4,)))], 8, 4, 3)
+    slots = [c.add_request(i) for i in range(3)]
+    assert c.padding_slot not in slots and sorted(slots) == [0, 1, 2]
+    import torch
+    c2 = CacheManager([(0, True, FULL, None), (1, True, None, StateSpec((4,)))], 8, 4, 3, dtype=torch.float32,
+                      device="cpu")
+    assert c2.state_tensors[1].shape == (4, 4)      # a row more than there are requests
+
+
+def test_window_pool_never_runs_short():
+    """A group with a window, sized by window_pool_pages, serves any schedule of portions that
+    keeps to the token budget, however long the requests grow."""
+    from tffinfer_amd.cache.sizing import window_pool_pages
+    rng = random.Random(5)
+    ps, window, seqs, budget = 8, 24, 4, 64
+    n = window_pool_pages(window, ps, seqs, budget)
+    c = CacheManager([(0, True, WIN, None)], ps, n, seqs)
+    for r in range(seqs):
+        c.add_request(r)
+    for _ in range(300):
+        left = budget
+        portions = {}
+        for r in range(seqs):
+            k = rng.choice([0, 1, 1, 2, 7, 30, 64])
+            k = min(k, left)
+            if k:
+                portions[r] = k
+                left -= k
+        for r, k in portions.items():
+            c.reserve(r, k)                  # never raises OutOfPages
+        for r, k in portions.items():
+            c.commit(r, k)
+        c.check()
+    assert max(c.num_tokens(r) for r in range(seqs)) > 50 * ps
+
+
+def test_plan_pages_sizes_groups_by_their_need():
+    from tffinfer_amd.cache.sizing import bytes_per_page, plan_pages, state_bytes, window_pool_pages
+    import torch
+    reqs = [(0, True, FULL, None), (1, True, WIN, None), (2, True, WIN, None), (3, True, None, StateSpec((100,), torch.float32))]
+    ps, seqs, budget = 8, 4, 64
+    pages = plan_pages(reqs, ps, 2, seqs, budget, tokens=4000)
+    assert pages[FULL] == 500 + seqs
+    assert pages[WIN] == window_pool_pages(24, ps, seqs, budget) < 40
+    # bytes: the window groups first, the rest to the group that keeps every key
+    per_full, per_win = bytes_per_page(FULL, 1, ps, 2), bytes_per_page(WIN, 2, ps, 2)
+    kv = 100 * per_full + pages[WIN] * per_win + 5
+    by = plan_pages(reqs, ps, 2, seqs, budget, kv_bytes=kv)
+    assert by[WIN] == pages[WIN] and by[FULL] == 100
+    # the free memory caps what the tokens ask for, and the state tensors come off it first
+    assert state_bytes(reqs, seqs) == 5 * 100 * 4
+    capped = plan_pages(reqs, ps, 2, seqs, budget, tokens=4000, free_bytes=kv + state_bytes(reqs, seqs))
+    assert capped[FULL] == 100 and capped[WIN] == pages[WIN]
+    # a request's short cache never asks a window group for more than the group that keeps all
+    small = plan_pages(reqs, ps, 2, seqs, budget, tokens=40)
+    assert small[FULL] == 5 + seqs and small[WIN] == small[FULL]
+    with pytest.raises(ValueError, match="holds no page"):
+        plan_pages(reqs, ps, 2, seqs, budget, kv_bytes=10)
+    assert plan_pages([(0, True, None, None)], ps, 2, seqs, budget, tokens=10) == {}

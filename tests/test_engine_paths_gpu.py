@@ -244,3 +244,72 @@ def test_random_workloads_on_small_pools(model_dirs, name, dtype, seed):
         check_choices(d, res, dtype, r["sampling"])
     assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
     assert eng.runner.cache.slots.num_free == slots
+
+
+@pytest.mark.parametrize("use_graphs", [False, True])
+def test_a_step_that_fails_gives_its_pages_back(model_dirs, use_graphs, monkeypatch):
+    """A step that raises after its pages were taken (a kernel that refuses its operands, memory
+    that runs out) leaves the cache as it found it: the pages go back, the requests keep their
+    counts, and the same step runs afterwards as if nothing had happened."""
+    from tffinfer_amd.engine import ModelRunner, StepEntry
+    from tffinfer_amd.engine.graphs import DecodeGraph
+    from tffinfer_amd.kernels import lib, ops
+    from tffinfer_amd.models import load_model
+    from helpers import rel_err, tol
+    d = model_dirs["A"]
+    V = read_config(d)["vocab_size"]
+
+    class Failing:
+        armed = 0
+
+        def __getattr__(self, name):
+            real = getattr(ops, name)
+            if name != "linear":
+                return real
+
+            def linear(*a, **kw):
+                if self.armed:
+                    self.armed -= 1
+                    if self.armed == 0:
+                        raise lib.KernelError("made to fail")
+                return real(*a, **kw)
+            return linear
+
+    stub = Failing()
+    model = load_model(d, torch.float32, "cuda:0")
+    rn = ModelRunner(model, page_size=8, num_pages=12, max_seqs=2, max_model_len=96, use_graphs=use_graphs, ops=stub)
+    a, b = random_tokens(40, V, 501), random_tokens(12, V, 502)
+    ref_a, ref_b = oracle_logits(d, a), oracle_logits(d, b)
+    rn.add_request("a")
+    rn.add_request("b")
+    rn.step([StepEntry("a", a[:5], [])])
+    used = [g.pool.num_used for g in rn.cache.groups]
+    stub.armed = 3                                          # the third product of the step raises
+    with pytest.raises(lib.KernelError, match="made to fail"):
+        rn.step([StepEntry("a", a[5:32], [26]), StepEntry("b", b[:11], [10])])
+    assert [g.pool.num_used for g in rn.cache.groups] == used
+    assert rn.cache.num_tokens("a") == 5 and rn.cache.num_tokens("b") == 0
+    rn.cache.check()
+    out = rn.step([StepEntry("a", a[5:32], [26]), StepEntry("b", b[:11], [10])])
+    assert rel_err(out[0], ref_a[31]) <= tol("float32", "A") and rel_err(out[1], ref_b[10]) <= tol("float32", "A")
+    # a decode step (through the graph, where there is one) that fails before anything ran
+    used = [g.pool.num_used for g in rn.cache.groups]
+    if use_graphs:
+        inner = DecodeGraph.run
+        state = {"fail": True}
+
+        def run(self, entries, token_source=None):
+            if state.pop("fail", False):
+                raise RuntimeError("made to fail")
+            return inner(self, entries, token_source)
+        monkeypatch.setattr(DecodeGraph, "run", run)
+    else:
+        stub.armed = 2
+    with pytest.raises((RuntimeError, lib.KernelError), match="made to fail"):
+        rn.step([StepEntry("a", [a[32]], [0]), StepEntry("b", [b[11]], [0])])      # a's token opens a new page
+    assert [g.pool.num_used for g in rn.cache.groups] == used and rn.cache.num_tokens("a") == 32
+    out = rn.step([StepEntry("a", [a[32]], [0]), StepEntry("b", [b[11]], [0])])
+    assert rel_err(out[0], ref_a[32]) <= tol("float32", "A") and rel_err(out[1], ref_b[11]) <= tol("float32", "A")
+    rn.free_request("a")
+    rn.free_request("b")
+    assert all(g.pool.num_used == 0 for g in rn.cache.groups)

@@ -7,7 +7,7 @@ import sys
 import pytest
 import torch
 
-from helpers import tol, oracle_logits, random_tokens, read_config, rel_err
+from helpers import note_error, tol, oracle_logits, random_tokens, read_config, rel_err
 from plain_qwen3 import plain_greedy, plain_inverse_cdf, plain_probs
 
 pytestmark = pytest.mark.gpu
@@ -31,7 +31,9 @@ def check_choices(model_dir, result, dtype, sampling=None):
     assert len(result.logits) == len(result.output)
     for i, (row, tok) in enumerate(zip(result.logits, result.output)):
         pos = len(result.prompt) + i - 1
-        assert rel_err(row, ref[pos]) <= tol(dtype, model_dir), f"output {i}"
+        err = rel_err(row, ref[pos])
+        note_error(dtype, model_dir, err)
+        assert err <= tol(dtype, model_dir), f"output {i}: {err:.3e}"
         if sampling is None or sampling.greedy:
             assert tok == plain_greedy(row)
         else:

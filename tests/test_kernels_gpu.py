@@ -182,7 +182,9 @@ def test_norm_taken_into_the_products_on_either_side(M, H, K, N2, glu):
     _close(y, ref, 1.2e-2, "product after the norm")
     for m in range(M):     # row by row: a row's factor is its own
         _close(y[m], ref[m], 1.5e-2, f"row {m}")
-    _close(rows.materialize(), normed, 8e-3, "normalised rows written out")
+    # written out for a consumer that is no such product: rounded to bfloat16 once (2^-9 of an element)
+    out = rows.materialize().double().cpu()
+    assert float(((out - normed).abs() / normed.abs().clamp_min(1e-3)).max()) <= 2.0 ** -8
     # the same through the separate kernels, to rounding
     r2 = resid.to(DEV).clone()
     z = ops.add_rmsnorm(r2, pending.run(), nw.to(DEV), eps, torch.bfloat16)

@@ -1,0 +1,102 @@
+"""Decode steps of twenty and more requests through the engine, against the plain
+implementation: the schedules that large batches take and small ones never reach.
+
+With eight kv heads, twenty requests are 160 (request, kv head) pairs, from which on a decode
+step gives every pair a block of waves of its own instead of splitting the keys over blocks and
+merging in a second kernel; products of 17 to 64 rows run on tiles whose blocks split K, with
+their partial sums added up by the norm that follows or by a kernel of their own; and the batch
+shrinks through the graph buckets 28, 24, 16, 12, 8, ... with a larger graph standing in for a
+smaller one on the way.  All of that runs inside captured HIP graphs with padding rows and with
+steps launched ahead.  Every kept row of logits is compared with the plain logits of the
+request's own sequence and every token with the plain sampler's choice from that row
+(``check_choices``).
+"""
+import pytest
+import torch
+
+from helpers import random_tokens, read_config
+from test_engine_paths_gpu import drive
+from test_generate_gpu import check_choices
+
+pytestmark = pytest.mark.gpu
+
+
+def _watch(monkeypatch):
+    """Records what the decode attention and the products were asked for."""
+    from tffinfer_amd.kernels import ops
+    seen = {"pairs": set(), "split_rows": set(), "stacks": set()}
+    inner_attn, inner_linear = ops.attention_decode_fused, ops.linear
+
+    def attn(qkv, nq, nkv, *a, **kw):
+        seen["pairs"].add(qkv.shape[0] * nkv)
+        return inner_attn(qkv, nq, nkv, *a, **kw)
+
+    def linear(x, weight, *a, **kw):
+        out = inner_linear(x, weight, *a, **kw)
+        if isinstance(out, torch.Tensor) and out.dim() == 3:
+            seen["stacks"].add((out.shape[1], out.shape[0]))     # (rows, parts of K kept for the norm)
+        return out
+
+    monkeypatch.setattr(ops, "attention_decode_fused", attn)
+    monkeypatch.setattr(ops, "linear", linear)
+    return seen
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,page_size", [("E", 16), ("W", 16), ("W", 64), ("W", 128)])
+def test_twenty_eight_requests_shrinking_through_the_graph_buckets(model_dirs, name, page_size, dtype, monkeypatch):
+    from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
+    from tffinfer_amd.engine.runner import ModelRunner
+    from tffinfer_amd.kernels import ops
+    d = model_dirs[name]
+    cfg = read_config(d)
+    V, nkv = cfg["vocab_size"], cfg["num_key_value_heads"]
+    n = 28
+    seen = _watch(monkeypatch)
+    # a smaller bucket's graph is captured after it has been wanted three times; until then a
+    # larger one stands in for it
+    monkeypatch.setattr(ModelRunner, "CAPTURE_AFTER", 3)
+    # prompts of 3 .. 140 tokens (pages of 128: some requests cross into a second page while they
+    # decode, most live in a part of one); a request ends after 7 + 3 i tokens, so that the batch
+    # loses one request every third step
+    plens = [3 + (37 * i) % 138 for i in range(n)]
+    news = [7 + 3 * i for i in range(n)]
+    sc = [SamplingConfig("random", temperature=0.9, seed=500 + i) if i % 3 == 1 else SamplingConfig()
+          for i in range(n)]
+    opt = EngineOptions(dtype=dtype, page_size=page_size, kv_tokens=n * 256, max_num_seqs=n,
+                        max_num_batched_tokens=1024, prefill_chunk=256, max_model_len=256,
+                        use_graphs=True, run_ahead=True)
+    eng = LLMEngine.from_model_dir(d, opt)
+    eng.keep_logits = True
+    reqs = [dict(prompt_ids=random_tokens(plens[i], V, 9000 + i), sampling=sc[i], max_new_tokens=news[i],
+                 ignore_eos=True, request_id=i) for i in range(n)]
+    standins = []
+    pick = ModelRunner._pick_bucket
+
+    def picked(self, R):
+        b = pick(self, R)
+        want = next(x for x in self._graph_buckets if x >= R)
+        if b != want:
+            standins.append((R, b))
+        return b
+
+    monkeypatch.setattr(ModelRunner, "_pick_bucket", picked)
+    drive(eng, {0: reqs})
+    graphs = sorted(eng.runner._graphs)
+    print(f"{name} {dtype} pages of {page_size}: {eng.scheduler.stats.steps} steps, {eng.steps_ahead} launched ahead, "
+          f"graphs {graphs}, stand-ins {sorted(set(standins))}, attention pairs {sorted(seen['pairs'])}, "
+          f"kept partial sums (rows, parts) {sorted(seen['stacks'])}")
+    assert eng.steps_ahead > 40
+    assert {28, 24, 16, 12, 8}.issubset(graphs), graphs
+    assert standins, "no graph ever stood in for a smaller one"
+    if dtype == "bfloat16":
+        assert any(p >= ops.BLOCK_DECODE_MIN_PAIRS for p in seen["pairs"]), "no step gave a block to every pair"
+        assert any(p < ops.BLOCK_DECODE_MIN_PAIRS for p in seen["pairs"]), "no step split the keys over blocks"
+        assert any(17 <= rows <= 64 and parts > 1 for rows, parts in seen["stacks"]), \
+            "no product of 17 to 64 rows kept partial sums for the norm"
+    for i in range(n):
+        r = eng.pop_result(i)
+        assert r.finish_reason == "length" and len(r.output) == news[i]
+        check_choices(d, r, dtype, sc[i])
+    assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
+    assert eng.runner.cache.slots.num_free == n

@@ -10,7 +10,8 @@ from helpers import PAGE_SIZE, tol, random_tokens, read_config, rel_err
 pytestmark = pytest.mark.gpu
 
 DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
-LENGTHS = {"A": [1, 9, 40, 100], "B": [3, 17, 31, 64, 100, 150], "C": [2, 33, 70, 129, 200], "D": [5, 41, 90, 160]}
+LENGTHS = {"A": [1, 9, 40, 100], "B": [3, 17, 31, 64, 100, 150], "C": [2, 33, 70, 129, 200], "D": [5, 41, 90, 160],
+           "B0": [3, 17, 31, 64, 100, 150]}
 
 
 def requests_for(name, model_dir):
@@ -26,7 +27,7 @@ def make_runner(model_dir, dtype, page_size, num_pages, max_seqs=8):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "B0"])
 @pytest.mark.parametrize("mode", ["whole", "tail", "chunks", "mixed"])
 def test_replay_modes(model_dirs, name, dtype, mode):
     model_dir = model_dirs[name]
@@ -38,7 +39,7 @@ def test_replay_modes(model_dirs, name, dtype, mode):
     num_pages = rl.max_live_tokens(steps, unit=ps) // ps
     runner = make_runner(model_dir, dtype, ps, num_pages)
     results = rl.run_steps_in_process(runner, steps)
-    worst = rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name))
+    worst = rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name), dtype)
     print(f"{name} {dtype} {mode}: worst rel. error {worst:.3e} over {len(steps)} steps, {num_pages} pages")
     assert all(g.pool.num_used == 0 for g in runner.cache.groups)
 
@@ -55,7 +56,7 @@ def test_replay_with_pages_that_are_no_power_of_two(model_dirs, name, ps, dtype)
     steps = rl.trace_mixed(reqs)
     runner = make_runner(model_dir, dtype, ps, rl.max_live_tokens(steps, unit=ps) // ps)
     results = rl.run_steps_in_process(runner, steps)
-    rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name))
+    rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name), dtype)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -68,11 +69,11 @@ def test_trace_run_program(model_dirs, tmp_path, dtype):
     assert any(not any(e["want"] for e in s["entries"]) for s in steps)
     out = rl.run_steps_subprocess(model_dir, dtype, steps, str(tmp_path / "out"),
                                   rl.max_live_tokens(steps, 64))
-    rl.check_against_oracle(model_dir, reqs, steps, out, tol(dtype, "B"))
+    rl.check_against_oracle(model_dir, reqs, steps, out, tol(dtype, "B"), dtype)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "B0"])
 @pytest.mark.parametrize("mode", ["tail", "mixed"])
 def test_replay_with_decode_graphs(model_dirs, name, dtype, mode):
     """Decode-only steps run as replays of a captured HIP graph: every replay,
@@ -92,11 +93,11 @@ def test_replay_with_decode_graphs(model_dirs, name, dtype, mode):
     assert runner._graphs, "no decode step went through a graph"
     decode_only = sum(1 for s in steps if s["entries"] and all(len(e["tokens"]) == 1 for e in s["entries"]))
     assert decode_only >= 3
-    rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name))
+    rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name), dtype)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])     # (C's and D's head sizes take the decode kernel that writes keys itself)
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "B0"])     # (C's and D's head sizes take the decode kernel that writes keys itself)
 def test_padding_rows_of_a_graph_write_nothing(model_dirs, name, dtype):
     """Three requests decode through the graph of four rows: the fourth row is padding (token 0
     at position 0 with a block table of zeros).  After every step the caches must hold, bit for
@@ -134,7 +135,7 @@ def _all_caches(runner):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,n", [("A", 128), ("B", 256), ("C", 300), ("D", 320)])
+@pytest.mark.parametrize("name,n", [("A", 128), ("B", 256), ("C", 300), ("D", 320), ("B0", 256)])
 @pytest.mark.parametrize("graphs", [False, True])
 def test_long_decoding(model_dirs, name, dtype, n, graphs):
     """A few prompt tokens, then one token a step up to the model's longest
@@ -150,13 +151,13 @@ def test_long_decoding(model_dirs, name, dtype, n, graphs):
     runner = ModelRunner(load_model(model_dir, DTYPES[dtype], "cuda:0"), page_size=ps,
                          num_pages=-(-n // ps), max_seqs=2, use_graphs=graphs)
     results = rl.run_steps_in_process(runner, steps)
-    rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name))
+    rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name), dtype)
     if name in ("B", "D"):   # the window groups gave pages back on the way
         assert any(g.spec.window > 0 for g in runner.cache.groups)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "B0"])
 def test_first_tokens(model_dirs, name, dtype):
     """Sequences of one, two and three tokens: whole, and token by token."""
     model_dir = model_dirs[name]
@@ -165,7 +166,7 @@ def test_first_tokens(model_dirs, name, dtype):
     for steps in (rl.trace_whole(reqs), rl.trace_tail(reqs, tail=3)):
         runner = make_runner(model_dir, dtype, PAGE_SIZE[name], 4)
         results = rl.run_steps_in_process(runner, steps)
-        rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name))
+        rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name), dtype)
 
 
 MID = dict(
@@ -198,7 +199,7 @@ def test_midsize_model_long_prompt(tmp_path_factory, dtype):
     for steps in (whole, parts):
         runner = make_runner(model_dir, dtype, 16, 72, max_seqs=2)
         results = rl.run_steps_in_process(runner, steps)
-        worst = rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, "mid"))
+        worst = rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, "mid"), dtype)
         print(f"mid {dtype}: worst rel. error {worst:.3e}")
 
 

@@ -288,3 +288,46 @@ def test_a_head_of_the_queue_that_fits_nowhere_is_finished_not_raised():
     sched.add_request(b)
     run_all(sched, runner, cache)
     assert b.output == expected_output(b.prompt, 3)
+
+
+def test_window_group_of_the_least_size_runs_under_a_large_budget():
+    """A window of 16 in pages of 8 needs ceil(15 / 8) + 1 = 3 pages to advance by a token.  On
+    exactly that pool a long request is admitted and runs to its end although the token budget
+    would let its portions grow to 64 tokens: portions are cut to what the free pages hold."""
+    from tffinfer_amd.cache.sizing import min_window_pages
+    assert min_window_pages(16, 8) == 3
+    cache, sched, runner = make(num_pages=3, ps=8, max_seqs=1, budget=64, chunk=24, specs=(WIN,))
+    r = Request("w", list(range(90)), max_new_tokens=20)
+    sched.add_request(r)
+    sizes = []
+    run_all(sched, runner, cache, on_step=lambda plan: sizes.append(plan[0].count))
+    assert r.output == expected_output(r.prompt, 20) and sched.stats.preemptions == 0
+    assert max(sizes) <= 3 * 8 and max(sizes) > 1
+    # one page fewer and the request can never advance past its window: refused when added
+    cache, sched, runner = make(num_pages=2, ps=8, max_seqs=1, budget=64, chunk=24, specs=(WIN,))
+    with pytest.raises(RequestRefused, match="cache pages"):
+        sched.add_request(Request("w", list(range(90)), max_new_tokens=20))
+    # a short one that fits its two pages whole is taken
+    sched.add_request(Request("s", list(range(10)), max_new_tokens=5))
+    run_all(sched, runner, cache)
+
+
+def test_window_pool_sized_by_the_engine_never_preempts():
+    """Pools as the engine sizes them: the group that keeps all keys holds every request, the
+    group with a window gets window_pool_pages; four long requests run under a budget that a lone
+    prompt may fill, and nothing is ever preempted for want of a window page."""
+    from tffinfer_amd.cache.sizing import plan_pages
+    ps, seqs, budget = 8, 4, 64
+    reqs_spec = [(0, True, SPEC, None), (1, True, WIN, None)]
+    pages = plan_pages(reqs_spec, ps, 2, seqs, budget, tokens=4 * 200)
+    assert pages[WIN] < pages[SPEC] // 4
+    cache = CacheManager(reqs_spec, ps, pages, seqs)
+    sched = Scheduler(cache, SchedulerOptions(seqs, budget, 24), 512)
+    runner = FakeRunner(cache)
+    reqs = [Request(i, [(3 * i + j) % 60 for j in range(n)], max_new_tokens=40)
+            for i, n in enumerate([150, 90, 30, 120, 77, 140])]
+    for r in reqs:
+        sched.add_request(r)
+    run_all(sched, runner, cache)
+    assert sched.stats.preemptions == 0
+    assert all(r.output == expected_output(r.prompt, 40) for r in reqs)

@@ -259,3 +259,60 @@ def test_a_part_that_cannot_be_captured_splits_the_graph(tmp_path):
         for g in runner._graphs.values():
             assert [pc.graph is not None for pc in g.pieces] == [True, False, True]
         _check(requests, refs, steps, results, mode.__name__ + " with graphs")
+
+
+@pytest.mark.parametrize("use_graphs", [False, True])
+def test_toy_architecture_through_the_engine_with_a_preemption(tmp_path, use_graphs):
+    """The scheduler, the cache manager and the state slots carry a model with per-request state
+    of fixed size: three requests on a pool so small that the newest is preempted while it
+    decodes, when its running mean is long past zero, and is computed again from its first
+    token (its slot is cleared when it comes back).  Every kept row of logits is compared with
+    the hand-written reference on the request's own sequence, and every request's tokens with
+    what the engine gives it alone."""
+    from safetensors.torch import load_file
+    from tffinfer_amd import EngineOptions, LLMEngine
+    from tffinfer_amd.models import load_model
+    from tffinfer_amd.weights import write_random_model
+    ToyConfig = _register()
+    d = write_random_model(str(tmp_path / "toy"), ToyConfig(), seed=79, dtype="float32")
+    raw = load_file(d + "/model.safetensors")
+    model = load_model(d, torch.float32, DEV)
+    prompts = [random_tokens(n, V, 25 + i) for i, n in enumerate([11, 30, 19])]
+    new = [40, 34, 45]
+    opt = EngineOptions(dtype="float32", page_size=8, num_pages=16, max_num_seqs=3, max_num_batched_tokens=32,
+                        prefill_chunk=16, max_model_len=128, use_graphs=use_graphs, run_ahead=True)
+    eng = LLMEngine(model, opt)
+    eng.keep_logits = True
+    preempted_with_state = []
+    inner = eng.scheduler._preempt_last
+
+    def preempt():
+        victim = eng.scheduler.running[-1]
+        slot = eng.runner.cache.slot(victim.id)
+        state = eng.runner.cache.state_tensors[1][slot]
+        preempted_with_state.append((victim.id, victim.num_computed, float(state[-1]), float(state[:-1].abs().max())))
+        return inner()
+
+    eng.scheduler._preempt_last = preempt
+    ids = [eng.add_request(p, max_new_tokens=n, ignore_eos=True) for p, n in zip(prompts, new)]
+    while eng.has_work:
+        eng.step()
+        eng.runner.cache.check()
+    assert eng.scheduler.stats.preemptions > 0, "the pool was meant to run out"
+    # a victim had tokens behind it: a count and a sum that the cleared slot must not keep
+    assert any(count > 0 and biggest > 0 for _, _, count, biggest in preempted_with_state), preempted_with_state
+    results = [eng.pop_result(i) for i in ids]
+    for r, n in zip(results, new):
+        assert len(r.output) == n and r.finish_reason == "length"
+        ref = toy_reference(raw, r.prompt + r.output)
+        for i, (row, tok) in enumerate(zip(r.logits[:n], r.output)):
+            want = ref[len(r.prompt) + i - 1]
+            err = float((row.double() - want).abs().max() / want.abs().max())
+            assert err < 2e-5, f"request {r.id} output {i}: {err:.2e}"
+            assert tok == int(torch.argmax(row))
+    assert any(r.num_preemptions > 0 for r in results)
+    for p, n, r in zip(prompts, new, results):
+        alone = LLMEngine(model, EngineOptions(dtype="float32", page_size=8, num_pages=24, max_num_seqs=1,
+                                               max_model_len=128, use_graphs=use_graphs))
+        assert alone.generate([p], max_new_tokens=n, ignore_eos=True)[0].output == r.output
+    assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)

@@ -104,8 +104,10 @@ class CacheManager:
             for g in self.groups:
                 g.kv = torch.zeros(len(g.cache_ids), 2, g.pool.num_pages, g.spec.num_kv_heads,
                                    self.page_size, g.spec.head_dim, dtype=dtype, device=device)
+            # one row more than there are requests: the row of the padding rows of a decode graph,
+            # which no request ever holds (``padding_slot``)
             for cache_id, st in self._state_specs.items():
-                self.state_tensors[cache_id] = torch.zeros(self.max_seqs, *st.shape, dtype=st.dtype,
+                self.state_tensors[cache_id] = torch.zeros(self.max_seqs + 1, *st.shape, dtype=st.dtype,
                                                            device=device)
 
     # ---- lookups ---------------------------------------------------------
@@ -124,6 +126,13 @@ class CacheManager:
 
     def slot(self, req) -> int:
         return self.requests[req].slot
+
+    @property
+    def padding_slot(self) -> int:
+        """The state slot of rows that stand for no request (the padding rows of a decode
+        graph): a row of its own in every state tensor, so that a part that updates its state
+        for every row of a step never touches a live request's."""
+        return self.max_seqs
 
     def life(self, req) -> int:
         """A number that no other stay of any request in this cache has had.  Whoever keeps
@@ -171,6 +180,21 @@ class CacheManager:
                     f"{g.pool.num_free} of {g.pool.num_pages} free (group {g.spec})")
         for n, g in zip(need, self.groups):
             g.tables[req].extend(g.pool.allocate(n))
+
+    def rollback(self, req) -> int:
+        """Gives back the pages that ``reserve`` took and no ``commit`` has filled (a step that
+        failed between the two); returns how many."""
+        st = self.requests[req]
+        keep = -(-st.num_tokens // self.page_size)
+        n = 0
+        for g in self.groups:
+            table = g.tables[req]
+            gone = [p for p in table[keep:] if p >= 0]
+            if gone:
+                g.pool.free(gone)
+                n += len(gone)
+            del table[keep:]
+        return n
 
     def commit(self, req, n_new: int) -> None:
         """``n_new`` tokens have been written.  Gives back the pages of window

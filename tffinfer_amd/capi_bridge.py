@@ -62,8 +62,6 @@ def create_random(config_file: str, seed: int, options_json: str) -> Handle:
     with open(config_file) as f:
         config = config_from_dict(json.load(f))
     dtype = resolve_dtype(opt.dtype)
-    if dtype == torch.float32:
-        torch.backends.cuda.matmul.allow_tf32 = False
     model = build_model_skeleton(config)
     model.init_random(int(seed), dtype, opt.device)
     return Handle(LLMEngine(model, opt))

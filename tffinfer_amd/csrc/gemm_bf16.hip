@@ -1306,42 +1306,6 @@ TFF_API int tff_gemm_row_scaled(const void* A, const void* Wp, void* C, int M, i
     return skinny_for<1>((const bf16_t*)A, (const bf16_t*)Wp, C, M, N, K, lda, c_dtype, glu_out, (hipStream_t)stream, &fz);
 }
 
-// out[m, :] = bfloat16(x[m, :] * rstd[m]): what tff_gemm_row_scaled's A stands for, written out
-// (for a consumer that is no such product).
-__global__ __launch_bounds__(256) void scale_rows_kernel(const bf16_t* __restrict__ x, const float* __restrict__ ss,
-                                                         int ss_stride, int ss_count, float inv_dim, float eps,
-                                                         bf16_t* __restrict__ out, int N) {
-    __shared__ float red[8];
-    const int m = blockIdx.x, tid = threadIdx.x;
-    // the same order of additions as in the product's prologue
-    float s4[4] = {0.f, 0.f, 0.f, 0.f};
-    if (tid < 4) {
-        const float* sp = ss + (size_t)m * ss_stride;
-        const int vec_end = ss_count & ~3;
-        for (int j = tid * 4; j < vec_end; j += 16) {
-            const float4 v = *reinterpret_cast<const float4*>(sp + j);
-            s4[0] += (v.x + v.y) + (v.z + v.w);
-        }
-        if (tid == 0)
-            for (int j = vec_end; j < ss_count; ++j) s4[0] += sp[j];
-        red[tid] = s4[0];
-    }
-    __syncthreads();
-    const float ssum = (red[0] + red[1]) + (red[2] + red[3]);
-    const float r = rsqrtf(ssum * inv_dim + eps);
-    for (int j = tid; j < N; j += blockDim.x) out[(size_t)m * N + j] = (bf16_t)((float)x[(size_t)m * N + j] * r);
-}
-
-TFF_API int tff_scale_rows(const void* x, const float* ss, int ss_stride, int ss_count, int dim, float eps, void* out,
-                           int M, int N, tff_stream_t stream) {
-    TFF_REQUIRE(x && ss && out && M >= 0 && M <= 16 && N > 0 && ss_count > 0 && ss_stride >= ss_count && dim > 0,
-                "scale_rows: bad operands (M=%d N=%d)", M, N);
-    if (M == 0) return 0;
-    scale_rows_kernel<<<M, 256, 0, (hipStream_t)stream>>>((const bf16_t*)x, ss, ss_stride, ss_count, 1.0f / (float)dim,
-                                                         eps, (bf16_t*)out, N);
-    return tff_check_launch("scale_rows");
-}
-
 int tff_gemm_f32(const float* A, const float* W, void* C, int M, int N, int K, int lda,
                  int c_dtype, hipStream_t s);
 

@@ -63,15 +63,12 @@ TFF_API int tff_gemm_plan(int M, int N, int K, int glu, int keep_partials, int* 
 //     columns 16 g .. 16 g + 15 of row m (16 rows of ss_stride floats).  N a multiple of 8.
 //   tff_gemm_row_scaled: C = rstd[m] * (A . W^T), rstd[m] = rsqrt(sum_{g < ss_count} ss[m][g] / dim
 //     + eps), the sums added in a fixed order; glu_out as in tff_gemm.
-//   tff_scale_rows: out = bfloat16(x * rstd[m]), for a consumer that is no such product.
 TFF_API int tff_gemm_residual_prenorm(const void* A, const void* Wp, int M, int N, int K, int lda, float* resid,
                                       const float* norm_w, void* x_out, float* ss_out, int ss_stride,
                                       tff_stream_t stream);
 TFF_API int tff_gemm_row_scaled(const void* A, const void* Wp, void* C, int M, int N, int K, int lda, int c_dtype,
                                 int glu_out, const float* ss, int ss_stride, int ss_count, int dim, float eps,
                                 tff_stream_t stream);
-TFF_API int tff_scale_rows(const void* x, const float* ss, int ss_stride, int ss_count, int dim, float eps, void* out,
-                           int M, int N, tff_stream_t stream);
 
 // bfloat16 row-major [N, K] (K a multiple of 8) -> fragment order: tiles of
 // 16 rows x 32 k, each stored as the 1 KB operand of a 16x16x32 MFMA, element

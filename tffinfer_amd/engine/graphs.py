@@ -7,7 +7,8 @@ size bucket into a HIP graph (through torch's CUDAGraph, which records the
 launches made on its capture stream, ours included) and replayed: the step's
 tables are written into fixed device buffers, the graph runs, the logits
 appear in a fixed tensor.  Rows beyond the live requests are padding: token 0
-at position 0 that writes no key and whose logits nobody reads.
+at position 0 that writes no key, whose state slot is a row of the state
+tensors that no request holds, and whose logits nobody reads.
 
 Nothing in a captured step clears memory with a memset node, and the kernels
 take every size from the tables, so one graph serves any mix of context
@@ -96,7 +97,7 @@ class DecodeTables:
         hv[o[1] + first:o[1] + B] = 0               # position
         hv[o[4] + first:o[4] + B] = 0               # start_pos
         hv[o[5] + first:o[5] + B] = 1               # context length
-        hv[o[6] + first:o[6] + B] = 0               # state slot
+        hv[o[6] + first:o[6] + B] = self.cache.padding_slot   # a state row that no request holds
         for gi, w in enumerate(self.widths):
             hv[o[10 + 2 * gi] + first:o[10 + 2 * gi] + B] = -1   # writes no key
             for r in range(first, B):
@@ -175,7 +176,7 @@ class DecodeGraph:
             b.groups.append(GroupTables(bt, sl(10 + 2 * gi, B), no_slot))
         b.host_cu_tokens = list(range(B + 1))
         b.host_start_pos = [0] * B
-        b.host_state_slots = [0] * B
+        b.host_state_slots = [cache.padding_slot] * B
         b.reqs = [None] * B
         self.batch = b
         self.pieces = [_Piece(safe, items) for safe, items in runner.model.graph_pieces()]
@@ -205,7 +206,6 @@ class DecodeGraph:
         gc.collect()
         gc_was_on = gc.isenabled()
         gc.disable()
-        H = rn.model.config.hidden_size
         try:
             with torch.cuda.stream(side):
                 self.dev.copy_(self.host, non_blocking=True)
@@ -216,7 +216,8 @@ class DecodeGraph:
                         # Not run here: every row is padding now, and such a part may keep state per
                         # request.  At every step it runs on the live rows and leaves its result in
                         # this tensor, which the next graph was captured to read.
-                        piece.pending = torch.zeros(self.B, H, dtype=torch.float32, device=rn.device)
+                        # (a pending term is added to the residual stream: it has the stream's shape)
+                        piece.pending = torch.zeros_like(resid)
                         piece.resid, pending = resid, piece.pending
                         continue
 

@@ -84,19 +84,11 @@ class LLMEngine:
         self.model = model
         cfg = model.config
         max_len = min(opt.max_model_len or cfg.max_position_embeddings, cfg.max_position_embeddings)
-        num_pages = opt.num_pages
         if sum(x is not None for x in (opt.num_pages, opt.kv_tokens, opt.kv_bytes)) > 1:
             raise ValueError("give one of num_pages, kv_tokens and kv_bytes")
-        if num_pages is None and opt.kv_bytes is not None:
-            per_page = self._bytes_per_page(model, opt.page_size)
-            num_pages = int(opt.kv_bytes) // per_page if per_page else 1
-            if num_pages < 1:
-                raise ValueError(f"kv_bytes={opt.kv_bytes} holds no page: one page of {opt.page_size} tokens "
-                                 f"takes {per_page} bytes over all layers")
-        elif num_pages is None:
-            tokens = opt.kv_tokens or opt.max_num_seqs * max_len
-            num_pages = -(-tokens // opt.page_size) + opt.max_num_seqs
-            num_pages = self._cap_pages_by_memory(model, num_pages, opt)
+        num_pages = opt.num_pages
+        if num_pages is None:
+            num_pages = self.plan_cache(model, opt, max_len)
         self.runner = ModelRunner(model, page_size=opt.page_size, num_pages=num_pages,
                                   max_seqs=opt.max_num_seqs, max_model_len=max_len,
                                   use_graphs=opt.use_graphs)
@@ -120,25 +112,26 @@ class LLMEngine:
         return cls(model, opt)
 
     @staticmethod
-    def _bytes_per_page(model, page_size: int) -> int:
-        """Device bytes of one page number over all caches (every group gets as many pages)."""
+    def plan_cache(model, opt: "EngineOptions", max_len: int, free_bytes: int | None = None) -> dict:
+        """Pages for every group of layers (``cache.sizing.plan_pages``): from ``kv_bytes``, or from
+        ``kv_tokens`` (by default what ``max_num_seqs`` requests of the longest length hold)
+        capped by ``memory_fraction`` of the free device memory, of which the per-request state
+        tensors come off first.  A group with a window gets the pages its window and a step's
+        tokens need, not the full pool."""
+        from ..cache.sizing import plan_pages
+        reqs = model.call_requirements()
         esz = 2 if model.dtype == torch.bfloat16 else 4
-        per_page = 0
-        seen = set()
-        for cache_id, _, kv, _ in model.call_requirements():
-            if kv is not None and cache_id not in seen:
-                seen.add(cache_id)
-                per_page += 2 * kv.num_kv_heads * kv.head_dim * page_size * esz
-        return per_page
-
-    @classmethod
-    def _cap_pages_by_memory(cls, model, num_pages: int, opt: EngineOptions) -> int:
-        free, _ = torch.cuda.mem_get_info(model.device)
-        per_page = cls._bytes_per_page(model, opt.page_size)
-        if per_page == 0:
-            return max(1, num_pages)
-        fit = int(free * opt.memory_fraction) // per_page
-        return max(1, min(num_pages, fit))
+        budget = max(opt.max_num_batched_tokens, opt.prefill_chunk)
+        try:
+            if opt.kv_bytes is not None:
+                return plan_pages(reqs, opt.page_size, esz, opt.max_num_seqs, budget, kv_bytes=int(opt.kv_bytes))
+            if free_bytes is None:
+                free_bytes = int(torch.cuda.mem_get_info(model.device)[0] * opt.memory_fraction)
+            tokens = opt.kv_tokens or opt.max_num_seqs * max_len
+            return plan_pages(reqs, opt.page_size, esz, opt.max_num_seqs, budget, tokens=tokens,
+                              free_bytes=free_bytes)
+        except ValueError as e:
+            raise ValueError(f"{e} (kv_bytes={opt.kv_bytes}, kv_tokens={opt.kv_tokens}, page_size={opt.page_size})") from None
 
     def warm_up(self) -> int:
         """What a server does before it takes requests: the decode graphs of all batch sizes are

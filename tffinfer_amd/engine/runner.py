@@ -151,15 +151,23 @@ class ModelRunner:
                     or token_source.device != torch.device(self.device):
                 raise StepError("token_source must be int32 [entries] on the runner's device")
         self.reserve(entries)
-        if self._graph_buckets and len(entries) <= self._graph_buckets[-1] \
-                and all(len(e.tokens) == 1 for e in entries):
-            return self._step_graph(entries, token_source)
-        with torch.cuda.device(self.device):
-            batch = build_step_batch(entries, self.cache, self.device, self._pinned)
-            if token_source is not None:
-                batch.token_ids[:len(entries)].copy_(token_source)
-            ctx = StepContext(self.ops, self.act_dtype, batch, self.max_model_len, self._calls, self.cache)
-            logits = self.model.forward(ctx)
+        try:
+            if self._graph_buckets and len(entries) <= self._graph_buckets[-1] \
+                    and all(len(e.tokens) == 1 for e in entries):
+                return self._step_graph(entries, token_source)
+            with torch.cuda.device(self.device):
+                batch = build_step_batch(entries, self.cache, self.device, self._pinned)
+                if token_source is not None:
+                    batch.token_ids[:len(entries)].copy_(token_source)
+                ctx = StepContext(self.ops, self.act_dtype, batch, self.max_model_len, self._calls, self.cache)
+                logits = self.model.forward(ctx)
+        except BaseException:
+            # The step did not run to its end: its tokens are not in the cache, so the pages taken
+            # for them (here or by a scheduler beforehand) go back and the requests stand where
+            # they stood; the caller may run the same step again.
+            for e in entries:
+                self.cache.rollback(e.req)
+            raise
         for e in entries:
             self.cache.commit(e.req, len(e.tokens))
         return logits

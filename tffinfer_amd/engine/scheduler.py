@@ -25,11 +25,13 @@ Rules of a step, in this order:
    recently admitted one is preempted and the step is planned again.
 
 A request that could never fit the pool or the model's length is refused when
-it is added, with an error, not truncated.  The check at that time is a bound
-for caches with a window; a request that passes it and still does not fit the
-cache when it is alone is taken out of the queue and finished with the reason
-"refused" (``Scheduler.refused`` holds such requests until the engine reports
-them), so that the requests behind it run.
+it is added, with an error, not truncated: a group that keeps every key must
+hold all its tokens, a group with a window the pages that one more token
+touches (portions are cut to what the free pages hold, however large the token
+budget lets them grow).  A request that passes this check and still does not
+fit the cache when it is alone is taken out of the queue and finished with the
+reason "refused" (``Scheduler.refused`` holds such requests until the engine
+reports them), so that the requests behind it run.
 """
 from __future__ import annotations
 
@@ -37,6 +39,7 @@ from collections import deque
 from dataclasses import dataclass, field
 
 from ..cache.manager import CacheManager
+from ..cache.sizing import min_window_pages
 from ..sampling.params import SamplingConfig
 
 
@@ -120,7 +123,9 @@ class Scheduler:
         # the last token chosen is never fed back, so total - 1 tokens reach the cache
         pages = -(-(total - 1) // ps)
         for g in self.cache.groups:
-            need = pages if g.spec.window <= 0 else min(pages, -(-(g.spec.window + self.opt.prefill_chunk) // ps) + 1)
+            # a group with a window must hold what one more token touches; portions are cut to
+            # what the free pages hold (_fit), so no larger bound is needed for the request to run
+            need = pages if g.spec.window <= 0 else min(pages, min_window_pages(g.spec.window, ps))
             if need > g.pool.num_pages:
                 raise RequestRefused(
                     f"request {req.id!r} needs {need} cache pages, the pool has {g.pool.num_pages} in all")

@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 
 class KernelLibraryError(RuntimeError):
@@ -28,7 +28,6 @@ _SIGNATURES = {
     "tff_gemm_plan": [_I, _I, _I, _I, _I, _P, _P, _P],
     "tff_gemm_residual_prenorm": [_P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P],
     "tff_gemm_row_scaled": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _F, _P],
-    "tff_scale_rows": [_P, _P, _I, _I, _I, _F, _P, _I, _I, _P],
     "tff_pack_weight": [_P, _P, _I, _I, _P],
     "tff_embed_packed": [_P, _P, _P, _I, _I, _I, _P],
     "tff_qk_norm_rope_kv": [_P, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _I, _P, _P, _P, _P,

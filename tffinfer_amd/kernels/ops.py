@@ -185,19 +185,19 @@ class ScaledRows:
     ``x`` [M, H] bfloat16 = (residual stream) * (norm weight), and the sums of
     squares of every row's groups of 16 columns, ``ss`` [16, stride] float32
     (``count`` of them a row).  ``linear`` applies rsqrt(sum / H + eps) to its
-    accumulators; :meth:`materialize` writes the normalised rows out."""
+    accumulators; :meth:`materialize` writes the normalised rows out, from the
+    float32 residual stream ``resid`` (which must still hold the sum the norm
+    was taken of) and the norm's ``weight``, so that they are rounded to
+    bfloat16 once, as the norm's own kernel rounds them."""
 
-    def __init__(self, x: torch.Tensor, ss: torch.Tensor, count: int, eps: float):
+    def __init__(self, x: torch.Tensor, ss: torch.Tensor, count: int, eps: float,
+                 resid: torch.Tensor, weight: torch.Tensor):
         self.x, self.ss, self.count, self.eps = x, ss, int(count), float(eps)
+        self.resid, self.weight = resid, weight
         self.shape, self.dtype, self.device = x.shape, x.dtype, x.device
 
     def materialize(self) -> torch.Tensor:
-        M, H = self.x.shape
-        out = torch.empty_like(self.x)
-        L = _lib.load()
-        _lib.check(L.tff_scale_rows(self.x.data_ptr(), self.ss.data_ptr(), self.ss.stride(0), self.count, H,
-                                    self.eps, out.data_ptr(), M, H, _stream()))
-        return out
+        return add_rmsnorm(self.resid, None, self.weight, self.eps, self.x.dtype)
 
 
 def as_tensor(t) -> torch.Tensor:
@@ -228,7 +228,7 @@ def _fused_prenorm(p: PendingProduct, resid: torch.Tensor, weight: torch.Tensor,
     L = _lib.load()
     _lib.check(L.tff_gemm_residual_prenorm(x.data_ptr(), p.weight.data_ptr(), M, N, K, lda, resid.data_ptr(),
                                            weight.data_ptr(), xs.data_ptr(), ss.data_ptr(), stride, _stream()))
-    return ScaledRows(xs, ss, groups, eps)
+    return ScaledRows(xs, ss, groups, eps, resid, weight)
 
 
 def add_rmsnorm(resid: torch.Tensor, delta, weight: torch.Tensor, eps: float,
@@ -644,7 +644,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
         # decoding only: a wave per request, kv head and run of keys; sizes come from the tables
         tiles = -(-G // 16)
         if splits is None:
-            splits = getattr(batch, "attn_splits", None) or pick_splits(R * tiles * nkv, batch.max_context)
+            splits = pick_splits(R * tiles * nkv, batch.max_context)
         launch(None, R * tiles, None, 0, tiles, 16, splits)
         return out
     # long portions: blocks that share their keys through LDS (128 columns); short ones: a wave
@@ -741,12 +741,10 @@ def attention_decode_fused(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weigh
     if scale is None:
         scale = 1.0 / math.sqrt(d)
     if splits is None:
-        splits = getattr(batch, "attn_splits", None)
-        if splits is None:
-            # entries x kv heads enough for a block each to saturate HBM between them: the keys of
-            # an entry are split among the eight waves of its block and merged in LDS (splits 0)
-            splits = 0 if (R * nkv >= BLOCK_DECODE_MIN_PAIRS and tiles == 1 and d <= 128) else \
-                pick_splits(R * tiles * nkv, batch.max_context)
+        # entries x kv heads enough for a block each to saturate HBM between them: the keys of
+        # an entry are split among the eight waves of its block and merged in LDS (splits 0)
+        splits = 0 if (R * nkv >= BLOCK_DECODE_MIN_PAIRS and tiles == 1 and d <= 128) else \
+            pick_splits(R * tiles * nkv, batch.max_context)
     out = torch.empty(R, nq * d, dtype=qkv.dtype, device=qkv.device)
     part_o = part_ml = None
     if splits > 1:

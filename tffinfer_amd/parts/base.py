@@ -52,7 +52,11 @@ class StateSpec:
 class Part:
     #: True if ``forward`` launches only kernels that take the step's sizes from
     #: device tables (no host loop over the step's entries), so that a decode step
-    #: with this part can be captured in a HIP graph and replayed.
+    #: with this part can be captured in a HIP graph and replayed.  A captured step
+    #: has padding rows (and runs twice on nothing but padding rows before it is
+    #: captured): they write no key, and their state slot is a row of the state
+    #: tensors that no request holds (``CacheManager.padding_slot``), so a part
+    #: with state of its own may update the state of every row it is given.
     graph_safe = False
 
     def weight_specs(self) -> dict[str, WeightSpec]:

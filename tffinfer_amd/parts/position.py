@@ -2,6 +2,7 @@
 from __future__ import annotations
 
 import math
+import weakref
 
 import torch
 
@@ -18,10 +19,11 @@ class NoPosition(PositionEncoding):
         return None
 
 
-# Rotation tables by (class, rotary size, theta, positions, device).  Layers with the same law share one
-# tensor, and a table is never dropped: a captured decode graph holds its address for as long as
-# the graph lives, whatever other runner asks for another length meanwhile.
-_TABLES: dict = {}
+# Rotation tables by (class, everything the law depends on, positions, device).  Layers with the same
+# law share one tensor.  The entries are weak: a table lives as long as an encoding that asked for
+# it does (``PositionEncoding.cached_table`` keeps it, and with it every captured decode graph that
+# holds its address), and goes when the last such model goes.
+_TABLES = weakref.WeakValueDictionary()
 
 
 @register_position_encoding("rope")
@@ -53,8 +55,15 @@ class RotaryEmbedding(PositionEncoding):
         inv = torch.exp(-(2.0 * i / self.rotary_dim) * math.log(self.theta))
         return torch.arange(max_positions, dtype=torch.float64)[:, None] * inv[None, :]
 
+    def table_key(self) -> tuple:
+        """Everything ``angles`` depends on: by default all the instance's public attributes, so
+        that a subclass whose law has a further parameter (a scaling factor, say) shares no table
+        with an instance that has another value of it."""
+        return tuple(sorted((k, v) for k, v in vars(self).items()
+                            if not k.startswith("_") and isinstance(v, (int, float, str, bool, tuple, type(None)))))
+
     def table(self, max_positions, device):
-        key = (type(self), self.rotary_dim, self.theta, int(max_positions), str(torch.device(device)))
+        key = (type(self), self.table_key(), int(max_positions), str(torch.device(device)))
         t = _TABLES.get(key)
         if t is None:
             a = self.angles(max_positions)
