@@ -67,6 +67,9 @@ def parse_args():
     ap.add_argument("--no-large-points", action="store_true",
                     help="skip the two points at the larger shapes (32 mixed requests at the 14B shape; batch 16 "
                          "at 8,192 tokens of context at the 32B shape), which the default run adds to 'points'")
+    ap.add_argument("--no-long-points", action="store_true",
+                    help="skip the points at long contexts (decode at batch 8 with 32,768 tokens of context and at "
+                         "batch 128 with 8,192; prefill of 8,192 and of 32,768 tokens), which the default run adds")
     return ap.parse_args()
 
 
@@ -127,6 +130,59 @@ def large_points(args, gen) -> dict:
     return out
 
 
+def long_points(args, model, cfg, gen) -> tuple[dict, dict]:
+    """Further sizes at the benchmark shape, on an engine of their own whose length limit holds
+    them (a decode graph's launches are sized for the limit, so the headline keeps its own):
+    decode steps of 8 requests at 32,768 tokens of context and of 128 requests at 8,192, and
+    prompts of 8,192 and 32,768 tokens in one step.  Returns (tokens a second, details) by
+    point; a point that fails is left null."""
+    import gc
+    import torch
+    from tffinfer_amd import EngineOptions, LLMEngine
+    from tffinfer_amd import measure as M
+    points, detail = {}, {}
+    vocab = cfg["vocab_size"]
+    L = cfg["num_hidden_layers"]
+    for key, batch, context, steps, warmup in (("decode_b8_ctx32768", 8, 32768, 16, 4),
+                                               ("decode_b128_ctx8192", 128, 8192, 12, 4)):
+        try:
+            total = steps + warmup + M.decode_slack(batch, context) + 16
+            opt = EngineOptions(dtype="bfloat16", page_size=args.page_size,
+                                kv_tokens=batch * (context + total + args.page_size), max_num_seqs=batch,
+                                max_num_batched_tokens=4096, prefill_chunk=2048, max_model_len=context + total + 16,
+                                use_graphs=not args.no_graphs)
+            engine = LLMEngine(model, opt)
+            r = M.measure_decode(engine, gen, batch, context, steps, warmup, vocab)
+            step = r["wall_s"] / steps
+            nbytes = M.decode_bytes(model, batch, context + warmup + steps / 2.0)
+            points[key] = round(batch / step, 1)
+            detail[key] = {"ms_per_step": round(1e3 * step, 4), "ms_per_step_median": round(1e3 * r["step_median_s"], 4),
+                           "frac": round(nbytes / step / 1e9 / M.HBM_PEAK_GBS, 4)}
+            del engine
+        except Exception as e:      # the headline figures must not be lost to a side measurement
+            print(f"bench: the point {key} failed: {e}", file=sys.stderr)
+            points[key] = None
+        gc.collect()
+        torch.cuda.empty_cache()
+    for key, T, reps in (("prefill_8192", 8192, 4), ("prefill_32768", 32768, 2)):
+        try:
+            opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=T + args.page_size, max_num_seqs=1,
+                                max_num_batched_tokens=T, prefill_chunk=T, max_model_len=T + 16,
+                                use_graphs=False)
+            engine = LLMEngine(model, opt)
+            r = M.measure_prefill(engine, gen, T, vocab, reps=reps, warm=1)
+            points[key] = round(T / r["wall_s"], 1)
+            detail[key] = {"ms": round(1e3 * r["wall_s"], 3), "ms_device": round(1e3 * r["device_s"], 3),
+                           "frac": round(M.prefill_flops(model, T) / r["wall_s"] / M.MFMA_PEAK["bf16"], 4)}
+            del engine
+        except Exception as e:
+            print(f"bench: the point {key} failed: {e}", file=sys.stderr)
+            points[key] = None
+        gc.collect()
+        torch.cuda.empty_cache()
+    return points, detail
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -153,8 +209,14 @@ def main():
     # a context beyond the shape's own limit: the limit grows with it (it sizes the rotation table only)
     longest = max(args.prefill_tokens,
                   args.context + args.steps + args.warmup + M.decode_slack(max(args.batch, 64), args.context) + 16)
+    want_long = (args.shape == "8b" and args.layers is None and not args.only and not args.no_points
+                 and not args.no_long_points and not args.mixed)
     if not args.mixed and longest > cfg["max_position_embeddings"]:
         cfg["max_position_embeddings"] = 1 << (longest - 1).bit_length()
+    headline_limit = cfg["max_position_embeddings"]
+    if want_long:
+        # the model's own limit sizes the rotation table only; every engine below has its own
+        cfg["max_position_embeddings"] = max(headline_limit, 65536)
     vocab = cfg["vocab_size"]
     gen = torch.Generator().manual_seed(args.seed)
     model = build_model(cfg, args.seed)
@@ -173,7 +235,7 @@ def main():
     kv_tokens = max_batch * (args.context + total_steps + args.page_size) + args.prefill_tokens
     opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=kv_tokens, max_num_seqs=max_batch,
                         max_num_batched_tokens=max(4096, max_batch), prefill_chunk=2048,
-                        max_model_len=cfg["max_position_embeddings"], use_graphs=not args.no_graphs)
+                        max_model_len=headline_limit, use_graphs=not args.no_graphs)
     engine = LLMEngine(model, opt)
 
     pre = dec = None
@@ -198,12 +260,17 @@ def main():
             part["sampling"] = args.sampling
         print(json.dumps({"only": args.only, **part, "batch": args.batch, "context": args.context}))
         return
-    points = {}
+    points, detail = {}, {}
     if not args.no_points:
         for b, key in ((1, "decode_b1"), (64, "decode_b64")):
             k = min(args.steps, 32)
-            r = M.measure_decode(engine, gen, b, args.context, k, min(args.warmup, 4), vocab)
+            w = min(args.warmup, 4)
+            r = M.measure_decode(engine, gen, b, args.context, k, w, vocab)
             points[key] = round(b * k / r["wall_s"], 1)
+            nb = M.decode_bytes(model, b, args.context + w + k / 2.0)
+            detail[key] = {"ms_per_step": round(1e3 * r["wall_s"] / k, 4),
+                           "ms_per_step_median": round(1e3 * r["step_median_s"], 4),
+                           "frac": round(nb / (r["wall_s"] / k) / 1e9 / M.HBM_PEAK_GBS, 4)}
         # the headline batch again with every request drawing from the top 50 tokens at top-p 0.95 and
         # temperature 0.8 instead of taking the most likely one
         from tffinfer_amd.sampling import SamplingConfig
@@ -217,9 +284,9 @@ def main():
     ms_step = 1000.0 * t_decode / args.steps
     value = args.batch * args.steps / t_decode
     mean_context = args.context + args.warmup + args.steps / 2.0
-    nbytes = M.decode_bytes(cfg, L, args.batch, mean_context)
+    nbytes = M.decode_bytes(model, args.batch, mean_context)
     achieved = nbytes / (t_decode / args.steps) / 1e9
-    pf = M.prefill_flops(cfg, L, args.prefill_tokens)
+    pf = M.prefill_flops(model, args.prefill_tokens)
     out = {
         "metric": "decode_tokens_per_s", "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
@@ -233,7 +300,7 @@ def main():
             "q_heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": vocab,
             "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],
-            "max_context": cfg["max_position_embeddings"], "global_batch": args.batch,
+            "max_context": headline_limit, "global_batch": args.batch,
             "seq_len": args.context, "prefill_tokens": args.prefill_tokens, "page_size": args.page_size,
             "hip_graphs": not args.no_graphs, "parallelism": "single GPU",
         },
@@ -248,7 +315,19 @@ def main():
         # issues bfloat16 MFMAs from registers
         "ceilings": ceilings,
         "points": points,
+        # per point: the step's (or the prompt's) time and its share of the published peak (HBM for decode
+        # steps, bf16 MFMA for prompts)
+        "points_detail": detail,
     }
+    if want_long:
+        del engine
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        engine = None
+        lp, ld = long_points(args, model, cfg, gen)
+        out["points"].update(lp)
+        out["points_detail"].update(ld)
     if args.shape == "8b" and args.layers is None and not args.no_points and not args.no_large_points:
         del engine, model
         import gc

@@ -248,3 +248,31 @@ def test_warm_up_captures_every_decode_graph_beforehand(model_dirs, dtype):
         else:
             assert captured == [1, 3, 6]      # 6 stood in for 4 and 3 for 2, which were wanted for a few steps only
     assert outs[0] == outs[1]
+
+
+@pytest.mark.parametrize("name", ["B", "D"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_window_groups_get_pools_of_their_own_size(model_dirs, dtype, name):
+    """Sized by the engine (not by a page count given to it), the layers with a window get the
+    pages their window and a step's tokens need, a fraction of the pool of the layers that keep
+    every key; requests far longer than that pool run beside each other without a preemption."""
+    from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
+    from tffinfer_amd.cache.sizing import window_pool_pages
+    d = model_dirs[name]
+    cfg = read_config(d)
+    V, limit = cfg["vocab_size"], cfg["max_position_embeddings"]
+    opt = EngineOptions(dtype=dtype, page_size=8, max_num_seqs=4, max_num_batched_tokens=64, prefill_chunk=24)
+    eng = LLMEngine.from_model_dir(d, opt)
+    groups = {g.spec.window: g.pool.num_pages for g in eng.runner.cache.groups}
+    w = cfg["sliding_window"]
+    assert groups[0] == 4 * limit // 8 + 4
+    assert groups[w] == window_pool_pages(w, 8, 4, 64) < groups[0] // 3
+    prompts = [random_tokens(n, V, 80 + n) for n in (limit - 60, 150, 9, 120, 77)]
+    sc = [SamplingConfig("random", temperature=0.8, seed=7 + i) if i % 2 else SamplingConfig() for i in range(5)]
+    eng.keep_logits = True
+    res = eng.generate(prompts, sc, max_new_tokens=40, ignore_eos=True)
+    assert eng.scheduler.stats.preemptions == 0
+    for r, s in zip(res, sc):
+        assert len(r.output) == 40
+        check_choices(d, r, dtype, s)
+    assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)

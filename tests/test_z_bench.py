@@ -48,4 +48,8 @@ def test_one_json_line_with_the_contract_keys():
     assert rec["roofline"]["frac"] == pytest.approx(rec["roofline"]["achieved"] / 8000.0, abs=1e-3)
     assert set(rec["points"]) == {"decode_b1", "decode_b64", "decode_b2_top_k50_top_p0.95"}
     assert all(v > 0 for v in rec["points"].values())
+    for key, b in (("decode_b1", 1), ("decode_b64", 64)):      # a point's own time and share of the HBM peak
+        d = rec["points_detail"][key]
+        assert rec["points"][key] == pytest.approx(b * 1000.0 / d["ms_per_step"], rel=1e-3)
+        assert 0 < d["ms_per_step_median"] < 3 * d["ms_per_step"] and 0 < d["frac"] < 1
     assert rec["points"]["decode_b2_top_k50_top_p0.95"] < 1.05 * rec["value"]      # drawing costs something, not nothing

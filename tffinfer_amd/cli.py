@@ -128,26 +128,21 @@ def _bench(args, rt, cfg) -> int:
                         kv_tokens=None if (args.num_pages or args.kv_bytes) else kv_tokens,
                         num_pages=args.num_pages, kv_bytes=args.kv_bytes)
     engine = LLMEngine(model, opt)
-    L = len(mc.layer_specs())
     rec = {"bench": args.bench, "dtype": dtype, "batch": args.batch, "context": args.context}
-    try:
-        if args.bench == "decode":
-            r = M.measure_decode(engine, gen, args.batch, args.context, args.gen, warmup, vocab)
-            step = r["wall_s"] / args.gen
-            rec.update(steps=args.gen, tokens_per_s=round(args.batch / step, 1), ms_per_step=round(1e3 * step, 4),
-                       ms_per_step_median=round(1e3 * r["step_median_s"], 4))
-            nbytes = M.decode_bytes(mc, L, args.batch, args.context + warmup + args.gen / 2.0,
-                                    2 if args.use_f16 else 4)
-            rec["hbm_GBps"] = round(nbytes / step / 1e9, 1)
-            rec["hbm_frac"] = round(nbytes / step / 1e9 / M.HBM_PEAK_GBS, 4)
-        else:
-            r = M.measure_prefill(engine, gen, args.context, vocab, reps=max(1, min(args.gen, 20)))
-            flops = M.prefill_flops(mc, L, args.context)
-            rec.update(tokens_per_s=round(args.context / r["wall_s"], 1), ms=round(1e3 * r["wall_s"], 3),
-                       ms_device=round(1e3 * r["device_s"], 3),
-                       mfma_frac=round(flops / r["wall_s"] / M.MFMA_PEAK[dtype], 6))
-    except AttributeError as e:     # a configuration without the sizes the byte and flop counts need
-        log.warning("no roofline figures for this architecture: %s", e)
+    if args.bench == "decode":
+        r = M.measure_decode(engine, gen, args.batch, args.context, args.gen, warmup, vocab)
+        step = r["wall_s"] / args.gen
+        rec.update(steps=args.gen, tokens_per_s=round(args.batch / step, 1), ms_per_step=round(1e3 * step, 4),
+                   ms_per_step_median=round(1e3 * r["step_median_s"], 4))
+        nbytes = M.decode_bytes(model, args.batch, args.context + warmup + args.gen / 2.0, 2 if args.use_f16 else 4)
+        rec["hbm_GBps"] = round(nbytes / step / 1e9, 1)
+        rec["hbm_frac"] = round(nbytes / step / 1e9 / M.HBM_PEAK_GBS, 4)
+    else:
+        r = M.measure_prefill(engine, gen, args.context, vocab, reps=max(1, min(args.gen, 20)))
+        flops = M.prefill_flops(model, args.context)
+        rec.update(tokens_per_s=round(args.context / r["wall_s"], 1), ms=round(1e3 * r["wall_s"], 3),
+                   ms_device=round(1e3 * r["device_s"], 3),
+                   mfma_frac=round(flops / r["wall_s"] / M.MFMA_PEAK[dtype], 6))
     print(json.dumps(rec))
     return 0
 

@@ -665,6 +665,12 @@ __global__ __launch_bounds__(256) void attn_split_reduce_few_kernel(const float*
         if (lane + 64 * e < d) o[lane + 64 * e] = (bf16_t)(acc[e] * inv);
 }
 
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // ------------------------------------------------- prompt portions, by block ---
 // For portions of many tokens a block of NW waves shares its keys and values:
 // every 32-key slice is copied once from the pages into LDS (by the load unit,
@@ -779,6 +785,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
     // in flight, in every iteration.
     __builtin_amdgcn_s_waitcnt(vmcnt_imm0());
 
+    // (what LDS holds is a page's start in units of 16 bytes: page number x page_stride / 8)
 #define ATTN_PAGE(j) pages[page_index((j), page_size, page_shift) - pg0]
     // fragment f of a slice: f < KFR is key tile f / KS, k-step f % KS; else value tile f - KFR
     // Every wave issues LPW copies per slice, also past the last slice (clamped to it) and past
@@ -807,10 +814,10 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
         if (f < KFR) {
             const int kt = f / KS, ks = f - kt * KS;
             cp_key[j] = (qc >> 2) * 8 + kt * 4 + (qc & 3);
-            cp_off[j] = min(ks * 32 + kg * 8, D - 8);
+            cp_off[j] = min(ks * 32 + kg * 8, D - 8) >> 3;          // in units of 8 elements, as the page starts are
         } else {
             cp_key[j] = kg * 8;
-            cp_off[j] = ((f - KFR) * 16 + qc) * page_size;
+            cp_off[j] = (((f - KFR) * 16 + qc) * page_size) >> 3;   // (pages hold a multiple of 8 tokens)
         }
     }
 #define ATTN_ISSUE(step)                                                                            \
@@ -821,12 +828,12 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
             const bf16_t* g_;                                                                       \
             if (cp_is_k[j]) {                                                                       \
                 const int key = min(kb_ + cp_key[j], kmax);                                         \
-                g_ = kbase + ((uint64_t)(uint32_t)ATTN_PAGE(key) * page_stride +                    \
-                              (uint32_t)(page_slot(key, page_size, page_shift) * D + cp_off[j]));   \
+                g_ = kbase + ((uint64_t)((uint32_t)ATTN_PAGE(key) +                                 \
+                              (uint32_t)(page_slot(key, page_size, page_shift) * (D / 8) + cp_off[j])) << 3); \
             } else {                                                                                \
                 const int j0 = min(kb_ + cp_key[j], vkmax);                                         \
-                g_ = vbase + ((uint64_t)(uint32_t)ATTN_PAGE(j0) * page_stride +                     \
-                              (uint32_t)(cp_off[j] + page_slot(j0, page_size, page_shift)));        \
+                g_ = vbase + ((uint64_t)((uint32_t)ATTN_PAGE(j0) +                                  \
+                              (uint32_t)(cp_off[j] + (page_slot(j0, page_size, page_shift) >> 3))) << 3); \
             }                                                                                       \
             copy16_to_lds_at(g_, smem_addr + (unsigned)(st_ * FRT + cp_F[j]) * 1024u);              \
         }                                                                                           \
@@ -861,7 +868,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
     pg0 = page_index(kb0 + seg0 * 32, page_size, page_shift);
     {
         const int npg = page_index(min(kmax, kb0 + seg1 * 32 - 1), page_size, page_shift) - pg0 + 1;
-        for (int i = tid; i < npg; i += 64 * NWT) pages[i] = bt[pg0 + i];
+        for (int i = tid; i < npg; i += 64 * NWT) pages[i] = (int32_t)((uint32_t)bt[pg0 + i] * (page_stride >> 3));
     }
     __syncthreads();   // pages[] is written
 #pragma unroll
@@ -913,8 +920,8 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
                     if (!(j >= c_lo[t] && j <= c_pos[t])) sv[e] = -INFINITY;
                 }
             }
-            float mt = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
-                             fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+            // (three-operand maxima as the instruction is: fmaxf has every operand quieted first, eight more instructions a slice)
+            float mt = max3_raw(max3_raw(sv[0], sv[1], sv[2]), max3_raw(sv[3], sv[4], sv[5]), fmaxf(sv[6], sv[7]));
             // m_run is the reference the exponentials are taken against: the largest score seen
             // when it was last moved, in raw score units.  It is moved (the maximum over a
             // column's four lanes, the accumulators rescaled) only when some score exceeds it by
@@ -1116,6 +1123,10 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                 "attention_mfma: head size %d with pages of %d is not supported by the matrix-core "
                 "kernel (head sizes 16..128 in steps of 16, 192, 256; pages of a power of two, at least 8)", d, page_size);
     TFF_REQUIRE((long)nkv * page_size * d < (1L << 31), "attention_mfma: a page of %d x %d x %d elements is too large", nkv, page_size, d);
+    // (the blocks of long portions keep a page's start as a 32-bit count of 16-byte units)
+    TFF_REQUIRE(cols_per_wave < 128 || (long)num_pages * nkv * page_size * d / 8 < (1L << 32),
+                "attention_mfma: a cache of %d pages of %d x %d x %d elements is too large for the kernel of long portions",
+                num_pages, nkv, page_size, d);
     TFF_REQUIRE(q_stride >= nq * d && q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0,
                 "attention_mfma: query rows must be 16-byte aligned (stride %d)", q_stride);
     TFF_REQUIRE(cols_per_wave == 16 || cols_per_wave == 128 || cols_per_wave == 256,

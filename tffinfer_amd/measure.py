@@ -11,6 +11,7 @@ repository root and ``tffinfer --bench`` both call these functions.
 """
 from __future__ import annotations
 
+import math
 import statistics
 import time
 
@@ -20,31 +21,49 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense, published
 
 
-def _get(c, key):
-    return c[key] if isinstance(c, dict) else getattr(c, key)
+def _matrix_elements(part) -> int:
+    """Elements of the matrices a part and its sub-parts multiply with."""
+    n = sum(math.prod(spec.shape) for spec in part.weight_specs().values()
+            if spec.init == "matrix" and len(spec.shape) == 2)
+    return n + sum(_matrix_elements(child) for child in part.children().values())
 
 
-def matmul_params_per_layer(c) -> int:
-    """Weights of a layer's four products, from a config.json dict or a typed configuration
-    of an attention + gated feed-forward layer."""
-    H, nq, nkv, d, I = (_get(c, "hidden_size"), _get(c, "num_attention_heads"), _get(c, "num_key_value_heads"),
-                        _get(c, "head_dim"), _get(c, "intermediate_size"))
-    return (nq + 2 * nkv) * d * H + nq * d * H + 3 * I * H
+def matrix_elements_per_step(model) -> int:
+    """Elements of all matrices a step multiplies a token's row with, a layer that the run order
+    names twice counted twice; without the output head."""
+    return sum(_matrix_elements(model.blocks[call.layer]) for call in model.schedule)
 
 
-def prefill_flops(c, L: int, T: int) -> float:
-    """Flops of one prompt of T tokens: the products of L layers, causal attention, the head
-    for one row."""
-    gemm = 2.0 * T * matmul_params_per_layer(c) * L
-    attn = 4.0 * _get(c, "num_attention_heads") * _get(c, "head_dim") * (T * (T + 1) / 2) * L
-    head = 2.0 * _get(c, "hidden_size") * _get(c, "vocab_size")
-    return gemm + attn + head
+def prefill_flops(model, T: int) -> float:
+    """Flops of one prompt of T tokens, from the model's own parts: the matrix products of every
+    layer call, what every mixer spends per (query, key) pair under its causal mask and window,
+    and the output head for one row."""
+    cfg = model.config
+    flops = 2.0 * T * matrix_elements_per_step(model)
+    for call in model.schedule:
+        mixer = model.blocks[call.layer].mixer
+        per_pair = mixer.flops_per_query_key_pair()
+        if per_pair:
+            spec = mixer.cache_spec()
+            w = spec.window if spec is not None and spec.window > 0 else T
+            w = min(w, T)
+            pairs = w * (w + 1) / 2 + (T - w) * w      # token t reads min(t + 1, window) keys
+            flops += per_pair * pairs
+    return flops + 2.0 * cfg.hidden_size * cfg.vocab_size
 
 
-def decode_bytes(c, L: int, batch: int, context: float, esz: int = 2) -> float:
-    """Bytes a decode step has to read: every weight once, and the cache of the live requests."""
-    weights = (matmul_params_per_layer(c) * L + _get(c, "hidden_size") * _get(c, "vocab_size")) * esz
-    kv = 2 * L * _get(c, "num_key_value_heads") * _get(c, "head_dim") * esz * batch * context
+def decode_bytes(model, batch: int, context: float, esz: int = 2) -> float:
+    """Bytes a decode step has to read, from the model's own parts: every matrix it multiplies
+    with once (a layer that the run order names twice, twice), the output head, and the keys and
+    values that every layer call reads for the live requests (a window's worth where it has one)."""
+    cfg = model.config
+    weights = (matrix_elements_per_step(model) + cfg.hidden_size * cfg.vocab_size) * esz
+    kv = 0.0
+    for call in model.schedule:
+        spec = model.blocks[call.layer].mixer.cache_spec()
+        if spec is not None:
+            keys = min(context, spec.window) if spec.window > 0 else context
+            kv += 2 * spec.num_kv_heads * spec.head_dim * esz * batch * keys
     return weights + kv
 
 

@@ -52,6 +52,9 @@ class GQAttention(Mixer):
     def cache_spec(self):
         return KVCacheSpec(self.num_kv_heads, self.head_dim, self.window)
 
+    def flops_per_query_key_pair(self):
+        return 4 * self.num_heads * self.head_dim      # q.k and p.v, a multiply and an add each
+
     def weight_specs(self):
         H, nq, nkv, d = self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim
         specs = {

@@ -125,6 +125,12 @@ class Mixer(Part):
     def state_spec(self) -> StateSpec | None:
         return None
 
+    def flops_per_query_key_pair(self) -> int:
+        """Flops the mixer spends on one (query token, key it reads) pair beyond its matrix
+        products with weights (attention: scores and weighted values over all heads); for the
+        measurements' flop counts.  0 for a mixer without such pairs."""
+        return 0
+
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
         """x [T, hidden] in the activation type -> float32 [T, hidden] to be
         added to the residual stream, or what ``ops.linear(..., partials=True)``
