@@ -35,4 +35,7 @@ def pytest_terminal_summary(terminalreporter):
         terminalreporter.write_line("worst error against the plain implementation / tolerance, per configuration:")
         for (dtype, name), err in sorted(WORST.items()):
             t = _TOL.get(dtype, {}).get(name)
+            if dtype == "kernels":
+                import test_kernels_gpu
+                t = test_kernels_gpu.ATTN_TOL
             terminalreporter.write_line(f"  {dtype:9s} {name:6s} {err:.2e}" + (f" / {t:.1e}" if t else ""))

@@ -100,3 +100,69 @@ def test_twenty_eight_requests_shrinking_through_the_graph_buckets(model_dirs, n
         check_choices(d, r, dtype, sc[i])
     assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
     assert eng.runner.cache.slots.num_free == n
+
+
+@pytest.mark.parametrize("seed", range(3))
+@pytest.mark.parametrize("name,dtype", [("E", "bfloat16"), ("E", "float32"), ("W", "bfloat16")])
+def test_random_workloads_of_many_requests_on_small_pools(model_dirs, name, dtype, seed):
+    """Random workloads of eighteen to twenty-six requests on sixteen to twenty-four slots and a
+    pool that holds some six tenths of what they need together (lengths, arrival steps,
+    sampling, an abort), with decode graphs and steps launched ahead: batches grow and shrink through the
+    buckets, requests are preempted out of large batches and come back, rows change hands.
+    Whatever the schedule, every kept row of logits matches the plain logits of the request's
+    own sequence and every token is the plain sampler's choice."""
+    import random
+    from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
+    from tffinfer_amd.engine.runner import ModelRunner
+    rng = random.Random(2000 * seed + 13 * ord(name) + (5 if dtype == "float32" else 0))
+    d = model_dirs[name]
+    cfg = read_config(d)
+    V, limit = cfg["vocab_size"], 200
+    n = rng.randrange(18, 27)
+    ps = rng.choice([16, 32])
+    reqs, need = [], 0
+    for i in range(n):
+        plen, new = rng.randrange(1, 90), rng.randrange(2, 50)
+        sc = SamplingConfig("random", temperature=rng.choice([0.6, 1.0, 1.3]), seed=rng.randrange(1 << 20)) \
+            if rng.random() < 0.4 else SamplingConfig()
+        reqs.append(dict(prompt_ids=random_tokens(plen, V, 8000 + 41 * seed + i), sampling=sc, max_new_tokens=new,
+                         ignore_eos=True, request_id=i))
+        need += -(-(plen + new) // ps)
+    biggest = max(-(-(len(r["prompt_ids"]) + r["max_new_tokens"]) // ps) for r in reqs)
+    pages = max(biggest + 1, int(need * (0.55, 0.62, 0.68)[seed % 3]))
+    slots = rng.randrange(16, 25)
+    opt = EngineOptions(dtype=dtype, page_size=ps, num_pages=pages, max_num_seqs=slots,
+                        max_num_batched_tokens=rng.choice([64, 128, 256]), prefill_chunk=rng.choice([16, 48, 96]),
+                        max_model_len=limit, use_graphs=True, run_ahead=True)
+    eng = LLMEngine.from_model_dir(d, opt)
+    eng.keep_logits = True
+    ModelRunner.CAPTURE_AFTER, kept = 4, ModelRunner.CAPTURE_AFTER
+    try:
+        arrivals = {}
+        for r in reqs:
+            arrivals.setdefault(rng.randrange(0, 12), []).append(r)
+        victim = rng.randrange(n)
+        state = {}
+
+        def on_step(step):
+            r = eng._requests.get(victim)
+            if "done" not in state and r is not None and r.status == "running" and len(r.output) >= 2:
+                eng.abort(victim)
+                state["done"] = True
+
+        drive(eng, arrivals, on_step)
+    finally:
+        ModelRunner.CAPTURE_AFTER = kept
+    st = eng.scheduler.stats
+    print(f"{name} {dtype} seed {seed}: {n} requests, {pages} pages of {ps}, {slots} slots: {st.steps} steps, "
+          f"{st.preemptions} preemptions, {eng.steps_ahead} steps launched ahead, graphs {sorted(eng.runner._graphs)}")
+    for r in reqs:
+        res = eng.pop_result(r["request_id"])
+        if res.finish_reason == "abort":
+            assert r["request_id"] == victim
+        else:
+            assert res.finish_reason == "length" and len(res.output) == r["max_new_tokens"]
+        assert len(res.logits) == len(res.output)
+        check_choices(d, res, dtype, r["sampling"])
+    assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
+    assert eng.runner.cache.slots.num_free == slots

@@ -101,6 +101,33 @@ def test_attention_reduces_to_library_softmax():
     assert torch.allclose(out, ref, rtol=1e-10)
 
 
+def test_attention_against_the_library_routine_with_groups_and_a_causal_mask():
+    """torch's own attention routine (no model code: one function of the tensor library), with
+    its causal mask and its grouping of query heads over key heads: scale 1/sqrt(d), which way
+    the mask faces, and q head h reading kv head h // (nq / nkv) in one comparison."""
+    F = torch.nn.functional
+    if "enable_gqa" not in (F.scaled_dot_product_attention.__doc__ or ""):
+        pytest.skip("this torch's attention routine has no grouped heads")
+    T, nq, nkv, d = 7, 6, 2, 8
+    q = torch.randn(T, nq, d, dtype=torch.float64)
+    k = torch.randn(T, nkv, d, dtype=torch.float64)
+    v = torch.randn(T, nkv, d, dtype=torch.float64)
+    out = P.plain_attention(q, k, v, list(range(T)))
+    ref = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None],
+                                         is_causal=True, enable_gqa=True)[0].transpose(0, 1)
+    assert torch.allclose(out, ref, rtol=1e-10, atol=1e-12)
+
+
+def test_rmsnorm_against_the_library_routine():
+    x = torch.randn(5, 24, dtype=torch.float64) * 3.0
+    w = torch.rand(24, dtype=torch.float64) + 0.5
+    if not hasattr(torch.nn.functional, "rms_norm"):
+        pytest.skip("this torch has no rms_norm routine")
+    for eps in (1e-6, 0.3):     # an eps large enough that its place (inside the root, on the mean) shows
+        ref = torch.nn.functional.rms_norm(x, (24,), w, eps)
+        assert torch.allclose(P.plain_rmsnorm(x, w, eps), ref, rtol=1e-12)
+
+
 def test_attention_single_key_and_uniform_scores():
     d = 4
     q = torch.randn(1, 2, d, dtype=torch.float64)

@@ -131,12 +131,13 @@ class DecodeTables:
                 base = o[9 + 2 * gi] + r * w
                 n = len(table)
                 old = prev[2][gi] if prev is not None else 0
-                grown = prev is not None and prev[0] == e.req and prev[1] == life \
-                    and cache.groups[gi].spec.window == 0 and n >= old
+                grown = prev is not None and prev[0] == e.req and prev[1] == life and n >= old
                 if grown:
-                    # same stay in the cache and a table that keeps all keys: it only grew
+                    # The same stay in the cache: the table only grew at its end.  (A window gives
+                    # pages back at the table's front; those entries stay as they are, no kernel
+                    # reads before the window's first key.)
                     if n > old:
-                        hv[base + old:base + n] = table[old:]
+                        hv[base + old:base + n] = [p if p >= 0 else 0 for p in table[old:]]
                 else:
                     hv[base:base + n] = [p if p >= 0 else 0 for p in table]
                     if old > n:
