@@ -56,6 +56,9 @@ def parse_args():
     ap.add_argument("--chunk", type=int, default=512, help="prompt portion of the --mixed workload")
     ap.add_argument("--budget", type=int, default=0,
                     help="tokens of a step of the --mixed workload (default: a portion beside every decoding request, at least 1,024)")
+    ap.add_argument("--token-quantum", type=int, default=None,
+                    help="with --mixed: the scheduler cuts steps a little over a multiple of this many tokens down "
+                         "to the multiple (default: the engine's own, 256; 0: off)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--ceilings", action="store_true",
                     help="measure streaming-read bandwidth, back-to-back MFMA rates and a large square product "
@@ -225,7 +228,7 @@ def main():
         opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=kv_tokens,
                             max_num_seqs=args.mixed, max_num_batched_tokens=args.budget or max(args.chunk + args.mixed, 1024),
                             prefill_chunk=args.chunk, max_model_len=cfg["max_position_embeddings"],
-                            use_graphs=not args.no_graphs)
+                            use_graphs=not args.no_graphs, token_quantum=args.token_quantum)
         engine = LLMEngine(model, opt)
         res = M.measure_mixed(engine, gen, args.mixed, vocab)
         print(json.dumps({"workload": "mixed", "model": shape_name, "layers_run": L, "chunk": args.chunk, **res}))

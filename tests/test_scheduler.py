@@ -331,3 +331,60 @@ def test_window_pool_sized_by_the_engine_never_preempts():
     run_all(sched, runner, cache)
     assert sched.stats.preemptions == 0
     assert all(r.output == expected_output(r.prompt, 40) for r in reqs)
+
+
+def test_a_step_a_little_over_a_multiple_of_the_quantum_is_cut_down_to_it():
+    """A quantum of 64 tokens: a portion of 64 beside 5 decoding requests makes 69 rows, a tile
+    row more than 64; the portion is cut to 59.  A prompt's last portion is never cut (its first
+    token would come a step later), nor is anything cut when the excess is more than a quarter
+    of the quantum, or when the step is below one quantum."""
+    cache = CacheManager([(0, True, SPEC, None)], 8, 200, 8)
+    sched = Scheduler(cache, SchedulerOptions(8, 256, 64, token_quantum=64), 1024)
+    runner = FakeRunner(cache)
+    short = [Request(i, [i + 1] * 3, max_new_tokens=40) for i in range(5)]
+    for r in short:
+        sched.add_request(r)
+    plan = sched.schedule()                      # five short prompts: 15 tokens, below a quantum
+    assert sum(p.count for p in plan) == 15
+    sched.update(plan, runner.run(plan))
+    long = Request("long", list(range(300)), max_new_tokens=8)
+    sched.add_request(long)
+    seen = []
+    while long.num_computed < 300:
+        plan = sched.schedule()
+        total = sum(p.count for p in plan)
+        portion = next(p for p in plan if p.request is long)
+        seen.append((total, portion.count, portion.samples))
+        sched.update(plan, runner.run(plan))
+        cache.check()
+    # 5 decodes + 64 = 69 -> 64 (59 of the prompt), four times; then the 64 tokens that are left: the
+    # prompt's last portion, uncut although 5 + 64 = 69 again
+    assert seen == [(64, 59, False)] * 4 + [(69, 64, True)]
+    run_all(sched, runner, cache)
+    assert long.output == expected_output(long.prompt, 8)
+    assert all(r.output == expected_output(r.prompt, 40) for r in short)
+    assert cache.groups[0].pool.num_used == 0
+    # an excess of more than a quarter of the quantum stays: 20 decodes + 64
+    cache = CacheManager([(0, True, SPEC, None)], 8, 400, 24)
+    sched = Scheduler(cache, SchedulerOptions(24, 256, 64, token_quantum=64), 1024)
+    runner = FakeRunner(cache)
+    for i in range(20):
+        sched.add_request(Request(i, [i + 1] * 2, max_new_tokens=30))
+    plan = sched.schedule()
+    sched.update(plan, runner.run(plan))
+    sched.add_request(Request("long", list(range(200)), max_new_tokens=4))
+    plan = sched.schedule()
+    assert sum(p.count for p in plan) == 84 and any(p.count == 64 for p in plan)
+    # and pages taken for the tokens cut away went back
+    cache = CacheManager([(0, True, SPEC, None)], 8, 50, 4)
+    sched = Scheduler(cache, SchedulerOptions(4, 256, 64, token_quantum=64), 1024)
+    runner = FakeRunner(cache)
+    for i in range(3):
+        sched.add_request(Request(i, [i + 1], max_new_tokens=30))
+    plan = sched.schedule()
+    sched.update(plan, runner.run(plan))
+    sched.add_request(Request("long", list(range(200)), max_new_tokens=4))
+    plan = sched.schedule()
+    assert sorted(p.count for p in plan) == [1, 1, 1, 61]
+    assert len(cache.block_table(0, "long")) == 8        # 61 tokens: eight pages of 8, not the nine of 64
+    cache.check()

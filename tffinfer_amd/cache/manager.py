@@ -181,11 +181,12 @@ class CacheManager:
         for n, g in zip(need, self.groups):
             g.tables[req].extend(g.pool.allocate(n))
 
-    def rollback(self, req) -> int:
-        """Gives back the pages that ``reserve`` took and no ``commit`` has filled (a step that
-        failed between the two); returns how many."""
+    def rollback(self, req, keep_new: int = 0) -> int:
+        """Gives back the pages that ``reserve`` took beyond what ``keep_new`` more tokens need
+        (none: a step that failed between ``reserve`` and ``commit``; some: a portion that was
+        cut down after its pages were taken); returns how many."""
         st = self.requests[req]
-        keep = -(-st.num_tokens // self.page_size)
+        keep = -(-(st.num_tokens + keep_new) // self.page_size)
         n = 0
         for g in self.groups:
             table = g.tables[req]

@@ -20,7 +20,7 @@ import numpy as np
 
 _ENGINE_KEYS = ("dtype", "device", "page_size", "num_pages", "kv_tokens", "kv_bytes", "max_num_seqs",
                 "max_num_batched_tokens", "prefill_chunk", "max_model_len", "memory_fraction", "use_graphs",
-                "run_ahead", "warm_up")
+                "run_ahead", "warm_up", "token_quantum")
 _SAMPLING_KEYS = ("type", "temperature", "top_k", "top_p", "min_p", "repetition_penalty", "seed")
 _REQUEST_KEYS = ("max_new_tokens", "eos_token_id", "ignore_eos", "sampling")
 

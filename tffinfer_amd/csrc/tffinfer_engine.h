@@ -47,7 +47,7 @@ typedef struct {
 
 // options_json: a JSON object with any of dtype ("bfloat16", "float32"), device, page_size,
 // num_pages | kv_tokens | kv_bytes, max_num_seqs, max_num_batched_tokens, prefill_chunk,
-// max_model_len, memory_fraction, use_graphs, run_ahead, warm_up; NULL or "" for the defaults.
+// max_model_len, memory_fraction, use_graphs, run_ahead, warm_up, token_quantum; NULL or "" for the defaults.
 // model_dir: a folder with config.json and model.safetensors; the model class is chosen by config.json.
 TFF_ENGINE_API tff_engine* engine_create(const char* model_dir, const char* options_json);
 // Seeded random weights for the configuration in config_json_file, no weight files.

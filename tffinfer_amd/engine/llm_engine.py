@@ -40,6 +40,9 @@ class EngineOptions:
     max_num_seqs: int = 8
     max_num_batched_tokens: int = 2048
     prefill_chunk: int = 512
+    #: steps a little over a multiple of this many tokens are cut down to the multiple (the
+    #: scheduler's rule 5); None: 256 for bfloat16 (the row tile of the matrix-core products), off for float32
+    token_quantum: int | None = None
     max_model_len: int | None = None
     memory_fraction: float = 0.85
     use_graphs: bool = True
@@ -92,9 +95,12 @@ class LLMEngine:
         self.runner = ModelRunner(model, page_size=opt.page_size, num_pages=num_pages,
                                   max_seqs=opt.max_num_seqs, max_model_len=max_len,
                                   use_graphs=opt.use_graphs)
+        quantum = opt.token_quantum
+        if quantum is None:
+            quantum = 256 if model.dtype == torch.bfloat16 else 0
         self.scheduler = Scheduler(self.runner.cache,
                                    SchedulerOptions(opt.max_num_seqs, opt.max_num_batched_tokens,
-                                                    opt.prefill_chunk), max_len)
+                                                    opt.prefill_chunk, int(quantum)), max_len)
         self.sampler = Sampler(model.device)
         self._ids = itertools.count()
         self.keep_logits = False

@@ -22,7 +22,14 @@ Rules of a step, in this order:
 3. waiting requests are admitted in arrival order while a slot is free, budget
    is left and pages for a first portion are free; the queue is not overtaken;
 4. if nothing at all could be scheduled although requests are running, the most
-   recently admitted one is preempted and the step is planned again.
+   recently admitted one is preempted and the step is planned again;
+5. with a ``token_quantum`` (the row tile of the products, 256 rows on the
+   matrix cores): a step whose tokens exceed a multiple of the quantum by a
+   little (a quarter of it at most) is cut down to the multiple, by shortening
+   the last prompt portion that does not end its prompt.  A step's time is a
+   staircase in its rows: at the 8B shape 512 rows take 9.0 ms and 520 rows
+   10.9 ms, so a portion of 512 beside 24 decoding requests is better cut to
+   488 tokens (the step a sixth shorter for a twentieth fewer prompt tokens).
 
 A request that could never fit the pool or the model's length is refused when
 it is added, with an error, not truncated: a group that keeps every key must
@@ -83,6 +90,8 @@ class SchedulerOptions:
     max_num_seqs: int = 8
     max_num_batched_tokens: int = 2048
     prefill_chunk: int = 512
+    #: > 0: steps a little over a multiple of this many tokens are cut down to the multiple (rule 5)
+    token_quantum: int = 0
 
 
 @dataclass
@@ -247,6 +256,18 @@ class Scheduler:
                     self._take(p.request, n, free)
                     budget -= n - p.count
                     plan[i] = ScheduledPortion(p.request, p.start, n, n == p.request.num_pending)
+        # 5. a step a little over a multiple of the quantum is cut down to the multiple
+        q = self.opt.token_quantum
+        total = sum(p.count for p in plan)
+        if q > 0 and total > q and 0 < total % q <= q // 4:
+            cut = total % q
+            for i in range(len(plan) - 1, -1, -1):
+                p = plan[i]
+                if not p.samples and p.count > cut:
+                    n = p.count - cut
+                    self.cache.rollback(p.request.id, keep_new=n)      # the pages of the tokens cut away
+                    plan[i] = ScheduledPortion(p.request, p.start, n, False)
+                    break
         return plan
 
     # ---- after the step --------------------------------------------------
