@@ -313,3 +313,59 @@ def test_a_step_that_fails_gives_its_pages_back(model_dirs, use_graphs, monkeypa
     rn.free_request("a")
     rn.free_request("b")
     assert all(g.pool.num_used == 0 for g in rn.cache.groups)
+
+
+@pytest.mark.parametrize("run_ahead", [False, True])
+def test_the_engine_goes_on_after_a_step_that_failed(model_dirs, run_ahead):
+    """A product refuses its operands in the middle of a prompt step, and again in a decode step
+    (launched ahead of the tokens of the step in flight, where that is on): step() raises, and
+    the engine, stepped on, gives every request the tokens of an undisturbed run."""
+    from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
+    from tffinfer_amd.kernels import lib, ops
+    d = model_dirs["A"]
+    V = read_config(d)["vocab_size"]
+    prompts = [random_tokens(n, V, 640 + n) for n in (30, 7, 19)]
+    sc = [SamplingConfig(), SamplingConfig("random", temperature=0.8, seed=3), SamplingConfig()]
+
+    class Failing:
+        calls, fail_at = 0, set()
+
+        def __getattr__(self, name):
+            real = getattr(ops, name)
+            if name != "linear":
+                return real
+
+            def linear(*a, **kw):
+                self.calls += 1
+                if self.calls in self.fail_at:
+                    raise lib.KernelError("made to fail")
+                return real(*a, **kw)
+            return linear
+
+    def run(fail_at):
+        opt = EngineOptions(dtype="float32", page_size=8, num_pages=40, max_num_seqs=3, max_num_batched_tokens=32,
+                            prefill_chunk=16, use_graphs=False, run_ahead=run_ahead)
+        eng = LLMEngine.from_model_dir(d, opt)
+        stub = Failing()
+        stub.fail_at = set(fail_at)
+        eng.runner.ops = stub
+        eng.keep_logits = True
+        ids = [eng.add_request(p, s, max_new_tokens=12, ignore_eos=True) for p, s in zip(prompts, sc)]
+        errors = 0
+        while eng.has_work:
+            try:
+                eng.step()
+            except lib.KernelError:
+                errors += 1
+            eng.runner.cache.check()
+        assert errors == len(fail_at)
+        res = [eng.pop_result(i) for i in ids]
+        assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
+        return res, stub.calls
+
+    clean, calls = run(())
+    # the tenth product lies in the first steps (prompts), one near the end in a decode step
+    broken, _ = run((10, calls - 40))
+    for a, b, s in zip(clean, broken, sc):
+        assert a.output == b.output and len(b.output) == 12
+        check_choices(d, b, "float32", s)

@@ -307,15 +307,24 @@ class LLMEngine:
                 return dropped
             st = self._launch(plan)
         nxt = self._plan_ahead(st)
+        failed = None
         if nxt is not None:
             src = st.tokens
             if len(nxt) != len(st.rows):          # some requests end with the token in flight
                 going = {id(p.request) for p in nxt}
                 src = self._take_rows(st.tokens, np.asarray([i for i, r in enumerate(st.rows) if id(r) in going],
                                                             dtype=np.int32))
-            self._ahead = self._launch(nxt, src)
-            self.steps_ahead += 1
-        return dropped + self._complete(st)
+            try:
+                self._ahead = self._launch(nxt, src)
+                self.steps_ahead += 1
+            except Exception as e:
+                # The step ahead did not run (its pages went back); the step in flight did and is
+                # completed first, so that scheduler and cache agree before the error is raised.
+                failed = e
+        done = dropped + self._complete(st)
+        if failed is not None:
+            raise failed
+        return done
 
     # ---- whole generations ----------------------------------------------
     def generate(self, prompts, sampling=None, max_new_tokens: int = 64, eos_token_id: int | None = None,
