@@ -91,7 +91,9 @@ def test_rmsnorm_eps_position():
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 320, 96), (33, 200, 200), (130, 130, 72), (257, 96, 256),
                                     (64, 4096, 512), (300, 1000, 1024), (50, 203, 1000), (40, 1024, 2056),
-                                    (100, 203, 2048), (520, 264, 1544)])
+                                    (100, 203, 2048), (520, 264, 1544),
+                                    # a little more groups of 16 columns than CUs: two groups a block (up to 16 rows)
+                                    (5, 5000, 1096), (16, 4100, 264), (1, 6544, 520), (3, 6560, 512)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_linear(M, N, K, dtype):
     ops = _ops()
@@ -111,7 +113,8 @@ def test_linear(M, N, K, dtype):
     _close(out_s, wide[:, :K].double().cpu() @ w.double().T, 2e-6 if dtype == torch.float32 else 2e-5, "strided")
 
 
-@pytest.mark.parametrize("M,N,K", [(40, 1024, 2056), (520, 264, 1544), (8, 64, 64), (8, 5120, 8192), (16, 5120, 8200)])
+@pytest.mark.parametrize("M,N,K", [(40, 1024, 2056), (520, 264, 1544), (8, 64, 64), (8, 5120, 8192), (16, 5120, 8200),
+                                    (16, 5120, 17408), (12, 5120, 25600)])
 def test_linear_partial_sums_feed_the_norm(M, N, K):
     """Where the product splits K over blocks it can hand out the partial sums; the fused
     residual sum and norm adds them up itself, in order, to what the whole product gives."""
@@ -122,12 +125,13 @@ def test_linear_partial_sums_feed_the_norm(M, N, K):
     pw = ops.pack_weight(w.to(DEV))
     whole = ops.linear(x, pw, out_dtype=torch.float32)
     parts = ops.linear(x, pw, out_dtype=torch.float32, partials=True)
-    # a few rows and 320 column groups: the whole product streams, the partial sums come from
-    # tiles that split K; the two kernels add in different orders
-    other_kernel = M <= 16 and N == 5120
+    # 9 to 16 rows, 320 column groups and a long K: the whole product streams, the partial sums come
+    # from tiles that split K; the two kernels add in different orders.  (Up to 8 rows, or with a
+    # shorter K, the streaming kernel gives a block two column groups and runs both.)
+    other_kernel = 8 < M <= 16 and N == 5120 and N * K >= 45e6
     same = (lambda a, b: torch.allclose(a.float(), b.float(), rtol=2e-2 if a.dtype == torch.bfloat16 else 1e-4,
                                         atol=2e-2 if a.dtype == torch.bfloat16 else 1e-3)) if other_kernel else torch.equal
-    if M == 8 and not other_kernel:
+    if M <= 16 and not other_kernel:
         assert isinstance(parts, ops.PendingProduct)   # a few rows: run by whoever consumes it
         assert torch.equal(parts.run(), whole)
     else:
@@ -151,7 +155,9 @@ def test_linear_partial_sums_feed_the_norm(M, N, K):
 @pytest.mark.parametrize("glu", [False, True])
 @pytest.mark.parametrize("M,H,K,N2", [(1, 64, 64, 96), (8, 4096, 4096, 6144), (5, 320, 96, 200), (16, 200, 1000, 72),
                                        (3, 1000, 256, 33000), (7, 4096, 12288, 24576), (16, 40, 8200, 136),
-                                       (16, 5120, 512, 51200), (11, 5120, 256, 49138), (2, 5120, 256, 51200)])
+                                       (16, 5120, 512, 51200), (11, 5120, 256, 49138), (2, 5120, 256, 51200),
+                                       # widths of a little more groups of 16 columns than CUs (two groups a block) and just past them
+                                       (9, 4112, 1000, 64), (8, 6544, 8200, 40), (16, 6544, 520, 40), (4, 6560, 512, 48), (8, 5120, 17408, 96)])
 def test_norm_taken_into_the_products_on_either_side(M, H, K, N2, glu):
     """Up to 16 rows: the product before a norm adds to the residual stream, writes (sum * norm
     weight) in bfloat16 and the sums of squares of its groups of 16 columns; the product after it
@@ -389,9 +395,11 @@ def test_gemm_plan():
         return r.value, c.value, s.value
 
     assert plan(8, 4096, 4096) == (0, 0, 1)
-    # a few rows, 320 column groups (two rounds for 64 CUs, one for the rest), partial sums wanted
-    # anyway and a weight large enough: tiles that split K instead of the streaming kernel
-    assert plan(8, 5120, 8192, keep=1)[0] in (64, 128) and plan(8, 5120, 8192, keep=1)[2] > 1
+    # 9 to 16 rows, 320 column groups (two rounds for 64 CUs, one for the rest), partial sums wanted
+    # anyway and a weight large enough: tiles that split K instead of the streaming kernel; up to 8
+    # rows, or with a weight that is not so large, the streaming kernel with two column groups a block
+    assert plan(12, 5120, 17408, keep=1)[0] in (64, 128) and plan(12, 5120, 17408, keep=1)[2] > 1
+    assert plan(8, 5120, 17408, keep=1) == (0, 0, 1) and plan(16, 5120, 8192, keep=1) == (0, 0, 1)
     assert plan(8, 5120, 8192) == (0, 0, 1) and plan(8, 5120, 5120, keep=1) == (0, 0, 1)
     assert plan(8, 4096, 12288, keep=1) == (0, 0, 1)
     assert plan(64, 4096, 12288) == (64, 128, 8)

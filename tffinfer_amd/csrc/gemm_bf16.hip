@@ -748,7 +748,7 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
     int K, int lda, int KB, int n_out, SkinnyFuse fz) {
     static_assert(EPI == 0 || MT == 1, "the fused norm is for up to 16 rows");
-    static_assert(EPI != 2 || (!GLU && R == 1), "the product before a norm has a plain float32 result");
+    static_assert(EPI != 2 || !GLU, "the product before a norm has a plain float32 result");
     constexpr int SK_WAVES = KSPLIT * NSETS;
     static_assert(!GLU || (R == 1 && NSETS % 2 == 0), "a gate and its up group are one row group each");
     __shared__ floatx4 part[SK_WAVES][R * MT][64];
@@ -781,7 +781,9 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
     // What the epilogue needs from memory is asked for first, so that it has arrived long
     // before the stream of W ends.
     float row_scale = 1.f;
-    float4 resid_in = make_float4(0.f, 0.f, 0.f, 0.f), normw_in = resid_in;
+    float4 resid_in[R], normw_in[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) resid_in[r] = normw_in[r] = make_float4(0.f, 0.f, 0.f, 0.f);
     // EPI 1: lane (fr, fg) of a set's first wave adds every fourth group of four sums of row fr,
     // then the four lanes of a row meet: the same order in every block.  The loads are issued
     // here, ahead of the stream of W, and added up (TFF_ROW_SCALE) when that stream has ended.
@@ -821,10 +823,13 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
     }
     if constexpr (EPI == 2) {
         if (wave == 0) {
-            const int n = nb0 * 16 + fg * 4;
-            if (fr < M && n < N) {
-                resid_in = *reinterpret_cast<const float4*>(fz.resid + (size_t)fr * N + n);
-                normw_in = *reinterpret_cast<const float4*>(fz.norm_w + n);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int n = (nb0 + r) * 16 + fg * 4;
+                if (fr < M && n < N) {
+                    resid_in[r] = *reinterpret_cast<const float4*>(fz.resid + (size_t)fr * N + n);
+                    normw_in[r] = *reinterpret_cast<const float4*>(fz.norm_w + n);
+                }
             }
         }
     }
@@ -954,14 +959,14 @@ __global__ __launch_bounds__(64 * KSPLIT * NSETS) void gemm_bf16_skinny_kernel(
                         // N is a multiple of 4 here: four columns are in or out together
                         float ss = 0.f;
                         if (m < M && n < N) {
-                            const float4 sum = make_float4(resid_in.x + v[0], resid_in.y + v[1],
-                                                           resid_in.z + v[2], resid_in.w + v[3]);
+                            const float4 sum = make_float4(resid_in[r].x + v[0], resid_in[r].y + v[1],
+                                                           resid_in[r].z + v[2], resid_in[r].w + v[3]);
                             *reinterpret_cast<float4*>(fz.resid + (size_t)m * N + n) = sum;
                             union { bf16_t h[4]; uint2 u; } pk;
-                            pk.h[0] = (bf16_t)(sum.x * normw_in.x);
-                            pk.h[1] = (bf16_t)(sum.y * normw_in.y);
-                            pk.h[2] = (bf16_t)(sum.z * normw_in.z);
-                            pk.h[3] = (bf16_t)(sum.w * normw_in.w);
+                            pk.h[0] = (bf16_t)(sum.x * normw_in[r].x);
+                            pk.h[1] = (bf16_t)(sum.y * normw_in[r].y);
+                            pk.h[2] = (bf16_t)(sum.z * normw_in[r].z);
+                            pk.h[3] = (bf16_t)(sum.w * normw_in[r].w);
                             *reinterpret_cast<uint2*>(fz.x_out + (size_t)m * N + n) = pk.u;
                             ss = fmaf(sum.x, sum.x, fmaf(sum.y, sum.y, fmaf(sum.z, sum.z, sum.w * sum.w)));
                         }
@@ -1013,6 +1018,13 @@ static int device_cus() {
     }
     return cached[dev];
 }
+// Up to 16 rows, not gated: more row groups of 16 columns than CUs, but at most 1.6 times as many
+// (a second round of blocks that would be less than 0.6 full): the streaming kernel then gives a block
+// two row groups (skinny_for).
+static bool two_row_groups(int N) {
+    const int nb = (N + 15) / 16, cus = device_cus();
+    return nb > cus && nb * 10 <= cus * 16;
+}
 // Up to 16 rows, gated, a very large weight (the 32B shape's gate+up, 262M elements): the streaming
 // kernel's blocks each fetch all of A's rows, and with so many blocks that is traffic enough to show:
 // 94 us against 90 on tiles with one row, 115 against 90 with 16.  Then tiles of 128 rows of the
@@ -1051,6 +1063,8 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
         const int nb = (N + 15) / 16;
         const double fill = (double)nb / (ceil(nb / CUS) * CUS);
         if (glu || !keep || fill >= 0.8 || (double)N * K < 40e6) return {0, 0, 1};
+        // (two row groups a block: ahead of the tiles up to 8 rows, and up to 16 where K is short)
+        if (two_row_groups(N) && (M <= 8 || (double)N * K < 45e6)) return {0, 0, 1};
     }
     const int nk = (K + 63) / 64;
     if (K % 64 == 0) {
@@ -1168,6 +1182,17 @@ static int skinny_for(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, 
         } else {
             return tff_fail("gemm: a gated product does not come before a norm");
         }
+    }
+    // A block per 16 columns goes badly round the CUs when there are a little more row groups than
+    // CUs (320 of them, N = 5120, take as long as 512 would).  Then a block takes two row groups:
+    // half as many blocks, all at once, and between them they still pull what HBM gives (some 130
+    // CUs do).  Measured at N = 5120 against tiles that split K with a norm kernel to add their
+    // parts: O of the 14B shape 11.9 / 14.1 / 16.7 us at 1 / 8 / 16 rows against 13.7 / 15.1 / 19.0,
+    // of the 32B shape 20.4 / 21.6 / 24.0 against 27.2 / 27.4 / 27.5; down of the 14B shape 33.4 /
+    // 39.8 against 42.9 / 42.8 at 1 / 8 rows (at 16 rows the tiles are ahead, see plan_for).  Not for
+    // the product after a norm: the row factors' registers do not fit beside two row groups.
+    if constexpr (EPI != 1) {
+        if (two_row_groups(N)) return launch_skinny<1, 2, 4, 16, 1, false, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, fuse);
     }
     // (K up to 1,024: sixteen waves would have two k-steps each, less than a group of four)
     if (N >= 32 * 1024 || K <= 1024)
