@@ -113,6 +113,21 @@ def test_linear(M, N, K, dtype):
     _close(out_s, wide[:, :K].double().cpu() @ w.double().T, 2e-6 if dtype == torch.float32 else 2e-5, "strided")
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 33000, 2560), (10, 40000, 4096), (3, 33000, 512)])
+def test_linear_very_wide(M, N, K):
+    """An output head's shape: thousands of groups of 16 columns; with many rows and a long K a block
+    of the streaming kernel takes two groups (the last case: one)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(M + N)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) * 0.1).to(torch.bfloat16)
+    ref = x.double() @ w.double().T
+    out = ops.linear(x.to(DEV), _w(w), out_dtype=torch.float32)
+    _close(out, ref, 2e-5, f"linear {M}x{N}x{K}")
+    for m in range(M):
+        _close(out[m], ref[m], 2e-5, f"row {m}")
+
+
 @pytest.mark.parametrize("M,N,K", [(40, 1024, 2056), (520, 264, 1544), (8, 64, 64), (8, 5120, 8192), (16, 5120, 8200),
                                     (16, 5120, 17408), (12, 5120, 25600)])
 def test_linear_partial_sums_feed_the_norm(M, N, K):

@@ -1194,6 +1194,14 @@ static int skinny_for(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, 
     if constexpr (EPI != 1) {
         if (two_row_groups(N)) return launch_skinny<1, 2, 4, 16, 1, false, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, fuse);
     }
+    // A very wide product (an output head) has thousands of blocks, each of which fetches all of A's
+    // rows: with many rows and a long K that traffic shows (152k columns, K = 4,096: 196 / 217 / 281 us
+    // at 1 / 8 / 16 rows).  Two groups of 16 columns a block halve it: 243 us at 16 rows, K = 5,120 at
+    // 8 / 16 rows 264 / 303 us against 278 / 366; with fewer rows one group a block stays ahead.
+    if constexpr (EPI == 0) {
+        if (N >= 32 * 1024 && (long)M * K >= 40000)
+            return launch_skinny<1, 2, 4, 8, 1, false, false, 0>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, fuse);
+    }
     // (K up to 1,024: sixteen waves would have two k-steps each, less than a group of four)
     if (N >= 32 * 1024 || K <= 1024)
         return launch_skinny<1, 1, 4, 8, 1, false, false, EPI>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, fuse);
