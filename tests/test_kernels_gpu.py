@@ -172,6 +172,8 @@ def test_linear_partial_sums_feed_the_norm(M, N, K):
                                        (3, 1000, 256, 33000), (7, 4096, 12288, 24576), (16, 40, 8200, 136),
                                        (16, 5120, 512, 51200), (11, 5120, 256, 49138), (2, 5120, 256, 51200),
                                        # widths of a little more groups of 16 columns than CUs (two groups a block) and just past them
+                                       # gated on tiles of 128 rows from fewer elements on where there are more rows
+                                       (12, 5120, 256, 34816), (16, 4096, 128, 24576), (14, 4096, 128, 24576),
                                        (9, 4112, 1000, 64), (8, 6544, 8200, 40), (16, 6544, 520, 40), (4, 6560, 512, 48), (8, 5120, 17408, 96)])
 def test_norm_taken_into_the_products_on_either_side(M, H, K, N2, glu):
     """Up to 16 rows: the product before a norm adds to the residual stream, writes (sum * norm

@@ -1030,9 +1030,13 @@ static bool two_row_groups(int N) {
 // 94 us against 90 on tiles with one row, 115 against 90 with 16.  Then tiles of 128 rows of the
 // four-wave kernel, K in one part.  (At the 8B and 14B shapes' sizes tiles gain only with K in two
 // parts, which the rows' factors in the epilogue do not go with: the streaming kernel stays.)
+// The streaming kernel's time also grows with the rows (every block fetches them all), the tiles' does
+// not, so smaller weights cross over at more rows: gate+up of the 14B shape (1.8e8 elements) 67 / 71 /
+// 78 / 87 us at 1 / 8 / 12 / 16 rows against 75 on tiles, of the 8B shape (1.0e8) 37 / 38 / 40 / 44 us
+// against 43, of the 4B shape (5e7) 21 / 22 / 25 / 28 against 28.
 static bool few_rows_gated_on_tiles(int M, int N, int K) {
-    (void)M;
-    return K % 64 == 0 && (double)N * K >= 2.4e8;
+    const double w = (double)N * K;
+    return K % 64 == 0 && (w >= 2.4e8 || (w >= 1.6e8 && M >= 11) || (w >= 0.9e8 && M >= 15));
 }
 // One row tile of 128 rows, K in one part: the width (128, 256 or 384 columns) that plan_for's model prices lowest.
 static int plan_rows128(int N, int K) {
