@@ -15,6 +15,8 @@ from tffinfer_amd.engine.graphs import DecodeTables, graph_buckets
 from tffinfer_amd.engine.scheduler import Request, Scheduler, SchedulerOptions
 from tffinfer_amd.parts.base import KVCacheSpec
 
+from test_key_runs import check_runs
+
 FULL = KVCacheSpec(2, 16, 0)
 WIN = KVCacheSpec(2, 16, 16)
 
@@ -33,11 +35,16 @@ def check_rows(tables: DecodeTables, cache, entries):
             for b in range(first_live, len(true)):
                 assert row[b] == true[b], (f"row {r} request {e.req!r} group {gi} block {b}: "
                                            f"graph says {row[b]}, the cache {true[b]}")
-            assert hv[o[10 + 2 * gi] + r] == true[P // ps] * ps + P % ps
+            assert hv[o[10 + 4 * gi] + r] == true[P // ps] * ps + P % ps
     for r in range(len(entries), tables.B):       # padding writes no key and reads position 0 only
         assert hv[o[5] + r] == 1 and hv[o[1] + r] == 0
         for gi in range(len(cache.groups)):
-            assert hv[o[10 + 2 * gi] + r] == -1
+            assert hv[o[10 + 4 * gi] + r] == -1
+    # the keys of every row, padding included, dealt into runs: each visible key in exactly one
+    for gi, g in enumerate(cache.groups):
+        cap = tables.run_caps[gi]
+        check_runs(hv[o[11 + 4 * gi]:o[11 + 4 * gi] + 4 * cap].reshape(-1, 4), hv[o[12 + 4 * gi]:o[12 + 4 * gi] + tables.B + 1],
+                   hv[o[4]:o[4] + tables.B], g.spec.window)
 
 
 class TableRunner:

@@ -935,7 +935,11 @@ def test_attention_mfma_decode_split_keys(nq, nkv, d, ps, window, splits):
     (16, 1, 64, 32, 0, 64, "half"), (4, 2, 192, 16, 0, 3, "half"), (2, 1, 256, 8, 0, None, "half"),
     # splits 0: a block of eight waves per entry and kv head, merged in LDS
     (32, 8, 128, 16, 0, 0, "half"), (4, 2, 16, 16, 0, 0, "interleaved"), (8, 2, 32, 8, 24, 0, "interleaved"),
-    (40, 2, 96, 8, 0, 0, "interleaved"), (6, 3, 48, 8, 100, 0, "interleaved"), (16, 1, 112, 32, 0, 0, "interleaved")])
+    (40, 2, 96, 8, 0, 0, "interleaved"), (6, 3, 48, 8, 100, 0, "interleaved"), (16, 1, 112, 32, 0, 0, "interleaved"),
+    # the entries' keys dealt into runs by the host, for so many waves
+    (32, 8, 128, 16, 0, "runs 768", "half"), (4, 2, 16, 16, 0, "runs 64", "interleaved"),
+    (8, 2, 32, 8, 24, "runs 100", "interleaved"), (40, 2, 96, 8, 0, "runs 30", "interleaved"),
+    (6, 3, 48, 8, 100, "runs 1000", "interleaved"), (4, 2, 192, 16, 0, "runs 16", "half"), (2, 1, 256, 8, 0, "runs 5", "half")])
 def test_attention_decode_fused(nq, nkv, d, ps, window, splits, pairing, with_norm, with_rope):
     """Decode steps from the raw projection output: q/k norm, rotation, the token's key and value
     into its page and attention in one kernel, against each part's formula; the slot of the new
@@ -1005,8 +1009,15 @@ def test_attention_decode_fused(nq, nkv, d, ps, window, splits, pairing, with_no
     kv.k_cache, kv.v_cache = kc0.to(DEV), vc0.to(DEV)
     w = (None if qw is None else qw.to(DEV), None if kw is None else kw.to(DEV))
     assert ops.decode_fused_supported(qkv.to(DEV), d, ps, table, pr, batch)
+    how = dict(splits=splits)
+    if isinstance(splits, str):
+        from tffinfer_amd.engine.key_runs import deal_key_runs
+        runs, run_start = deal_key_runs([P for P, _ in entries], window, nkv, target=int(splits.split()[1]), min_steps=1)
+        assert run_start[-1] > R, "no entry has several runs"
+        how = dict(key_runs=torch.from_numpy(runs.copy()).to(DEV), run_start=torch.from_numpy(run_start.copy()).to(DEV))
+        splits = None
     out = ops.attention_decode_fused(qkv.to(DEV), nq, nkv, d, w[0], w[1], eps, table, pr, kv, batch, window, scale,
-                                     slot_mapping=slots, splits=splits)
+                                     slot_mapping=slots, **how)
     _close(out.reshape(R, nq, d), ref, ATTN_TOL, "fused decode attention")
     kc1, vc1 = kv.k_cache.cpu(), kv.v_cache.cpu()
     expect_k, expect_v = kc0.clone(), vc0.clone()
@@ -1020,7 +1031,7 @@ def test_attention_decode_fused(nq, nkv, d, ps, window, splits, pairing, with_no
     assert torch.equal(kc1, expect_k) and torch.equal(vc1, expect_v), "a slot of another token was written"
     # a call that only reads: the pages hold the tokens already
     out2 = ops.attention_decode_fused(qkv.to(DEV), nq, nkv, d, w[0], w[1], eps, table, pr, kv, batch, window, scale,
-                                      slot_mapping=None, splits=splits)
+                                      slot_mapping=None, **how)
     assert torch.equal(kv.k_cache.cpu(), kc1) and torch.equal(kv.v_cache.cpu(), vc1)
     _close(out2.reshape(R, nq, d), ref, ATTN_TOL, "fused decode attention, cache read only")
     # the two-kernel path gives the same to rounding
@@ -1079,6 +1090,59 @@ def test_attention_decode_fused_blocks_of_eight_waves_over_long_contexts(d, ps, 
     b = ops.attention_decode_fused(qkv2.to(DEV), nq, nkv, d, None, None, 1e-6, None, 0, kv2, batch2, window, scale,
                                    slot_mapping=None, splits=0)
     assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("nq,nkv,d,ps,window,waves,blocks", [
+    (8, 2, 32, 8, 0, 768, False), (8, 2, 128, 16, 0, 64, False), (16, 2, 64, 8, 5000, 200, False), (34, 2, 64, 16, 0, 96, False),
+    (4, 4, 256, 32, 0, 768, False), (8, 8, 128, 128, 700, 768, False),
+    # a block of eight waves per run and kv head
+    (8, 2, 32, 8, 0, 64, True), (8, 2, 128, 16, 0, 40, True), (16, 2, 64, 8, 5000, 96, True), (8, 8, 112, 128, 700, 256, True)])
+def test_attention_decode_fused_keys_dealt_into_runs(nq, nkv, d, ps, window, waves, blocks):
+    """Entries of very different lengths with their keys dealt into runs by the host, as the engine
+    deals them (the long entry is many runs, most others one, which write their result themselves;
+    a wave with more pages than it keeps at hand works through them in segments; a kv head with
+    more than sixteen query heads has several column tiles; a wave per run, or a block of eight
+    that split the run among them), one key far back made to dominate,
+    the token's own key and value from registers and into their page.  Tables with runs that are
+    not in use, and with a padding row's run, as a captured step has them."""
+    ops = _ops()
+    from tffinfer_amd.engine.key_runs import deal_key_runs
+    far = 77
+    entries = [(20000, 1), (40, 1), (0, 1), (95, 1), (96, 1), (3000, 1), (255, 1), (256, 1), (31, 1), (32, 1), (1023, 1)]
+    batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=3 + d)
+    R = len(entries)
+    g = torch.Generator().manual_seed(7)
+    qkv = torch.randn(R, (nq + 2 * nkv) * d, generator=g).to(torch.bfloat16)
+    q = qkv[:, :nq * d].reshape(R, nq, d)
+    k_new = qkv[:, nq * d:(nq + nkv) * d].reshape(R, nkv, d)
+    v_new = qkv[:, (nq + nkv) * d:].reshape(R, nkv, d)
+    if window == 0:
+        kfar = (30 * q[0, 0].float() / q[0, 0].float().norm()).to(torch.bfloat16)
+        kv.k_cache[int(kv.block_tables[0, far // ps]), 0, far % ps] = kfar.to(DEV)
+        ks[0][far, 0] = kfar
+    scale = 1 / math.sqrt(d)
+    bt = kv.block_tables.cpu()
+    slots = torch.tensor([int(bt[r, P // ps]) * ps + P % ps for r, (P, _) in enumerate(entries)], dtype=torch.int32, device=DEV)
+    refs = []
+    for r, (P, _) in enumerate(entries):
+        k = torch.cat([ks[r][:P], k_new[r:r + 1]])
+        v = torch.cat([vs[r][:P], v_new[r:r + 1]])
+        refs.append(_attn_ref(q[r:r + 1], k, v, positions[r:r + 1], window, scale)[0])
+    ref = torch.stack(refs)
+    runs, run_start = deal_key_runs([P for P, _ in entries], window, nkv, target=waves, blocks=blocks)
+    counts = run_start[1:] - run_start[:-1]
+    assert counts[0] > 4 and (counts == 1).sum() >= 6 and (runs[:, 0] == -1).any()
+    out = ops.attention_decode_fused(qkv.to(DEV), nq, nkv, d, None, None, 1e-6, None, 0, kv, batch, window, scale,
+                                     slot_mapping=slots, key_runs=torch.from_numpy(runs.copy()).to(DEV),
+                                     run_start=torch.from_numpy(run_start.copy()).to(DEV), runs_for_blocks=blocks)
+    _close(out.reshape(R, nq, d), ref, ATTN_TOL, "keys dealt into runs")
+    if window == 0:
+        assert torch.allclose(out.reshape(R, nq, d)[0, 0].float().cpu(), vs[0][far, 0].float(), atol=5e-2)
+    for r, (P, _) in enumerate(entries):
+        assert torch.equal(kv.v_cache[int(bt[r, P // ps]), :, :, P % ps].cpu(), v_new[r]), f"value of entry {r} in its page"
+    # what the kernel picks by itself (every entry's keys split alike) agrees to rounding
+    same = ops.attention_decode_fused(qkv.to(DEV), nq, nkv, d, None, None, 1e-6, None, 0, kv, batch, window, scale)
+    _close(out.reshape(R, nq, d), same.reshape(R, nq, d).double().cpu(), ATTN_TOL, "runs against equal splits")
 
 
 @pytest.mark.parametrize("nq,nkv,d,ps,window", [(32, 8, 128, 16, 0), (8, 2, 32, 8, 300), (40, 2, 96, 8, 0)])

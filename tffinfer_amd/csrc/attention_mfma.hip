@@ -73,6 +73,10 @@ struct AttnFuse {
     const int32_t* slot_mapping;   // per token; a negative entry: this token's key and value are not written
     float eps;
     int pairing;
+    // Runs of keys dealt by the host (null: the launch splits every entry's keys alike): run i is
+    // (entry, first key, end of keys, the entry's position), 16 bytes, and gets a wave per kv head.
+    // An entry of negative number: the run is not in use.
+    const int32_t* key_runs;
 };
 
 // RMS norm over the head and rotation of one head held as MFMA operand fragments: lane group kg
@@ -177,19 +181,40 @@ __global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
             __builtin_amdgcn_wave_barrier();
         }
     };
-    int r, col0;
-    if (work) {
+    // Runs dealt by the host: a grid of one dimension over (run, kv head), a multiple of eight
+    // runs, in this order: eight runs by eight, within them the kv heads, within a kv head the
+    // eight runs.  Blocks go to the XCDs in turn by their number, so run i is on XCD i % 8 with
+    // all its kv heads: the runs of a long entry, which follow each other, land on all XCDs
+    // (splitting every entry alike puts all waves of an entry on the one XCD that the entry's
+    // number selects), and a page of keys is read through one XCD's L2 and address translation,
+    // not through all eight.  The runs that are not in use come last, after every wave with work
+    // has its place: strewn among the others they took places on half of the CUs and left the
+    // waves with work crowded on the other half (a fifth slower at 64 entries of one run each).
+    bool by_runs = false;
+    if constexpr (FUSED && (SPLIT || BW > 1)) by_runs = fz.key_runs != nullptr;
+    int r, col0, g = blockIdx.y, run_index = 0;
+    int4 run = make_int4(0, 0, 0, 0);
+    if (by_runs) {
+        const int eight = blockIdx.x / (8 * nkv), within = blockIdx.x - eight * (8 * nkv);
+        run_index = eight * 8 + (within & 7);
+        g = within >> 3;
+        run = reinterpret_cast<const int4*>(fz.key_runs)[run_index];
+        r = run.x;
+        if (r < 0) return;
+        col0 = blockIdx.z * 16;
+    } else if (work) {
         r = work[2 * blockIdx.x];
         col0 = work[2 * blockIdx.x + 1];
     } else {
         r = blockIdx.x / tiles_per_entry;
         col0 = (blockIdx.x % tiles_per_entry) * 16;
     }
-    const int g = blockIdx.y;
     const int G = nq / nkv;
-    const int tok0 = cu_tokens[r];
-    const int n = cu_tokens[r + 1] - tok0;
-    const int P = start_pos[r];
+    // (a run brings its entry's position with it, and its entry has one token: nothing to wait
+    // for between the run and the page numbers)
+    const int tok0 = by_runs ? r : cu_tokens[r];
+    const int n = by_runs ? 1 : cu_tokens[r + 1] - tok0;
+    const int P = by_runs ? run.w : start_pos[r];
     const int ncols = n * G;
     const int32_t* bt = block_tables + (size_t)r * bt_stride;
 
@@ -209,13 +234,22 @@ __global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
     const int kb0 = (kmin / 32) * 32;
     const int nsteps = (kmax - kb0) / 32 + 1;
     int s_begin = 0, s_end = nsteps;
-    if constexpr (BW > 1) {
-        // (never under 96 keys a wave, as below)
-        const int per = max((nsteps + BW - 1) / BW, min(3, nsteps));
-        s_begin = min(nsteps, wv * per);
-        s_end = min(nsteps, s_begin + per);
+    if (by_runs) {
+        s_begin = min(nsteps, max(0, (run.y - kb0) >> 5));
+        s_end = min(nsteps, max(s_begin, (run.z - kb0 + 31) >> 5));
     }
-    if (SPLIT) {
+    // (an entry whose keys are one run has its result from that run's wave or block, no partial one;
+    // runs neither overlap nor leave a gap)
+    const bool run_is_partial = by_runs && (s_begin > 0 || s_end < nsteps);
+    if constexpr (BW > 1) {
+        // the block's keys (all of the entry's, or its run) among its waves, never under 96 keys a
+        // wave, as below
+        const int lo = s_begin, hi = s_end;
+        const int per = max((hi - lo + BW - 1) / BW, min(3, hi - lo));
+        s_begin = min(hi, lo + wv * per);
+        s_end = min(hi, s_begin + per);
+    }
+    if (SPLIT && !by_runs) {
         // The launch is sized for the longest context the engine allows; with shorter ones a run
         // of keys is not made shorter than 256 keys as long as some 256 waves are left with
         // work (the other waves of the launch end at once; their partial results are empty), and
@@ -520,6 +554,12 @@ __global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
         }
         const float inv = 1.0f / lsum;
         bf16_t* op = out + ((size_t)c_tok * nq + c_head) * D;
+        // (a run of an entry that has several: the block's result is a partial one, kept by run)
+        const size_t prow = (size_t)run_index * nq + c_head;
+        if (run_is_partial && wv == 0 && kg == 0) {
+            part_ml[prow * 2] = m;
+            part_ml[prow * 2 + 1] = lsum;
+        }
         for (int dt = wv; dt < DT; dt += BW) {
             float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
@@ -529,6 +569,10 @@ __global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
                 acc.y = fmaf(o.y, wgt[w], acc.y);
                 acc.z = fmaf(o.z, wgt[w], acc.z);
                 acc.w = fmaf(o.w, wgt[w], acc.w);
+            }
+            if (run_is_partial) {
+                *reinterpret_cast<float4*>(part_o + prow * D + dt * 16 + kg * 4) = acc;
+                continue;
             }
             union { bf16_t h[4]; uint2 u; } pk;
             pk.h[0] = (bf16_t)(acc.x * inv);
@@ -540,9 +584,10 @@ __global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
         return;
     }
     if (!c_ok) return;
-    if (SPLIT) {
-        // keys are split for entries of one token only: partial results are kept by entry
-        const size_t row = ((size_t)blockIdx.z * T_total + r) * nq + c_head;
+    const bool partial = by_runs ? run_is_partial : SPLIT;
+    if (partial) {
+        // keys are split for entries of one token only: partial results are kept by entry, or by run
+        const size_t row = by_runs ? (size_t)run_index * nq + c_head : ((size_t)blockIdx.z * T_total + r) * nq + c_head;
         float* po = part_o + row * D;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -663,6 +708,89 @@ __global__ __launch_bounds__(256) void attn_split_reduce_few_kernel(const float*
 #pragma unroll
     for (int e = 0; e < 4; ++e)
         if (lane + 64 * e < d) o[lane + 64 * e] = (bf16_t)(acc[e] * inv);
+}
+
+// The same for runs of keys dealt by the host: entry r has the runs run_start[r] ..
+// run_start[r + 1] - 1, any number of them, their partial results one after the other.  One wave
+// per (entry, head), four to a block; an entry of one run has its result already.  The first
+// sixteen runs' elements are asked for together with the maxima and sums (lane s takes those of
+// run s, s + 64, ...), the weights of those runs then come from the lanes that hold them; further
+// runs are fetched sixteen at a time, every lane reading their maxima and sums itself (one address
+// for the whole wave).  Every lane adds up its own elements of the head in the order of the runs.
+__global__ __launch_bounds__(256) void attn_run_merge_kernel(const float* __restrict__ part_o,
+                                                              const float* __restrict__ part_ml,
+                                                              bf16_t* __restrict__ out,
+                                                              const int32_t* __restrict__ run_start,
+                                                              int R, int nq, int d) {
+    const int lane = threadIdx.x & 63;
+    const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);     // (entry, head), heads fastest
+    if (pair >= R * nq) return;
+    const int r = pair / nq, h = pair - r * nq;
+    const int first = run_start[r], count = run_start[r + 1] - first;
+    if (count <= 1) return;
+    const size_t stride_ml = (size_t)nq * 2, stride_o = (size_t)nq * d;
+    const float* ml = part_ml + ((size_t)first * nq + h) * 2;
+    const float* po = part_o + ((size_t)first * nq + h) * d;
+    constexpr int AHEAD = 16;
+    const int e0 = 2 * lane, e1 = 128 + 2 * lane;             // d <= 256 and even: up to two pairs of elements a lane
+    float ms0 = -INFINITY, ls0 = 0.f, m = -INFINITY;
+    if (lane < count) {
+        ms0 = ml[lane * stride_ml];
+        ls0 = ml[lane * stride_ml + 1];
+        m = ms0;
+    }
+    float2 v[AHEAD][2];
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+        const size_t o = (size_t)min(u, count - 1) * stride_o;
+        v[u][0] = e0 < d ? *reinterpret_cast<const float2*>(po + o + e0) : make_float2(0.f, 0.f);
+        v[u][1] = e1 < d ? *reinterpret_cast<const float2*>(po + o + e1) : make_float2(0.f, 0.f);
+    }
+    for (int s = lane + 64; s < count; s += 64) m = fmaxf(m, ml[s * stride_ml]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    const float w0 = ms0 == -INFINITY ? 0.f : __expf(ms0 - m);   // (a lane past the last run: 0)
+    float l = 0.f;
+    float2 acc[2] = {make_float2(0.f, 0.f), make_float2(0.f, 0.f)};
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+        const float w = __shfl(w0, u, 64);
+        l = fmaf(__shfl(ls0, u, 64), w, l);
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            acc[k].x = fmaf(v[u][k].x, w, acc[k].x);
+            acc[k].y = fmaf(v[u][k].y, w, acc[k].y);
+        }
+    }
+    for (int s0 = AHEAD; s0 < count; s0 += AHEAD) {
+        float w[AHEAD];
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u) {
+            const int s = min(s0 + u, count - 1);
+            const float ms = ml[s * stride_ml];
+            w[u] = (s0 + u < count && ms != -INFINITY) ? __expf(ms - m) : 0.f;
+            l = fmaf(ml[s * stride_ml + 1], w[u], l);
+            v[u][0] = e0 < d ? *reinterpret_cast<const float2*>(po + s * stride_o + e0) : make_float2(0.f, 0.f);
+            v[u][1] = e1 < d ? *reinterpret_cast<const float2*>(po + s * stride_o + e1) : make_float2(0.f, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u)
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                acc[k].x = fmaf(v[u][k].x, w[u], acc[k].x);
+                acc[k].y = fmaf(v[u][k].y, w[u], acc[k].y);
+            }
+    }
+    const float inv = 1.0f / l;
+    bf16_t* o = out + ((size_t)r * nq + h) * d;
+    if (e0 < d) {
+        o[e0] = (bf16_t)(acc[0].x * inv);
+        o[e0 + 1] = (bf16_t)(acc[0].y * inv);
+    }
+    if (e1 < d) {
+        o[e1] = (bf16_t)(acc[1].x * inv);
+        o[e1 + 1] = (bf16_t)(acc[1].y * inv);
+    }
 }
 
 __device__ __forceinline__ float max3_raw(float a, float b, float c) {
@@ -1069,19 +1197,24 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
         return tff_check_launch("attention_mfma_block");
     }
     const dim3 grid(num_work, nkv, max(splits, 1));
-    const AttnFuse fz = fuse ? *fuse : AttnFuse{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
+    const AttnFuse fz = fuse ? *fuse : AttnFuse{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0, nullptr};
 #define TFF_ATTN_ARGS                                                                              \
     q, q_stride, out, part_o, part_ml, k_cache, v_cache, block_tables, bt_stride, cu_tokens,       \
         start_pos, work, tiles_per_entry, nq, nkv, page_size, page_shift, window, scale, T_total
     if (fuse && splits == 0) {
-        // a block of eight waves per entry and kv head: the keys split among its waves, merged in LDS
+        // a block of eight waves per entry (or run of keys dealt by the host) and kv head: the keys split
+        // among its waves, merged in LDS
         if constexpr (DT <= 8) {
             // (two waves to a SIMD have 256 registers each: four steps of keys and values in flight a wave up to
             // a head size of 64, two up to 96, one beyond; eight waves keep a CU's 100 GB/s busy either way)
-            attn_wave_kernel<DT, false, (DT <= 4 ? 4 : DT <= 6 ? 2 : 1), true, 8><<<dim3(num_work, nkv, 1), 512, 0, s>>>(TFF_ATTN_ARGS, fz);
+            const dim3 bgrid = fuse->key_runs ? dim3(num_work * nkv, 1, 1) : dim3(num_work, nkv, 1);
+            attn_wave_kernel<DT, false, (DT <= 4 ? 4 : DT <= 6 ? 2 : 1), true, 8><<<bgrid, 512, 0, s>>>(TFF_ATTN_ARGS, fz);
         } else {
             return tff_fail("attention_decode_fused: blocks of eight waves take head sizes up to 128");
         }
+    } else if (fuse && fuse->key_runs) {
+        // runs of keys dealt by the host: num_work runs, a wave per run, kv head and column tile
+        attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 1), true><<<dim3(num_work * nkv, 1, tiles_per_entry), 64, 0, s>>>(TFF_ATTN_ARGS, fz);
     } else if (fuse) {
         if (splits > 1)
             attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 1), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
@@ -1206,7 +1339,7 @@ TFF_API int tff_attention_decode_fused(const void* qkv, int qkv_stride, void* ou
     if (R == 0) return 0;
     const int tiles = (nq / nkv + 15) / 16;
     AttnFuse fz{q_weight, k_weight, cos_sin, slot_mapping ? (bf16_t*)k_cache : nullptr,
-                slot_mapping ? (bf16_t*)v_cache : nullptr, slot_mapping, eps, pairing};
+                slot_mapping ? (bf16_t*)v_cache : nullptr, slot_mapping, eps, pairing, nullptr};
     hipStream_t s = (hipStream_t)stream;
 #define TFF_ATTN_CASE(DTV)                                                                          \
     case DTV * 16:                                                                                  \
@@ -1240,6 +1373,77 @@ TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml
         attn_split_reduce_kernel<<<dim3(n, nq), 256, 0, (hipStream_t)stream>>>(
             part_o, part_ml, (bf16_t*)out, splits, R_total, nq, d, rows);
     return tff_check_launch("attention_split_reduce");
+}
+
+// The same step with every entry's keys dealt into runs by the caller, who knows the entries'
+// lengths: key_runs [num_runs][4] = (entry, first key, end of keys, the entry's position), 16-byte
+// aligned, the runs of entry r being run_start[r] .. run_start[r + 1] - 1 (run_start [R + 1]), in
+// the order of the keys, without gap or overlap; a run's first key is the entry's first visible
+// key rounded down to a multiple of 32, plus a multiple of 32; an entry number < 0 marks a run that
+// is not in use.  A wave per run, kv head and column tile; runs
+// of similar length keep all waves busy alike however uneven the entries' lengths are, where
+// equal splits of every entry leave the longest entry's waves at work long after the others.
+// block_waves 8: a block of eight waves per run and kv head instead, which split the run among them
+// and merge in LDS (head sizes up to 128, one column tile).  merge 0: the caller knows that every
+// entry is one run (run_start[r] = r), so nothing is partial and the second kernel is left out.
+// Partial results (part_o [num_runs][nq][d], part_ml [num_runs][nq][2]) of the entries with more
+// than one run are merged by a second kernel.
+TFF_API int tff_attention_decode_runs(const void* qkv, int qkv_stride, void* out, float* part_o,
+                                      float* part_ml, void* k_cache, void* v_cache,
+                                      const int32_t* block_tables, int bt_stride,
+                                      const int32_t* cu_tokens, const int32_t* start_pos,
+                                      const int32_t* slot_mapping,
+                                      const float* q_weight, const float* k_weight, float eps,
+                                      const float* cos_sin, int max_pos, int pairing,
+                                      const int32_t* key_runs, const int32_t* run_start, int num_runs,
+                                      int block_waves, int merge, int R, int nq, int nkv, int d, int page_size,
+                                      int num_pages, int window, float scale, tff_stream_t stream) {
+    TFF_REQUIRE(qkv && out && k_cache && v_cache && block_tables && cu_tokens && start_pos,
+                "attention_decode_runs: null pointer");
+    TFF_REQUIRE(block_waves == 1 || (block_waves == 8 && d <= 128 && nq / nkv <= 16),
+                "attention_decode_runs: a run gets one wave, or a block of eight (head sizes up to 128, up to 16 "
+                "query heads a kv head), not %d with head size %d and %d query heads a kv head", block_waves, d, nq / nkv);
+    TFF_REQUIRE(key_runs && run_start && part_o && part_ml, "attention_decode_runs: the runs and the workspace are needed");
+    TFF_REQUIRE(((uintptr_t)key_runs % 16) == 0, "attention_decode_runs: key_runs must be 16-byte aligned");
+    TFF_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0,
+                "attention_decode_runs: %d query heads are not a multiple of %d key heads", nq, nkv);
+    TFF_REQUIRE(tff_attention_mfma_supported(d, page_size),
+                "attention_decode_runs: head size %d with pages of %d is not supported by the "
+                "matrix-core kernel", d, page_size);
+    TFF_REQUIRE(qkv_stride >= (nq + 2 * nkv) * d && qkv_stride % 8 == 0 && ((uintptr_t)qkv % 16) == 0,
+                "attention_decode_runs: rows of %d elements do not hold (nq + 2 nkv) d = %d, 16-byte aligned",
+                qkv_stride, (nq + 2 * nkv) * d);
+    TFF_REQUIRE((q_weight == nullptr) == (k_weight == nullptr),
+                "attention_decode_runs: q and k norm weights must both be given or both be absent");
+    TFF_REQUIRE(!cos_sin || ((pairing == 1 || (pairing == 0 && d % 64 == 0)) && max_pos > 0),
+                "attention_decode_runs: pairing %d with head size %d is not supported here", pairing, d);
+    const int tiles = (nq / nkv + 15) / 16;
+    TFF_REQUIRE(num_runs >= 0 && num_runs % 8 == 0 && (long)num_runs * nkv < (1L << 31) && tiles <= 65535 && d <= 256,
+                "attention_decode_runs: %d runs (a multiple of eight is needed), %d kv heads, %d column tiles (at most "
+                "65,535), head size %d (at most 256)", num_runs, nkv, tiles, d);
+    TFF_REQUIRE(bt_stride > 0 && num_pages > 0 && window >= 0 && R >= 0, "attention_decode_runs: bad geometry");
+    if (R == 0 || num_runs == 0) return 0;
+    AttnFuse fz{q_weight, k_weight, cos_sin, slot_mapping ? (bf16_t*)k_cache : nullptr,
+                slot_mapping ? (bf16_t*)v_cache : nullptr, slot_mapping, eps, pairing, key_runs};
+    hipStream_t s = (hipStream_t)stream;
+    int rc = -1;
+#define TFF_ATTN_CASE(DTV)                                                                          \
+    case DTV * 16:                                                                                  \
+        rc = launch_attn<DTV>((const bf16_t*)qkv, qkv_stride, (bf16_t*)out, part_o, part_ml,        \
+                              (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,         \
+                              bt_stride, cu_tokens, start_pos, nullptr, num_runs, nullptr, 0,       \
+                              tiles, 16, block_waves == 8 ? 0 : 2, nq, nkv, page_size, window,      \
+                              scale, R, s, &fz);                                                    \
+        break;
+    switch (d) {
+        TFF_ATTN_CASE(1) TFF_ATTN_CASE(2) TFF_ATTN_CASE(3) TFF_ATTN_CASE(4) TFF_ATTN_CASE(5)
+        TFF_ATTN_CASE(6) TFF_ATTN_CASE(7) TFF_ATTN_CASE(8) TFF_ATTN_CASE(12) TFF_ATTN_CASE(16)
+        default: return tff_fail("attention_decode_runs: head size %d", d);
+    }
+#undef TFF_ATTN_CASE
+    if (rc || !merge) return rc;
+    attn_run_merge_kernel<<<(R * nq + 3) / 4, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, run_start, R, nq, d);
+    return tff_check_launch("attention_run_merge");
 }
 
 // ------------------------------------------ decoding without any allocation ---

@@ -156,6 +156,31 @@ TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml
                                        int splits, int R_total, int nq, int d, const int32_t* rows,
                                        int num_rows, tff_stream_t stream);
 
+// tff_attention_decode_fused with every entry's keys dealt into runs by the caller, who knows
+// the entries' lengths, and the merge of the partial results, in one call.  key_runs
+// [num_runs][4] = (entry, first key, end of keys, the entry's position = start_pos[entry]), 16-byte
+// aligned: a wave per run, kv head and column tile; the runs of entry r are run_start[r] ..
+// run_start[r + 1] - 1 (run_start [R + 1]) and follow each other in the order of the keys, without
+// gap or overlap; a run's first key is the entry's first visible key rounded down to a multiple
+// of 32, plus a multiple of 32; an entry number < 0: the run is not in use.
+// Workspace: part_o [num_runs, nq, d], part_ml [num_runs, nq, 2] (float32).  Runs of similar
+// length keep the waves busy alike however uneven the entries' lengths are.  block_waves 1: a wave
+// per run and kv head; 8: a block of eight waves that split the run among them and merge in LDS
+// (head sizes up to 128, up to 16 query heads a kv head), for runs dealt with that in mind.
+// num_runs is a multiple of eight.  merge 0: the caller knows that every entry is one run, so no
+// result is partial and the merging kernel is not launched (a wrong 0 leaves the entries of
+// several runs without a result).
+TFF_API int tff_attention_decode_runs(const void* qkv, int qkv_stride, void* out, float* part_o,
+                                      float* part_ml, void* k_cache, void* v_cache,
+                                      const int32_t* block_tables, int bt_stride,
+                                      const int32_t* cu_tokens, const int32_t* start_pos,
+                                      const int32_t* slot_mapping,
+                                      const float* q_weight, const float* k_weight, float eps,
+                                      const float* cos_sin, int max_pos, int pairing,
+                                      const int32_t* key_runs, const int32_t* run_start, int num_runs,
+                                      int block_waves, int merge, int R, int nq, int nkv, int d, int page_size,
+                                      int num_pages, int window, float scale, tff_stream_t stream);
+
 // tff_attention_decode_fused followed by tff_attention_split_reduce, for callers that cannot
 // allocate device memory: code under HIP graph capture, tight serving loops, harnesses that
 // forbid hipMalloc.  It has no counterpart in the reference.  The partial results of split keys

@@ -13,6 +13,8 @@ from dataclasses import dataclass, field
 
 import torch
 
+from .key_runs import deal_key_runs, wants_blocks
+
 
 @dataclass
 class StepEntry:
@@ -25,24 +27,41 @@ class StepEntry:
 
 class KVView:
     """What a mixer sees of the cache in one layer call."""
-    __slots__ = ("k_cache", "v_cache", "block_tables", "slot_mapping", "page_size", "group")
+    __slots__ = ("k_cache", "v_cache", "block_tables", "slot_mapping", "page_size", "group", "key_runs",
+                 "run_start", "runs_window", "runs_for_blocks", "runs_merge")
 
-    def __init__(self, k_cache, v_cache, block_tables, slot_mapping, page_size, group):
+    def __init__(self, k_cache, v_cache, block_tables, slot_mapping, page_size, group, key_runs=None,
+                 run_start=None, runs_window=0, runs_for_blocks=False, runs_merge=True):
         self.k_cache = k_cache
         self.v_cache = v_cache
         self.block_tables = block_tables
         self.slot_mapping = slot_mapping     # per token; -1: not written (a call that only reads, padding)
         self.page_size = page_size
         self.group = group
+        # a step of one token per request: the requests' visible keys dealt into runs of similar
+        # length (engine.key_runs), for a window of runs_window, for single waves or for blocks
+        # of eight; else None
+        self.key_runs = key_runs
+        self.run_start = run_start
+        self.runs_window = runs_window
+        self.runs_for_blocks = runs_for_blocks
+        self.runs_merge = runs_merge         # False: every request is one run, no result is partial
 
 
 class GroupTables:
-    __slots__ = ("block_tables", "slot_mapping", "no_slot_mapping")
+    __slots__ = ("block_tables", "slot_mapping", "no_slot_mapping", "key_runs", "run_start", "runs_window",
+                 "runs_for_blocks", "runs_merge")
 
-    def __init__(self, block_tables, slot_mapping, no_slot_mapping):
+    def __init__(self, block_tables, slot_mapping, no_slot_mapping, key_runs=None, run_start=None, runs_window=0,
+                 runs_for_blocks=False, runs_merge=True):
         self.block_tables = block_tables        # int32 [R, max_blocks]
         self.slot_mapping = slot_mapping        # int32 [T]: page * page_size + offset of each new token
         self.no_slot_mapping = no_slot_mapping  # int32 [T] of -1: for calls that only read a cache
+        self.key_runs = key_runs                # int32 [runs, 4] or None (engine.key_runs)
+        self.run_start = run_start              # int32 [R + 1] or None
+        self.runs_window = runs_window
+        self.runs_for_blocks = runs_for_blocks
+        self.runs_merge = runs_merge            # False: the host knows that every request is one run
 
 
 class StepBatch:
@@ -136,6 +155,11 @@ def build_step_batch(entries, cache, device, pinned: PinnedTables | None = None)
         group_meta.append((len(sections), width))
         sections.append(flat)
         sections.append(sm)
+        # a step of one token per request: the requests' keys dealt into runs for the attention
+        if b.max_new_tokens == 1:
+            runs, run_start = deal_key_runs(start, g.spec.window, g.spec.num_kv_heads)
+            sections.append(runs.reshape(-1))
+            sections.append(run_start)
     offs, total = [], 0
     for s in sections:
         offs.append(total)
@@ -143,7 +167,7 @@ def build_step_batch(entries, cache, device, pinned: PinnedTables | None = None)
     host = pinned.take(max(total, 4)) if pinned is not None else torch.empty(max(total, 4), dtype=torch.int32)
     hv = host.numpy()
     for s, o in zip(sections, offs):
-        if s:
+        if len(s):
             hv[o:o + len(s)] = s
     dev = host.to(device, non_blocking=True)
     if pinned is not None:
@@ -157,9 +181,16 @@ def build_step_batch(entries, cache, device, pinned: PinnedTables | None = None)
     b.cu_tokens, b.start_pos, b.context_lens = sl(3, R + 1), sl(4, R), sl(5, R)
     b.state_slots, b.logit_rows = sl(6, R), sl(7, len(rows))
     no_slot = sl(8, T)
-    for (si, width) in group_meta:
+    for (si, width), g in zip(group_meta, cache.groups):
         bt = dev[offs[si]:offs[si] + R * width].view(R, width)
-        b.groups.append(GroupTables(bt, sl(si + 1, T), no_slot))
+        gt = GroupTables(bt, sl(si + 1, T), no_slot)
+        if b.max_new_tokens == 1:
+            gt.key_runs = sl(si + 2, len(sections[si + 2])).view(-1, 4)
+            gt.run_start = sl(si + 3, R + 1)
+            gt.runs_window = g.spec.window
+            gt.runs_for_blocks = wants_blocks(R, g.spec.num_kv_heads)
+            gt.runs_merge = int(sections[si + 3][R]) > R
+        b.groups.append(gt)
     b.host_cu_tokens, b.host_start_pos, b.host_state_slots = cu, start, slots
     b.reqs = [e.req for e in entries]
     return b

@@ -30,19 +30,22 @@ import numpy as np
 import torch
 
 from .batch import GroupTables, StepBatch
+from .key_runs import deal_key_runs, max_key_runs, wants_blocks
 
 
 def _pad4(n: int) -> int:
     return (n + 3) & ~3
 
 
-def table_layout(bucket: int, widths: list[int]) -> tuple[list[int], int]:
+def table_layout(bucket: int, widths: list[int], run_caps: list[int]) -> tuple[list[int], int]:
     """Offsets of the sections of a decode step's packed tables (the order of
-    build_step_batch) and their total length, for ``bucket`` rows."""
+    build_step_batch) and their total length, for ``bucket`` rows; per cache group a block table
+    of ``widths`` pages a row, the slots of the new tokens, ``run_caps`` runs of keys (four ints
+    each) and the rows' first runs."""
     B = bucket
     sizes = [B, B, B, B + 1, B, B, B, B, B]
-    for w in widths:
-        sizes += [B * w, B]
+    for w, cap in zip(widths, run_caps):
+        sizes += [B * w, B, 4 * cap, B + 1]
     offs, total = [], 0
     for n in sizes:
         offs.append(total)
@@ -68,7 +71,8 @@ class DecodeTables:
         self.B = B = int(bucket)
         ps = cache.page_size
         self.widths = [-(-max_model_len // ps) for _ in cache.groups]
-        self.offs, self.total = table_layout(B, self.widths)
+        self.run_caps = [max_key_runs(B, g.spec.num_kv_heads) for g in cache.groups]
+        self.offs, self.total = table_layout(B, self.widths, self.run_caps)
         if hv is None:
             hv = np.zeros(self.total, dtype=np.int32)
         if hv.dtype != np.int32 or hv.shape != (self.total,):
@@ -82,11 +86,13 @@ class DecodeTables:
         hv[o[8]:o[8] + B] = -1                      # no-slot mapping
         self._row_state = [None] * B                # (request, life, table lengths) last written per row
         self.host_start_pos, self.host_state_slots = [], []    # of the live rows of the last fill
+        self.needs_merge = False                    # whether the last fill cut some row's keys into several runs
         self._pad_rows(0)
+        self._deal_runs()
 
     def block_table_row(self, group: int, row: int) -> np.ndarray:
         w = self.widths[group]
-        base = self.offs[9 + 2 * group] + row * w
+        base = self.offs[9 + 4 * group] + row * w
         return self.hv[base:base + w]
 
     def _pad_rows(self, first: int) -> None:
@@ -99,10 +105,10 @@ class DecodeTables:
         hv[o[5] + first:o[5] + B] = 1               # context length
         hv[o[6] + first:o[6] + B] = self.cache.padding_slot   # a state row that no request holds
         for gi, w in enumerate(self.widths):
-            hv[o[10 + 2 * gi] + first:o[10 + 2 * gi] + B] = -1   # writes no key
+            hv[o[10 + 4 * gi] + first:o[10 + 4 * gi] + B] = -1   # writes no key
             for r in range(first, B):
                 if self._row_state[r] is not None:
-                    hv[o[9 + 2 * gi] + r * w:o[9 + 2 * gi] + (r + 1) * w] = 0
+                    hv[o[9 + 4 * gi] + r * w:o[9 + 4 * gi] + (r + 1) * w] = 0
         for r in range(first, B):
             self._row_state[r] = None
 
@@ -128,7 +134,7 @@ class DecodeTables:
             lens = []
             for gi, w in enumerate(self.widths):
                 table = cache.block_table(gi, e.req)
-                base = o[9 + 2 * gi] + r * w
+                base = o[9 + 4 * gi] + r * w
                 n = len(table)
                 old = prev[2][gi] if prev is not None else 0
                 grown = prev is not None and prev[0] == e.req and prev[1] == life and n >= old
@@ -143,9 +149,23 @@ class DecodeTables:
                     if old > n:
                         hv[base + n:base + old] = 0
                 lens.append(n)
-                hv[o[10 + 2 * gi] + r] = table[P // ps] * ps + P % ps
+                hv[o[10 + 4 * gi] + r] = table[P // ps] * ps + P % ps
             self._row_state[r] = (e.req, life, lens)
         self._pad_rows(R)
+        self._deal_runs()
+
+    def _deal_runs(self) -> None:
+        """The keys of all rows (a padding row has the one key of position 0) dealt into runs for
+        the attention, per cache group."""
+        o, hv, B = self.offs, self.hv, self.B
+        positions = hv[o[4]:o[4] + B]
+        self.needs_merge = False
+        for gi, g in enumerate(self.cache.groups):
+            _, start = deal_key_runs(positions, g.spec.window, g.spec.num_kv_heads,
+                                     runs_out=hv[o[11 + 4 * gi]:o[11 + 4 * gi] + 4 * self.run_caps[gi]],
+                                     start_out=hv[o[12 + 4 * gi]:o[12 + 4 * gi] + B + 1])
+            if int(start[B]) > B:
+                self.needs_merge = True     # some row's keys are several runs, in some group
 
 
 class DecodeGraph:
@@ -154,7 +174,7 @@ class DecodeGraph:
         self.B = B = int(bucket)
         cache = runner.cache
         widths = [-(-runner.max_model_len // cache.page_size) for _ in cache.groups]
-        _, total = table_layout(B, widths)
+        _, total = table_layout(B, widths, [max_key_runs(B, g.spec.num_kv_heads) for g in cache.groups])
         self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
         self.tables = DecodeTables(cache, B, runner.max_model_len, self.host.numpy())
         self.widths = self.tables.widths
@@ -173,19 +193,32 @@ class DecodeGraph:
         b.state_slots, b.logit_rows = sl(6, B), sl(7, B)
         no_slot = sl(8, B)
         for gi, w in enumerate(self.widths):
-            bt = self.dev[o[9 + 2 * gi]:o[9 + 2 * gi] + B * w].view(B, w)
-            b.groups.append(GroupTables(bt, sl(10 + 2 * gi, B), no_slot))
+            bt = self.dev[o[9 + 4 * gi]:o[9 + 4 * gi] + B * w].view(B, w)
+            b.groups.append(GroupTables(bt, sl(10 + 4 * gi, B), no_slot,
+                                        sl(11 + 4 * gi, 4 * self.tables.run_caps[gi]).view(-1, 4),
+                                        sl(12 + 4 * gi, B + 1), cache.groups[gi].spec.window,
+                                        wants_blocks(B, cache.groups[gi].spec.num_kv_heads)))
         b.host_cu_tokens = list(range(B + 1))
         b.host_start_pos = [0] * B
         b.host_state_slots = [cache.padding_slot] * B
         b.reqs = [None] * B
         self.batch = b
-        self.pieces = [_Piece(safe, items) for safe, items in runner.model.graph_pieces()]
+        # The step is captured in up to two variants: one in which the attention merges the partial
+        # results of rows whose keys are several runs, and one without that kernel, for steps in
+        # which every row is one run (the host knows when it deals the runs).  Each is captured
+        # when it is first wanted, on tables of padding rows only.
+        self._variants: dict[bool, list[_Piece]] = {}
+        self._padding = self.host.clone()           # the tables as they are with no live row
         self._copied = torch.cuda.Event()
 
     @property
     def runner(self):
         return self._runner()
+
+    @property
+    def pieces(self) -> list:
+        """The pieces of the variant captured first (all variants are cut alike)."""
+        return next(iter(self._variants.values())) if self._variants else []
 
     def fill(self, entries) -> None:
         self._copied.synchronize()      # the last copy out of the host buffer is done
@@ -196,8 +229,15 @@ class DecodeGraph:
         rn = self.runner
         return StepContext(rn.ops, rn.act_dtype, batch, rn.max_model_len, rn._calls, rn.cache)
 
-    def capture(self) -> None:
+    def capture(self, merge: bool = True) -> None:
+        """Captures the variant with (or without) the kernel that merges partial attention
+        results, unless it exists."""
+        if merge in self._variants:
+            return
         rn = self.runner
+        pieces = [_Piece(safe, items) for safe, items in rn.model.graph_pieces()]
+        for gt in self.batch.groups:
+            gt.runs_merge = merge
         # the decode attention sizes its key splits for the longest context the engine allows
         # (batch.max_context), so the launch is the same whatever the requests hold
         side = torch.cuda.Stream(device=rn.device)
@@ -209,10 +249,12 @@ class DecodeGraph:
         gc.disable()
         try:
             with torch.cuda.stream(side):
-                self.dev.copy_(self.host, non_blocking=True)
+                # every row is padding while the step runs to warm up and to be recorded: a part
+                # may keep state per request, which these runs must not touch
+                self.dev.copy_(self._padding.to(rn.device))
                 ctx = self._context(self.batch)
                 resid = pending = None
-                for piece in self.pieces:
+                for piece in pieces:
                     if not piece.safe:
                         # Not run here: every row is padding now, and such a part may keep state per
                         # request.  At every step it runs on the live rows and leaves its result in
@@ -240,6 +282,7 @@ class DecodeGraph:
                 gc.enable()
         torch.cuda.current_stream(rn.device).wait_stream(side)
         torch.cuda.synchronize(rn.device)
+        self._variants[merge] = pieces
 
     def _live_batch(self, R: int) -> StepBatch:
         """The first R rows of the graph's tables as a step of their own, with the host's
@@ -253,6 +296,7 @@ class DecodeGraph:
         b.cu_tokens, b.start_pos, b.context_lens = g.cu_tokens[:R + 1], g.start_pos[:R], g.context_lens[:R]
         b.state_slots, b.logit_rows = g.state_slots[:R], g.logit_rows[:R]
         for gt in g.groups:
+            # (no runs of keys: those of the graph's tables cover its padding rows too)
             b.groups.append(GroupTables(gt.block_tables[:R], gt.slot_mapping[:R], gt.no_slot_mapping[:R]))
         b.host_cu_tokens = list(range(R + 1))
         b.host_start_pos = list(t.host_start_pos)
@@ -265,6 +309,10 @@ class DecodeGraph:
         step that is launched before the host knows them.  Returns the logits of the graph's
         rows ([bucket, vocab], or [len(entries), vocab] if the step's last piece ran eagerly)."""
         self.fill(entries)
+        merge = self.tables.needs_merge
+        if merge not in self._variants:
+            self.capture(merge)
+        pieces = self._variants[merge]
         self.dev.copy_(self.host, non_blocking=True)
         self._copied.record()
         R = len(entries)
@@ -272,7 +320,7 @@ class DecodeGraph:
             self.dev[self.offs[0]:self.offs[0] + R].copy_(token_source)
         rn = self.runner
         logits = live = None
-        for piece in self.pieces:
+        for i, piece in enumerate(pieces):
             if piece.safe:
                 piece.graph.replay()
                 logits = piece.logits
@@ -281,7 +329,7 @@ class DecodeGraph:
                 live = self._context(self._live_batch(R))
             # the piece before left the residual stream and its pending term in fixed tensors;
             # this one adds to the stream's live rows in place
-            before = self.pieces[self.pieces.index(piece) - 1]
+            before = pieces[i - 1]
             _, p, lg = rn.model.run_items(live, piece.items, piece.resid[:R],
                                           None if before.pending is None else before.pending[:R])
             if lg is not None:

@@ -51,7 +51,8 @@ class StepContext(LayerContext):
         if group is not None:
             gt = self.batch.groups[group]
             c.kv = KVView(k, v, gt.block_tables, gt.slot_mapping if writes else gt.no_slot_mapping,
-                          self._cache.page_size, group)
+                          self._cache.page_size, group, gt.key_runs, gt.run_start, gt.runs_window,
+                          gt.runs_for_blocks, gt.runs_merge)
         c.state = state
         return c
 
@@ -193,14 +194,16 @@ class ModelRunner:
         return want if n >= self.CAPTURE_AFTER else have
 
     def capture_graphs(self) -> int:
-        """Captures the decode graph of every bucket that has none yet (some 50 ms each), so that
-        no step stops for a capture later; returns how many it captured."""
+        """Captures the decode graph of every bucket that has none yet (some 50 ms each, in both
+        of its variants), so that no step stops for a capture later; returns for how many
+        buckets it did."""
         n = 0
         with torch.cuda.device(self.device):
             for bucket in self._graph_buckets:
                 if bucket not in self._graphs:
                     g = self._graphs[bucket] = DecodeGraph(self, bucket)
-                    g.capture()
+                    g.capture(True)
+                    g.capture(False)
                     n += 1
         return n
 
@@ -213,8 +216,7 @@ class ModelRunner:
             g = self._graphs.get(bucket)
             if g is None:
                 g = self._graphs[bucket] = DecodeGraph(self, bucket)
-                g.capture()
-            logits = g.run(entries, token_source)
+            logits = g.run(entries, token_source)       # (captures the variant the step needs, if it is new)
             rows = [r for r, e in enumerate(entries) if e.want]
             if len(rows) == R:
                 out = logits[:R]

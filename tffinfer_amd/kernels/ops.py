@@ -697,13 +697,22 @@ def decode_fused_supported(qkv: torch.Tensor, d: int, page_size: int, cos_sin, p
 
 def attention_decode_fused(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, eps: float,
                            cos_sin, pairing: int, kv, batch, window: int = 0, scale: float | None = None,
-                           slot_mapping: torch.Tensor | None = None, splits: int | None = None) -> torch.Tensor:
+                           slot_mapping: torch.Tensor | None = None, splits: int | None = None,
+                           key_runs: torch.Tensor | None = None, run_start: torch.Tensor | None = None,
+                           runs_for_blocks: bool = False, runs_merge: bool = True) -> torch.Tensor:
     """A decode-only step from the fused projection's output ``qkv`` [R, (nq +
     2 nkv) d]: q/k norm, rotation, the new keys and values into their pages and
     the attention over the pages, in one kernel (plus the merge of split keys).
     ``slot_mapping`` (int32 [R]) says which tokens' keys and values are written
     (entries >= 0; the place is the one the block table gives for the token's
-    position); None: no token's, the pages hold them already."""
+    position); None: no token's, the pages hold them already.  ``key_runs``
+    (int32 [runs, 4]: row, first key, end of keys, the row's position) and ``run_start`` (int32
+    [R + 1]): the rows' keys dealt into runs by the host, a wave per run and
+    kv head (``engine.key_runs``), or a block of eight waves if they were
+    dealt for that (``runs_for_blocks``) and the head size allows it;
+    ``runs_merge`` False: the caller knows that every row is one run, and the
+    kernel that merges partial results is left out.  Without runs every
+    row's keys are split alike (``splits``)."""
     _req(qkv, "attention_decode_fused qkv", torch.bfloat16, 2)
     R = batch.num_reqs
     if qkv.shape[0] != R or batch.num_tokens != R or batch.max_new_tokens != 1:
@@ -740,6 +749,24 @@ def attention_decode_fused(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weigh
     tiles = -(-G // 16)
     if scale is None:
         scale = 1.0 / math.sqrt(d)
+    if key_runs is not None and splits is None:
+        _req(key_runs, "key_runs", torch.int32, 2)
+        _req(run_start, "run_start", torch.int32, 1)
+        if key_runs.shape[1] != 4 or run_start.numel() != R + 1:
+            raise _lib.KernelError(f"attention_decode_fused: runs of shape {tuple(key_runs.shape)} and "
+                                   f"{run_start.numel()} run starts for {R} rows")
+        P = key_runs.shape[0]
+        out = torch.empty(R, nq * d, dtype=qkv.dtype, device=qkv.device)
+        part_o = torch.empty(P, nq, d, dtype=torch.float32, device=qkv.device)
+        part_ml = torch.empty(P, nq, 2, dtype=torch.float32, device=qkv.device)
+        _lib.check(_lib.load().tff_attention_decode_runs(
+            qkv.data_ptr(), qkv.stride(0), out.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), k_cache.data_ptr(),
+            v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(), batch.start_pos.data_ptr(),
+            _ptr(slot_mapping), _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin), max_pos, int(pairing),
+            key_runs.data_ptr(), run_start.data_ptr(), P, 8 if (runs_for_blocks and d <= 128 and tiles == 1) else 1,
+            1 if runs_merge else 0, R, nq, nkv, d, k_cache.shape[2], k_cache.shape[0],
+            int(window), float(scale), _stream()))
+        return out
     if splits is None:
         # entries x kv heads enough for a block each to saturate HBM between them: the keys of
         # an entry are split among the eight waves of its block and merged in LDS (splits 0)
@@ -771,8 +798,14 @@ def qkv_attention(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weig
     that another call fills, or the row is padding), attention over the cache.  Decode-only steps in bfloat16 are one kernel."""
     if decode_fused_supported(qkv, d, kv.k_cache.shape[2], cos_sin, pairing, batch):
         # (a call that only reads its cache, or a padding row, has negative slots)
+        runs = getattr(kv, "key_runs", None)
+        if runs is not None and kv.runs_window != int(window):
+            runs = None       # dealt for another window than this call's
         return attention_decode_fused(qkv, nq, nkv, d, q_weight, k_weight, eps, cos_sin, pairing, kv, batch,
-                                      window, scale, slot_mapping=kv.slot_mapping)
+                                      window, scale, slot_mapping=kv.slot_mapping, key_runs=runs,
+                                      run_start=kv.run_start if runs is not None else None,
+                                      runs_for_blocks=runs is not None and kv.runs_for_blocks,
+                                      runs_merge=runs is None or kv.runs_merge)
     qk_norm_rope_kv(qkv, nq, nkv, d, q_weight, k_weight, eps, cos_sin, pairing, batch.positions,
                     kv.slot_mapping, kv.k_cache, kv.v_cache)
     return paged_attention(qkv, nq, nkv, d, kv, batch, window, scale)
