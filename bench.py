@@ -136,8 +136,9 @@ def large_points(args, gen) -> dict:
 def long_points(args, model, cfg, gen) -> tuple[dict, dict]:
     """Further sizes at the benchmark shape, on an engine of their own whose length limit holds
     them (a decode graph's launches are sized for the limit, so the headline keeps its own):
-    decode steps of 8 requests at 32,768 tokens of context and of 128 requests at 8,192, and
-    prompts of 8,192 and 32,768 tokens in one step.  Returns (tokens a second, details) by
+    decode steps of 8 requests at 32,768 tokens of context, of 128 requests at 8,192 and of 64
+    requests of which one has 32,768 tokens and the others 1,024 (as many keys as 64 requests of
+    1,520), and prompts of 8,192 and 32,768 tokens in one step.  Returns (tokens a second, details) by
     point; a point that fails is left null."""
     import gc
     import torch
@@ -147,17 +148,20 @@ def long_points(args, model, cfg, gen) -> tuple[dict, dict]:
     vocab = cfg["vocab_size"]
     L = cfg["num_hidden_layers"]
     for key, batch, context, steps, warmup in (("decode_b8_ctx32768", 8, 32768, 16, 4),
-                                               ("decode_b128_ctx8192", 128, 8192, 12, 4)):
+                                               ("decode_b128_ctx8192", 128, 8192, 12, 4),
+                                               ("decode_b64_ctx1024_one_of_32768", 64, [32768] + [1024] * 63, 16, 4)):
         try:
-            total = steps + warmup + M.decode_slack(batch, context) + 16
+            longest = max(context) if isinstance(context, list) else context
+            mean = sum(context) / batch if isinstance(context, list) else context
+            total = steps + warmup + M.decode_slack(batch, longest) + 16
             opt = EngineOptions(dtype="bfloat16", page_size=args.page_size,
-                                kv_tokens=batch * (context + total + args.page_size), max_num_seqs=batch,
-                                max_num_batched_tokens=4096, prefill_chunk=2048, max_model_len=context + total + 16,
+                                kv_tokens=int(batch * (mean + total + args.page_size)), max_num_seqs=batch,
+                                max_num_batched_tokens=4096, prefill_chunk=2048, max_model_len=longest + total + 16,
                                 use_graphs=not args.no_graphs)
             engine = LLMEngine(model, opt)
             r = M.measure_decode(engine, gen, batch, context, steps, warmup, vocab)
             step = r["wall_s"] / steps
-            nbytes = M.decode_bytes(model, batch, context + warmup + steps / 2.0)
+            nbytes = M.decode_bytes(model, batch, mean + warmup + steps / 2.0)
             points[key] = round(batch / step, 1)
             detail[key] = {"ms_per_step": round(1e3 * step, 4), "ms_per_step_median": round(1e3 * r["step_median_s"], 4),
                            "frac": round(nbytes / step / 1e9 / M.HBM_PEAK_GBS, 4)}

@@ -1,12 +1,13 @@
 """Decode steps of twenty and more requests through the engine, against the plain
 implementation: the schedules that large batches take and small ones never reach.
 
-With eight kv heads, twenty requests are 160 (request, kv head) pairs, from which on a decode
-step gives every pair a block of waves of its own instead of splitting the keys over blocks and
-merging in a second kernel; products of 17 to 64 rows run on tiles whose blocks split K, with
-their partial sums added up by the norm that follows or by a kernel of their own; and the batch
-shrinks through the graph buckets 28, 24, 16, 12, 8, ... with a larger graph standing in for a
-smaller one on the way.  All of that runs inside captured HIP graphs with padding rows and with
+With eight kv heads, twenty to thirty-two requests are 160 to 256 (request, kv head) pairs,
+between which a decode step gives every run of keys a block of eight waves instead of a single
+wave; products of 17 to 64 rows run on tiles whose blocks split K, with their partial sums added
+up by the norm that follows or by a kernel of their own; and the batch shrinks through the graph
+buckets 28, 24, 16, 12, 8, ... with a larger graph standing in for a smaller one on the way.  One
+request many times longer than the others is cut into many runs of keys, whose partial results a
+second kernel merges, while the short ones are a run each.  All of that runs inside captured HIP graphs with padding rows and with
 steps launched ahead.  Every kept row of logits is compared with the plain logits of the
 request's own sequence and every token with the plain sampler's choice from that row
 (``check_choices``).
@@ -24,11 +25,14 @@ pytestmark = pytest.mark.gpu
 def _watch(monkeypatch):
     """Records what the decode attention and the products were asked for."""
     from tffinfer_amd.kernels import ops
-    seen = {"pairs": set(), "split_rows": set(), "stacks": set()}
+    seen = {"pairs": set(), "split_rows": set(), "stacks": set(), "blocks": set(), "merge": set()}
     inner_attn, inner_linear = ops.attention_decode_fused, ops.linear
 
     def attn(qkv, nq, nkv, *a, **kw):
         seen["pairs"].add(qkv.shape[0] * nkv)
+        assert kw.get("key_runs") is not None, "a decode step without runs of keys"
+        seen["blocks"].add(bool(kw["runs_for_blocks"]))
+        seen["merge"].add(bool(kw["runs_merge"]))
         return inner_attn(qkv, nq, nkv, *a, **kw)
 
     def linear(x, weight, *a, **kw):
@@ -90,8 +94,7 @@ def test_twenty_eight_requests_shrinking_through_the_graph_buckets(model_dirs, n
     assert {28, 24, 16, 12, 8}.issubset(graphs), graphs
     assert standins, "no graph ever stood in for a smaller one"
     if dtype == "bfloat16":
-        assert any(p >= ops.BLOCK_DECODE_MIN_PAIRS for p in seen["pairs"]), "no step gave a block to every pair"
-        assert any(p < ops.BLOCK_DECODE_MIN_PAIRS for p in seen["pairs"]), "no step split the keys over blocks"
+        assert seen["blocks"] == {True, False}, "blocks of eight waves and single waves should both have run"
         assert any(17 <= rows <= 64 and parts > 1 for rows, parts in seen["stacks"]), \
             "no product of 17 to 64 rows kept partial sums for the norm"
     for i in range(n):
@@ -166,3 +169,37 @@ def test_random_workloads_of_many_requests_on_small_pools(model_dirs, name, dtyp
         check_choices(d, res, dtype, r["sampling"])
     assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
     assert eng.runner.cache.slots.num_free == slots
+
+
+@pytest.mark.parametrize("n,graphs", [(12, True), (24, True), (24, False), (40, True)])
+def test_a_long_request_among_short_ones(tmp_path, n, graphs, monkeypatch):
+    """One request of two thousand tokens beside requests of a few dozen: the long one's keys are
+    cut into runs of the short ones' measure (single waves at twelve and forty requests, blocks of
+    eight waves at twenty-four) and merged, the short ones are a run each; once the long request
+    has ended no step merges anything, and a captured step then runs in its variant without the
+    merging kernel.  Every row of logits against the plain implementation."""
+    from helpers import TINY_E, make_model_dir
+    from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
+    cfg = dict(TINY_E, max_position_embeddings=4096)
+    d = make_model_dir(str(tmp_path / "E"), cfg, 61)
+    V = cfg["vocab_size"]
+    seen = _watch(monkeypatch)
+    plens = [2000] + [5 + (13 * i) % 60 for i in range(1, n)]
+    news = [6] + [14] * (n - 1)
+    opt = EngineOptions(dtype="bfloat16", page_size=16, kv_tokens=2100 + n * 96, max_num_seqs=n,
+                        max_num_batched_tokens=4096, prefill_chunk=2048, max_model_len=2100,
+                        use_graphs=graphs, run_ahead=graphs)
+    eng = LLMEngine.from_model_dir(d, opt)
+    eng.keep_logits = True
+    reqs = [dict(prompt_ids=random_tokens(plens[i], V, 700 + i), sampling=SamplingConfig(), max_new_tokens=news[i],
+                 ignore_eos=True, request_id=i) for i in range(n)]
+    drive(eng, {0: reqs})
+    assert seen["merge"] == {True, False}
+    assert seen["blocks"] == ({True} if n == 24 else {False})
+    if graphs:
+        g = eng.runner._graphs[n]
+        assert set(g._variants) == {True, False}, "the step of this many rows should exist with and without the merge"
+    for i in range(n):
+        r = eng.pop_result(i)
+        assert r.finish_reason == "length" and len(r.output) == news[i]
+        check_choices(d, r, "bfloat16", None)

@@ -101,20 +101,22 @@ def measure_prefill(engine, gen, T: int, vocab: int, reps: int = 5, warm: int = 
     return {"wall_s": statistics.median(wall), "device_s": statistics.median(dev), "reps": reps}
 
 
-def measure_decode(engine, gen, batch: int, context: int, steps: int, warmup: int, vocab: int,
+def measure_decode(engine, gen, batch: int, context, steps: int, warmup: int, vocab: int,
                    sampling=None) -> dict:
-    """Fills ``batch`` requests with ``context`` tokens each (untimed prefill), then times
+    """Fills ``batch`` requests with ``context`` tokens each (a list: request i with context[i];
+    untimed prefill), then times
     ``steps`` decode steps of the whole engine (plan, tables, model, sampling, tokens back on
     the host).  ``wall_s``: all the steps by the wall clock between two synchronisations;
     ``step_median_s``: the median of the device-event intervals between consecutive steps.
     ``sampling``: a SamplingConfig for every request (its seed is offset by the request's number);
     greedy without one."""
     import dataclasses
+    contexts = list(context) if isinstance(context, (list, tuple)) else [context] * batch
     for i in range(batch):
         # requests that finish their prompt early decode while the others still prefill
-        engine.add_request(random_prompt(gen, context, vocab),
+        engine.add_request(random_prompt(gen, contexts[i], vocab),
                            sampling=dataclasses.replace(sampling, seed=sampling.seed + i) if sampling else None,
-                           max_new_tokens=warmup + steps + decode_slack(batch, context) + 8, ignore_eos=True)
+                           max_new_tokens=warmup + steps + decode_slack(batch, max(contexts)) + 8, ignore_eos=True)
     # untimed: prompts, up to the first decode-only step
     while any(r.num_pending > 1 for r in engine.scheduler.running) or engine.scheduler.waiting:
         engine.step()
