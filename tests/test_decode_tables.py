@@ -43,8 +43,9 @@ def check_rows(tables: DecodeTables, cache, entries):
     # the keys of every row, padding included, dealt into runs: each visible key in exactly one
     for gi, g in enumerate(cache.groups):
         cap = tables.run_caps[gi]
-        check_runs(hv[o[11 + 4 * gi]:o[11 + 4 * gi] + 4 * cap].reshape(-1, 4), hv[o[12 + 4 * gi]:o[12 + 4 * gi] + tables.B + 1],
-                   hv[o[4]:o[4] + tables.B], g.spec.window)
+        start = hv[o[12 + 4 * gi]:o[12 + 4 * gi] + tables.B + 1]
+        check_runs(hv[o[11 + 4 * gi]:o[11 + 4 * gi] + 4 * cap].reshape(-1, 4), start, hv[o[4]:o[4] + tables.B], g.spec.window)
+        assert tables.variant[0] or start[tables.B] == tables.B, "rows of several runs, and a variant that merges nothing"
 
 
 class TableRunner:

@@ -1012,8 +1012,9 @@ def test_attention_decode_fused(nq, nkv, d, ps, window, splits, pairing, with_no
     how = dict(splits=splits)
     if isinstance(splits, str):
         from tffinfer_amd.engine.key_runs import deal_key_runs
-        runs, run_start = deal_key_runs([P for P, _ in entries], window, nkv, target=int(splits.split()[1]), min_steps=1)
-        assert run_start[-1] > R, "no entry has several runs"
+        runs, run_start, _, merge = deal_key_runs([P for P, _ in entries], window, nkv, target=int(splits.split()[1]), min_steps=1,
+                                                  blocks=False)
+        assert merge and run_start[-1] > R, "no entry has several runs"
         how = dict(key_runs=torch.from_numpy(runs.copy()).to(DEV), run_start=torch.from_numpy(run_start.copy()).to(DEV))
         splits = None
     out = ops.attention_decode_fused(qkv.to(DEV), nq, nkv, d, w[0], w[1], eps, table, pr, kv, batch, window, scale,
@@ -1129,7 +1130,8 @@ def test_attention_decode_fused_keys_dealt_into_runs(nq, nkv, d, ps, window, wav
         v = torch.cat([vs[r][:P], v_new[r:r + 1]])
         refs.append(_attn_ref(q[r:r + 1], k, v, positions[r:r + 1], window, scale)[0])
     ref = torch.stack(refs)
-    runs, run_start = deal_key_runs([P for P, _ in entries], window, nkv, target=waves, blocks=blocks)
+    runs, run_start, _, merge = deal_key_runs([P for P, _ in entries], window, nkv, target=waves, blocks=blocks)
+    assert merge
     counts = run_start[1:] - run_start[:-1]
     assert counts[0] > 4 and (counts == 1).sum() >= 6 and (runs[:, 0] == -1).any()
     out = ops.attention_decode_fused(qkv.to(DEV), nq, nkv, d, None, None, 1e-6, None, 0, kv, batch, window, scale,

@@ -7,7 +7,7 @@ import random
 import numpy as np
 import pytest
 
-from tffinfer_amd.engine.key_runs import (BLOCK_PAIRS, BLOCK_SLOTS, BUSY_WAVES, KEY_STEP, LONG_STEPS, MIN_STEPS, RESIDENT_WAVES,
+from tffinfer_amd.engine.key_runs import (BLOCK_PAIRS, BUSY_WAVES, KEY_STEP, LONG_STEPS, MIN_STEPS, RESIDENT_WAVES,
                                           TARGET_WAVES, deal_key_runs, max_key_runs, wants_blocks)
 
 
@@ -49,61 +49,70 @@ def test_every_key_in_exactly_one_run(window, nkv):
             pos = [30000] + [rng.randrange(0, 600) for _ in range(R - 1)]
         else:
             pos = [2047] * R
-        runs, start = deal_key_runs(pos, window, nkv)
-        assert runs.shape[0] == max_key_runs(R, nkv)
-        check_runs(runs, start, pos, window)
+        live = rng.choice([None, R, max(1, R - 3)])
+        dealt = deal_key_runs(pos, window, nkv, live=live)
+        assert dealt.runs.shape[0] == max_key_runs(R, nkv)
+        check_runs(dealt.runs, dealt.run_start, pos, window)
+        assert dealt.merge == (dealt.run_start[-1] > R)
+        assert not (dealt.blocks and dealt.merge), "blocks of eight waves are for rows of one run each"
+        assert dealt.run_start[-1] * nkv <= max(RESIDENT_WAVES, R * nkv), "more waves than the GPU holds at once"
 
 
 def test_runs_are_of_similar_length():
     # one long request beside many short ones: the long one's runs are about as long as the
     # waves' fair share of all keys, not a fixed fraction of its own length
     pos = [32767] + [1023] * 63
-    runs, start = deal_key_runs(pos, 0, 8)
+    runs, start, blocks, merge = deal_key_runs(pos, 0, 8)
     steps = -(-(runs[:start[-1], 2] - runs[:start[-1], 1]) // KEY_STEP)
     fair = -(-sum((p // KEY_STEP + 1) for p in pos) * 8 // TARGET_WAVES)
     assert steps.max() <= 1.5 * fair, (steps.max(), fair)
     assert start[1] - start[0] >= 16, "the long request is many runs"
     assert np.all(np.diff(start)[1:] == 1), "a short request is one run"
-    assert start[-1] * 8 <= RESIDENT_WAVES
+    assert start[-1] * 8 <= RESIDENT_WAVES and merge and not blocks
     # few requests: runs no shorter than MIN_STEPS steps, and no shorter than LONG_STEPS while
     # BUSY_WAVES waves have work
-    runs, start = deal_key_runs([2047], 0, 8)
-    assert start[1] == 2048 // KEY_STEP // MIN_STEPS
+    runs, start, _, _ = deal_key_runs([2047], 0, 8)
+    assert start[1] == -(-64 // -(-64 // (64 // MIN_STEPS)))
     for P in (2047, 2099, 2111):
-        runs, start = deal_key_runs([P] * 8, 0, 8)
+        runs, start, _, _ = deal_key_runs([P] * 8, 0, 8)
         n = start[1] - start[0]
         assert n == (P // KEY_STEP + 1) // LONG_STEPS and n * 8 * 8 >= BUSY_WAVES
     # a short request is one run whatever its neighbours
-    runs, start = deal_key_runs([5, 100000], 0, 8)
+    runs, start, _, _ = deal_key_runs([5, 100000], 0, 8)
     assert start[1] == 1
     # requests of one length: the launch stays within the waves that the GPU holds at once
     for R, per_row in ((16, 6), (40, 3), (48, 2), (64, 1), (72, 1), (128, 1), (200, 1)):
         assert not wants_blocks(R, 8)
-        runs, start = deal_key_runs([2100] * R, 0, 8)
+        runs, start, blocks, merge = deal_key_runs([2100] * R, 0, 8)
         assert start[-1] == per_row * R, (R, start[-1])
-        assert per_row == 1 or start[-1] * 8 <= RESIDENT_WAVES
+        assert (per_row == 1 or start[-1] * 8 <= RESIDENT_WAVES) and merge == (per_row > 1) and not blocks
 
 
-def test_runs_for_blocks_are_cut_to_the_measure_of_the_typical_request():
+def test_blocks_of_eight_waves_are_for_requests_of_about_one_length():
+    rng = random.Random(5)
     for R in (20, 24, 32):
         assert wants_blocks(R, 8) and BLOCK_PAIRS[0] <= R * 8 <= BLOCK_PAIRS[1]
-        # requests of one length: one run each, the block's waves split it among them
-        runs, start = deal_key_runs([2100] * R, 0, 8)
-        assert start[-1] == R
-        check_runs(runs, start, [2100] * R, 0)
-        # ... and of about one length
-        near = [2000 + 37 * i for i in range(R)]
-        runs, start = deal_key_runs(near, 0, 8)
-        assert start[-1] == R
-        # long requests among short ones are cut to the measure of the average request
-        pos = [16383] * 3 + [1023] * (R - 3)
-        runs, start = deal_key_runs(pos, 0, 8)
-        check_runs(runs, start, pos, 0)
-        lens = -(-(runs[:start[-1], 2] - runs[:start[-1], 1]) // KEY_STEP)
-        assert R < start[-1] <= BLOCK_SLOTS // 8 and lens.max() <= 1.5 * 32
-        assert np.all(np.diff(start)[3:] == 1) and np.all(np.diff(start)[:3] >= 4)
-        assert runs.shape[0] == max_key_runs(R, 8) == BLOCK_SLOTS // 8
+        # requests of one length, or of about one: a run each, the block's waves split it among them
+        for pos in ([2100] * R, [2000 + 11 * i for i in range(R)]):
+            runs, start, blocks, merge = deal_key_runs(pos, 0, 8)
+            assert blocks and not merge and start[-1] == R
+            check_runs(runs, start, pos, 0)
+        # padding rows of a captured step do not count
+        runs, start, blocks, merge = deal_key_runs([2100] * R + [0] * 4, 0, 8, live=R)
+        assert blocks and not merge and start[-1] == R + 4
+        # uneven lengths go to single waves, the long requests cut to the others' measure
+        for pos in ([16383] * 3 + [1023] * (R - 3), [rng.randrange(300, 4300) for _ in range(R)]):
+            runs, start, blocks, merge = deal_key_runs(pos, 0, 8)
+            assert not blocks and merge and R < start[-1] <= RESIDENT_WAVES // 8
+            check_runs(runs, start, pos, 0)
+            lens = -(-(runs[:start[-1], 2] - runs[:start[-1], 1]) // KEY_STEP)
+            steps = sorted(p // KEY_STEP + 1 for p in pos)
+            fair = -(-sum(steps) * 8 // TARGET_WAVES)
+            assert lens.max() <= 1.5 * max(fair, steps[R // 2]) + 1, "a run much longer than the fair share and the median request"
     assert not wants_blocks(19, 8) and not wants_blocks(33, 8) and wants_blocks(128, 2) and not wants_blocks(1, 8)
+    # too few or too many requests: single waves whatever the lengths
+    for R in (8, 19, 33, 64):
+        assert not deal_key_runs([2100] * R, 0, 8).blocks
 
 
 def test_tables_too_small_are_refused():
@@ -114,5 +123,5 @@ def test_tables_too_small_are_refused():
 
 
 def test_no_rows():
-    runs, start = deal_key_runs([], 0, 8)
-    assert start.tolist() == [0] and np.all(runs[:, 0] == -1)
+    runs, start, blocks, merge = deal_key_runs([], 0, 8)
+    assert start.tolist() == [0] and np.all(runs[:, 0] == -1) and not blocks and not merge

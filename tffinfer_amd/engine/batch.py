@@ -13,7 +13,7 @@ from dataclasses import dataclass, field
 
 import torch
 
-from .key_runs import deal_key_runs, wants_blocks
+from .key_runs import deal_key_runs
 
 
 @dataclass
@@ -157,9 +157,10 @@ def build_step_batch(entries, cache, device, pinned: PinnedTables | None = None)
         sections.append(sm)
         # a step of one token per request: the requests' keys dealt into runs for the attention
         if b.max_new_tokens == 1:
-            runs, run_start = deal_key_runs(start, g.spec.window, g.spec.num_kv_heads)
-            sections.append(runs.reshape(-1))
-            sections.append(run_start)
+            dealt = deal_key_runs(start, g.spec.window, g.spec.num_kv_heads)
+            sections.append(dealt.runs.reshape(-1))
+            sections.append(dealt.run_start)
+            group_meta[-1] += (dealt.blocks, dealt.merge)
     offs, total = [], 0
     for s in sections:
         offs.append(total)
@@ -181,15 +182,14 @@ def build_step_batch(entries, cache, device, pinned: PinnedTables | None = None)
     b.cu_tokens, b.start_pos, b.context_lens = sl(3, R + 1), sl(4, R), sl(5, R)
     b.state_slots, b.logit_rows = sl(6, R), sl(7, len(rows))
     no_slot = sl(8, T)
-    for (si, width), g in zip(group_meta, cache.groups):
+    for (si, width, *dealt), g in zip(group_meta, cache.groups):
         bt = dev[offs[si]:offs[si] + R * width].view(R, width)
         gt = GroupTables(bt, sl(si + 1, T), no_slot)
-        if b.max_new_tokens == 1:
+        if dealt:
             gt.key_runs = sl(si + 2, len(sections[si + 2])).view(-1, 4)
             gt.run_start = sl(si + 3, R + 1)
             gt.runs_window = g.spec.window
-            gt.runs_for_blocks = wants_blocks(R, g.spec.num_kv_heads)
-            gt.runs_merge = int(sections[si + 3][R]) > R
+            gt.runs_for_blocks, gt.runs_merge = dealt
         b.groups.append(gt)
     b.host_cu_tokens, b.host_start_pos, b.host_state_slots = cu, start, slots
     b.reqs = [e.req for e in entries]

@@ -30,7 +30,7 @@ import numpy as np
 import torch
 
 from .batch import GroupTables, StepBatch
-from .key_runs import deal_key_runs, max_key_runs, wants_blocks
+from .key_runs import deal_key_runs, max_key_runs
 
 
 def _pad4(n: int) -> int:
@@ -86,9 +86,9 @@ class DecodeTables:
         hv[o[8]:o[8] + B] = -1                      # no-slot mapping
         self._row_state = [None] * B                # (request, life, table lengths) last written per row
         self.host_start_pos, self.host_state_slots = [], []    # of the live rows of the last fill
-        self.needs_merge = False                    # whether the last fill cut some row's keys into several runs
+        self.variant = (False, ())                  # (some row has several runs, per group: dealt for blocks) at the last fill
         self._pad_rows(0)
-        self._deal_runs()
+        self._deal_runs(0)
 
     def block_table_row(self, group: int, row: int) -> np.ndarray:
         w = self.widths[group]
@@ -152,20 +152,22 @@ class DecodeTables:
                 hv[o[10 + 4 * gi] + r] = table[P // ps] * ps + P % ps
             self._row_state[r] = (e.req, life, lens)
         self._pad_rows(R)
-        self._deal_runs()
+        self._deal_runs(R)
 
-    def _deal_runs(self) -> None:
+    def _deal_runs(self, live: int) -> None:
         """The keys of all rows (a padding row has the one key of position 0) dealt into runs for
-        the attention, per cache group."""
+        the attention, per cache group; the first ``live`` rows are requests."""
         o, hv, B = self.offs, self.hv, self.B
         positions = hv[o[4]:o[4] + B]
-        self.needs_merge = False
+        merge, blocks = False, []
         for gi, g in enumerate(self.cache.groups):
-            _, start = deal_key_runs(positions, g.spec.window, g.spec.num_kv_heads,
-                                     runs_out=hv[o[11 + 4 * gi]:o[11 + 4 * gi] + 4 * self.run_caps[gi]],
-                                     start_out=hv[o[12 + 4 * gi]:o[12 + 4 * gi] + B + 1])
-            if int(start[B]) > B:
-                self.needs_merge = True     # some row's keys are several runs, in some group
+            dealt = deal_key_runs(positions, g.spec.window, g.spec.num_kv_heads,
+                                  runs_out=hv[o[11 + 4 * gi]:o[11 + 4 * gi] + 4 * self.run_caps[gi]],
+                                  start_out=hv[o[12 + 4 * gi]:o[12 + 4 * gi] + B + 1], live=live)
+            merge = merge or dealt.merge        # some row's keys are several runs, in some group
+            blocks.append(dealt.blocks)
+        #: what the last fill's dealing found: the variant of the captured step that fits these tables
+        self.variant = (merge, tuple(blocks))
 
 
 class DecodeGraph:
@@ -196,18 +198,17 @@ class DecodeGraph:
             bt = self.dev[o[9 + 4 * gi]:o[9 + 4 * gi] + B * w].view(B, w)
             b.groups.append(GroupTables(bt, sl(10 + 4 * gi, B), no_slot,
                                         sl(11 + 4 * gi, 4 * self.tables.run_caps[gi]).view(-1, 4),
-                                        sl(12 + 4 * gi, B + 1), cache.groups[gi].spec.window,
-                                        wants_blocks(B, cache.groups[gi].spec.num_kv_heads)))
+                                        sl(12 + 4 * gi, B + 1), cache.groups[gi].spec.window))
         b.host_cu_tokens = list(range(B + 1))
         b.host_start_pos = [0] * B
         b.host_state_slots = [cache.padding_slot] * B
         b.reqs = [None] * B
         self.batch = b
-        # The step is captured in up to two variants: one in which the attention merges the partial
-        # results of rows whose keys are several runs, and one without that kernel, for steps in
-        # which every row is one run (the host knows when it deals the runs).  Each is captured
-        # when it is first wanted, on tables of padding rows only.
-        self._variants: dict[bool, list[_Piece]] = {}
+        # The step is captured in variants, by what the host finds when it deals the rows' keys into
+        # runs: whether some row has several runs (else the kernel that merges partial attention
+        # results is left out), and, per cache group, whether a run gets a block of eight waves or a
+        # single one.  Each variant is captured when it is first wanted, on tables of padding rows.
+        self._variants: dict[tuple, list[_Piece]] = {}
         self._padding = self.host.clone()           # the tables as they are with no live row
         self._copied = torch.cuda.Event()
 
@@ -224,20 +225,36 @@ class DecodeGraph:
         self._copied.synchronize()      # the last copy out of the host buffer is done
         self.tables.fill(entries)
 
+    def possible_variants(self) -> list:
+        """The variants that steps in this bucket can ask for (for a warm-up that captures them
+        all): single waves with and without the merge, and blocks of eight waves in the groups
+        where some number of requests that runs in this bucket gets them."""
+        from .key_runs import wants_blocks
+        heads = [g.spec.num_kv_heads for g in self.runner.cache.groups]
+        out = [(True, (False,) * len(heads)), (False, (False,) * len(heads))]
+        for r in range(self.B // 2 + 1, self.B + 1):
+            v = (False, tuple(wants_blocks(r, h) for h in heads))
+            if any(v[1]) and v not in out:
+                out.append(v)
+        return out
+
     def _context(self, batch):
         from .runner import StepContext
         rn = self.runner
         return StepContext(rn.ops, rn.act_dtype, batch, rn.max_model_len, rn._calls, rn.cache)
 
-    def capture(self, merge: bool = True) -> None:
-        """Captures the variant with (or without) the kernel that merges partial attention
-        results, unless it exists."""
-        if merge in self._variants:
+    def capture(self, variant: tuple | None = None) -> None:
+        """Captures a variant of the step, unless it exists: ``variant`` = (whether partial
+        attention results are merged, per cache group whether a run of keys gets a block of eight
+        waves); None: with the merge, single waves."""
+        if variant is None:
+            variant = (True, (False,) * len(self.batch.groups))
+        if variant in self._variants:
             return
         rn = self.runner
         pieces = [_Piece(safe, items) for safe, items in rn.model.graph_pieces()]
-        for gt in self.batch.groups:
-            gt.runs_merge = merge
+        for gt, blocks in zip(self.batch.groups, variant[1]):
+            gt.runs_merge, gt.runs_for_blocks = variant[0], blocks
         # the decode attention sizes its key splits for the longest context the engine allows
         # (batch.max_context), so the launch is the same whatever the requests hold
         side = torch.cuda.Stream(device=rn.device)
@@ -282,7 +299,7 @@ class DecodeGraph:
                 gc.enable()
         torch.cuda.current_stream(rn.device).wait_stream(side)
         torch.cuda.synchronize(rn.device)
-        self._variants[merge] = pieces
+        self._variants[variant] = pieces
 
     def _live_batch(self, R: int) -> StepBatch:
         """The first R rows of the graph's tables as a step of their own, with the host's
@@ -309,10 +326,10 @@ class DecodeGraph:
         step that is launched before the host knows them.  Returns the logits of the graph's
         rows ([bucket, vocab], or [len(entries), vocab] if the step's last piece ran eagerly)."""
         self.fill(entries)
-        merge = self.tables.needs_merge
-        if merge not in self._variants:
-            self.capture(merge)
-        pieces = self._variants[merge]
+        variant = self.tables.variant
+        if variant not in self._variants:
+            self.capture(variant)
+        pieces = self._variants[variant]
         self.dev.copy_(self.host, non_blocking=True)
         self._copied.record()
         R = len(entries)

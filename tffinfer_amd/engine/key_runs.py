@@ -5,37 +5,41 @@ waves is as slow as its longest request: sixty-three requests of a thousand
 tokens beside one of thirty thousand wait for the waves of that one, five times
 as long as the bytes of the step need.  The host knows every request's length
 when it writes the step's tables, so it cuts each request's visible keys into
-runs of about the same length and the kernel gives a wave (or a block of
-waves) to every (run, kv head): a short request is one run, a long one many,
-and all waves end together.  The tables are written anew for every step,
-captured or not; their size depends only on the number of rows, so a captured
-launch serves any mix of lengths.
+runs of about the same length and the kernel gives a wave to every (run, kv
+head): a short request is one run, a long one many, and all waves end
+together.  The tables are written anew for every step, captured or not; their
+size depends only on the number of rows, so a captured launch serves any mix of
+lengths.
 
 How many runs: the kernel's waves fill a SIMD's registers alone, so the GPU
 holds RESIDENT_WAVES of them at once, and a wave that streams alone is bound by
 latency, not by bandwidth.  Measured on decode steps of 1 to 128 requests: some
 TARGET_WAVES waves, none beyond what is resident, runs of LONG_STEPS steps and
-more as long as BUSY_WAVES waves have work, never under MIN_STEPS.  Between
-BLOCK_PAIRS[0] and BLOCK_PAIRS[1] pairs of request and kv head a block of eight
-waves per run, which merges its waves' results in LDS, is faster than single
-waves whose results a second kernel merges; a CU holds one such block, so
-requests of about one length stay a run each, and only a request longer than
-one and a half times the median is cut, into runs no longer than that.
+more as long as BUSY_WAVES waves have work, never under MIN_STEPS; with so many
+requests that the waves' fair share is most of a request, a run a request.
+
+Between BLOCK_PAIRS[0] and BLOCK_PAIRS[1] pairs of request and kv head, and
+requests of about one length (the longest within BLOCK_SPREAD of the average),
+a block of eight waves per request and kv head, which merges its waves'
+results in LDS, is faster than single waves whose results a second kernel
+merges: every request is one run then, and ``blocks`` says so.  A CU holds one
+such block, and a block is as slow as its request is long, so uneven lengths
+go to single waves.
 
 Pure host code (numpy).  The reference has one sequence per forward and no such
 table (src/core/runtime/InferRuntime.cu:415-429).
 """
 from __future__ import annotations
 
+from typing import NamedTuple
+
 import numpy as np
 
 #: keys a wave works through at a time: a run begins a multiple of this after its request's
 #: first visible key rounded down to a multiple of it
 KEY_STEP = 32
-#: compute units; a block of eight waves has one to itself
-CUS = 256
-#: waves of one wave a block that the GPU holds at once (four SIMDs a CU, a wave a SIMD)
-RESIDENT_WAVES = 4 * CUS
+#: waves of one wave a block that the GPU holds at once (256 CUs, four SIMDs a CU, a wave a SIMD)
+RESIDENT_WAVES = 1024
 #: waves a launch aims at when single waves take the runs
 TARGET_WAVES = 768
 #: no run is shorter than this many steps of keys (a request that has fewer is one run) ...
@@ -43,50 +47,52 @@ MIN_STEPS = 4
 #: ... nor shorter than this many while as many waves as BUSY_WAVES are left with work
 LONG_STEPS = 8
 BUSY_WAVES = 256
-#: pairs of request and kv head between which a run gets a block of eight waves
+#: pairs of request and kv head between which requests of about one length get a block of eight
+#: waves each ...
 BLOCK_PAIRS = (160, 256)
-#: no block's run is shorter than this many steps (three a wave)
-BLOCK_MIN_STEPS = 24
-#: blocks of a launch at most: two rounds of a block a CU
-BLOCK_SLOTS = 2 * CUS
+#: ... "about one length": the longest request has at most this many times the average's keys
+BLOCK_SPREAD = 1.2
+
+
+class KeyRuns(NamedTuple):
+    runs: np.ndarray         # int32 [max_key_runs, 4]: (row, first key, end of keys, the row's position); row -1: not in use
+    run_start: np.ndarray    # int32 [rows + 1]: row r has the runs run_start[r] .. run_start[r + 1] - 1
+    blocks: bool             # dealt for a block of eight waves per run
+    merge: bool              # some row has several runs: partial results have to be merged
 
 
 def wants_blocks(rows: int, waves_per_run: int) -> bool:
-    """Whether the runs of ``rows`` requests are dealt for blocks of eight waves."""
+    """Whether ``rows`` requests, if they are of about one length, get a block of eight waves each."""
     return BLOCK_PAIRS[0] <= int(rows) * max(1, int(waves_per_run)) <= BLOCK_PAIRS[1]
 
 
-def max_key_runs(rows: int, waves_per_run: int, blocks: bool | None = None) -> int:
+def max_key_runs(rows: int, waves_per_run: int) -> int:
     """Runs that :func:`deal_key_runs` makes at most for ``rows`` requests, whatever their lengths:
     the size of the tables.  A multiple of eight: the kernel's blocks go to the eight XCDs in turn,
     and run i is to be on XCD i % 8 with all its kv heads."""
-    if blocks is None:
-        blocks = wants_blocks(rows, waves_per_run)
-    slots = BLOCK_SLOTS if blocks else RESIDENT_WAVES
-    return (max(int(rows), slots // max(1, int(waves_per_run))) + 7) & ~7
+    return (max(int(rows), RESIDENT_WAVES // max(1, int(waves_per_run))) + 7) & ~7
 
 
 def deal_key_runs(positions, window: int, waves_per_run: int, runs_out: np.ndarray | None = None,
                   start_out: np.ndarray | None = None, blocks: bool | None = None,
-                  target: int | None = None, min_steps: int | None = None):
+                  target: int | None = None, min_steps: int | None = None, live: int | None = None) -> KeyRuns:
     """``positions`` [R]: the position of each request's one new token (as many tokens are cached
     before it); ``window`` > 0: a token sees only the last ``window`` keys, itself included;
     ``waves_per_run``: waves (or blocks) that the kernel starts per run: the kv heads.  ``blocks``:
-    whether a run gets a block of eight waves (None: by the number of rows).  ``target`` and
-    ``min_steps`` override the number of waves aimed at and the shortest run (for tests).
+    whether a run gets a block of eight waves (None: by the number of rows and their lengths).
+    ``live``: the first so many rows are requests, the others padding (a captured step's), which
+    does not count where the requests' number and lengths decide.  ``target`` and ``min_steps`` override the number of waves (or blocks) aimed at and the
+    shortest run (for tests).
 
-    Returns (runs int32 [max_key_runs(R), 4], run_start int32 [R + 1]): run i is (row, first key,
-    end of keys, the row's position); the runs of row r are run_start[r] .. run_start[r + 1] - 1,
-    in the order of their keys, without gap or overlap, from the row's first visible key rounded
-    down to a multiple of KEY_STEP to its new token, all of one length but the last, which is no
-    longer; runs beyond run_start[R] have row -1.  ``runs_out`` (flat, 4 ints a run) and
-    ``start_out`` are written if given."""
+    The runs of row r are ``run_start[r] .. run_start[r + 1] - 1``, in the order of their keys,
+    without gap or overlap, from the row's first visible key rounded down to a multiple of
+    KEY_STEP to its new token, all of one length but the last, which is no longer; runs beyond
+    ``run_start[R]`` have row -1.  ``runs_out`` (flat, 4 ints a run) and ``start_out`` are
+    written if given."""
     P = np.asarray(positions, dtype=np.int64)
     R = P.shape[0]
     wps = max(1, int(waves_per_run))
-    if blocks is None:
-        blocks = wants_blocks(R, wps)
-    cap = max_key_runs(R, wps, blocks)
+    cap = max_key_runs(R, wps)
     runs = np.empty(4 * cap, dtype=np.int32) if runs_out is None else runs_out
     start = np.empty(R + 1, dtype=np.int32) if start_out is None else start_out
     if runs.shape[0] < 4 * cap or start.shape[0] < R + 1:
@@ -95,28 +101,30 @@ def deal_key_runs(positions, window: int, waves_per_run: int, runs_out: np.ndarr
     start[0] = 0
     if R == 0:
         runs[0:4 * cap:4] = -1
-        return runs[:4 * cap].reshape(-1, 4), start[:1]
+        return KeyRuns(runs[:4 * cap].reshape(-1, 4), start[:1], False, False)
     lo = np.maximum(0, P - window + 1) if window > 0 else np.zeros_like(P)
     first = lo // KEY_STEP * KEY_STEP
     steps = (P - first) // KEY_STEP + 1
     wave_steps = int(steps.sum()) * wps
-    typical = int(np.median(steps))
+    mine = steps if live is None else steps[:max(1, int(live))]
+    if blocks is None:
+        blocks = wants_blocks(mine.shape[0], wps) and int(mine.max()) * mine.shape[0] <= BLOCK_SPREAD * int(mine.sum())
+    slots = RESIDENT_WAVES
     if blocks:
-        # no run longer than one and a half times the typical request: requests of about one
-        # length are a run each, a block a CU at most; a request much longer than the others is
-        # cut to their measure
-        slots = BLOCK_SLOTS
-        chunk = max(BLOCK_MIN_STEPS if min_steps is None else int(min_steps), -(-3 * typical // 2))
+        # a run a row, unless a test asks for more
+        n = np.ones(R, dtype=np.int64)
+        chunk = int(steps.max())
         if target is not None:
-            chunk = max(1, -(-wave_steps // int(target)))
-        n = -(-steps // chunk)
+            chunk = max(1 if min_steps is None else int(min_steps), -(-wave_steps // int(target)))
+            n = -(-steps // chunk)
     else:
-        slots = RESIDENT_WAVES
+        typical = int(np.median(mine))
         floor = max(MIN_STEPS, min(LONG_STEPS, -(-wave_steps // BUSY_WAVES))) if min_steps is None else int(min_steps)
         share = -(-wave_steps // max(1, TARGET_WAVES if target is None else int(target)))
         if target is None and share * 5 > typical * 3:
             # so many requests that the waves' fair share is most of a request: requests of about
-            # one length stay a run each (nothing to merge then), as above
+            # one length stay a run each (nothing to merge then); a request much longer than the
+            # others is cut to their measure
             chunk = max(share, -(-3 * typical // 2))
             n = -(-steps // chunk)
         elif share >= floor:
@@ -144,4 +152,4 @@ def deal_key_runs(positions, window: int, waves_per_run: int, runs_out: np.ndarr
     runs[2:4 * total:4] = np.minimum(P[row] + 1, kb + KEY_STEP * per[row])
     runs[3:4 * total:4] = P[row]
     runs[4 * total:4 * cap:4] = -1
-    return runs[:4 * cap].reshape(-1, 4), start[:R + 1]
+    return KeyRuns(runs[:4 * cap].reshape(-1, 4), start[:R + 1], bool(blocks), total > R)

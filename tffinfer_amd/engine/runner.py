@@ -194,16 +194,17 @@ class ModelRunner:
         return want if n >= self.CAPTURE_AFTER else have
 
     def capture_graphs(self) -> int:
-        """Captures the decode graph of every bucket that has none yet (some 50 ms each, in both
-        of its variants), so that no step stops for a capture later; returns for how many
-        buckets it did."""
+        """Captures the decode graph of every bucket that has none yet (some 50 ms a variant: with
+        and without the merge of partial attention results on single waves, and for blocks of eight
+        waves where the bucket's rows may get them), so that no step stops for a capture later;
+        returns for how many buckets it did."""
         n = 0
         with torch.cuda.device(self.device):
             for bucket in self._graph_buckets:
                 if bucket not in self._graphs:
                     g = self._graphs[bucket] = DecodeGraph(self, bucket)
-                    g.capture(True)
-                    g.capture(False)
+                    for variant in g.possible_variants():
+                        g.capture(variant)
                     n += 1
         return n
 
