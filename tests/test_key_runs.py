@@ -81,17 +81,17 @@ def test_runs_are_of_similar_length():
     runs, start, _, _ = deal_key_runs([5, 100000], 0, 8)
     assert start[1] == 1
     # requests of one length: the launch stays within the waves that the GPU holds at once
+    assert deal_key_runs([2100] * 64, 0, 8).blocks
     for R, per_row in ((16, 6), (40, 3), (48, 2), (64, 1), (72, 1), (128, 1), (200, 1)):
-        assert not wants_blocks(R, 8)
-        runs, start, blocks, merge = deal_key_runs([2100] * R, 0, 8)
+        runs, start, blocks, merge = deal_key_runs([2100] * R, 0, 8, blocks=False)
         assert start[-1] == per_row * R, (R, start[-1])
-        assert (per_row == 1 or start[-1] * 8 <= RESIDENT_WAVES) and merge == (per_row > 1) and not blocks
+        assert (per_row == 1 or start[-1] * 8 <= RESIDENT_WAVES) and merge == (per_row > 1)
 
 
 def test_blocks_of_eight_waves_are_for_requests_of_about_one_length():
     rng = random.Random(5)
     for R in (20, 24, 32):
-        assert wants_blocks(R, 8) and BLOCK_PAIRS[0] <= R * 8 <= BLOCK_PAIRS[1]
+        assert wants_blocks(R, 8) and BLOCK_PAIRS[0][0] <= R * 8 <= BLOCK_PAIRS[0][1]
         # requests of one length, or of about one: a run each, the block's waves split it among them
         for pos in ([2100] * R, [2000 + 11 * i for i in range(R)]):
             runs, start, blocks, merge = deal_key_runs(pos, 0, 8)
@@ -111,7 +111,7 @@ def test_blocks_of_eight_waves_are_for_requests_of_about_one_length():
             assert lens.max() <= 1.5 * max(fair, steps[R // 2]) + 1, "a run much longer than the fair share and the median request"
     assert not wants_blocks(19, 8) and not wants_blocks(33, 8) and wants_blocks(128, 2) and not wants_blocks(1, 8)
     # too few or too many requests: single waves whatever the lengths
-    for R in (8, 19, 33, 64):
+    for R in (8, 19, 33, 48, 72):
         assert not deal_key_runs([2100] * R, 0, 8).blocks
 
 

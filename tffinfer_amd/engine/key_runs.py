@@ -18,8 +18,8 @@ TARGET_WAVES waves, none beyond what is resident, runs of LONG_STEPS steps and
 more as long as BUSY_WAVES waves have work, never under MIN_STEPS; with so many
 requests that the waves' fair share is most of a request, a run a request.
 
-Between BLOCK_PAIRS[0] and BLOCK_PAIRS[1] pairs of request and kv head, and
-requests of about one length (the longest within BLOCK_SPREAD of the average),
+With as many pairs of request and kv head as BLOCK_PAIRS says (most of a round
+of a block a CU, or of two), and requests of about one length (the longest within BLOCK_SPREAD of the average),
 a block of eight waves per request and kv head, which merges its waves'
 results in LDS, is faster than single waves whose results a second kernel
 merges: every request is one run then, and ``blocks`` says so.  A CU holds one
@@ -48,8 +48,8 @@ MIN_STEPS = 4
 LONG_STEPS = 8
 BUSY_WAVES = 256
 #: pairs of request and kv head between which requests of about one length get a block of eight
-#: waves each ...
-BLOCK_PAIRS = (160, 256)
+#: waves each (one round of a block a CU, or two full ones) ...
+BLOCK_PAIRS = ((160, 256), (448, 512))
 #: ... "about one length": the longest request has at most this many times the average's keys
 BLOCK_SPREAD = 1.2
 
@@ -63,7 +63,8 @@ class KeyRuns(NamedTuple):
 
 def wants_blocks(rows: int, waves_per_run: int) -> bool:
     """Whether ``rows`` requests, if they are of about one length, get a block of eight waves each."""
-    return BLOCK_PAIRS[0] <= int(rows) * max(1, int(waves_per_run)) <= BLOCK_PAIRS[1]
+    pairs = int(rows) * max(1, int(waves_per_run))
+    return any(lo <= pairs <= hi for lo, hi in BLOCK_PAIRS)
 
 
 def max_key_runs(rows: int, waves_per_run: int) -> int:
