@@ -93,7 +93,7 @@ def test_blocks_of_eight_waves_are_for_requests_of_about_one_length():
     for R in (20, 24, 32):
         assert wants_blocks(R, 8) and BLOCK_PAIRS[0][0] <= R * 8 <= BLOCK_PAIRS[0][1]
         # requests of one length, or of about one: a run each, the block's waves split it among them
-        for pos in ([2100] * R, [2000 + 11 * i for i in range(R)]):
+        for pos in ([2100] * R, [2000 + 11 * i for i in range(R)], [2000 + (997 * i) % 1000 for i in range(R)]):
             runs, start, blocks, merge = deal_key_runs(pos, 0, 8)
             assert blocks and not merge and start[-1] == R
             check_runs(runs, start, pos, 0)
@@ -101,7 +101,7 @@ def test_blocks_of_eight_waves_are_for_requests_of_about_one_length():
         runs, start, blocks, merge = deal_key_runs([2100] * R + [0] * 4, 0, 8, live=R)
         assert blocks and not merge and start[-1] == R + 4
         # uneven lengths go to single waves, the long requests cut to the others' measure
-        for pos in ([16383] * 3 + [1023] * (R - 3), [rng.randrange(300, 4300) for _ in range(R)]):
+        for pos in ([16383] * 3 + [1023] * (R - 3), [rng.choice([300, 300, 300, 4300]) for _ in range(R - 1)] + [4300]):
             runs, start, blocks, merge = deal_key_runs(pos, 0, 8)
             assert not blocks and merge and R < start[-1] <= RESIDENT_WAVES // 8
             check_runs(runs, start, pos, 0)

@@ -19,8 +19,8 @@ more as long as BUSY_WAVES waves have work, never under MIN_STEPS; with so many
 requests that the waves' fair share is most of a request, a run a request.
 
 With as many pairs of request and kv head as BLOCK_PAIRS says (most of a round
-of a block a CU, or of two), and requests of about one length (the longest within BLOCK_SPREAD of the average),
-a block of eight waves per request and kv head, which merges its waves'
+of a block a CU, or of two), and requests of about one length (the longest no more than some two times the
+average, see BLOCK_RATE_SHARE), a block of eight waves per request and kv head, which merges its waves'
 results in LDS, is faster than single waves whose results a second kernel
 merges: every request is one run then, and ``blocks`` says so.  A CU holds one
 such block, and a block is as slow as its request is long, so uneven lengths
@@ -50,8 +50,11 @@ BUSY_WAVES = 256
 #: pairs of request and kv head between which requests of about one length get a block of eight
 #: waves each (one round of a block a CU, or two full ones) ...
 BLOCK_PAIRS = ((160, 256), (448, 512))
-#: ... "about one length": the longest request has at most this many times the average's keys
-BLOCK_SPREAD = 1.2
+#: ... "about one length": a block's eight waves stream some 45 GB/s, all blocks together what HBM
+#: gives (5 TB/s, 111 times as much), so the blocks are as fast as the bytes allow as long as the
+#: longest request has no more than pairs / 111 times the average's keys (per round of blocks)
+BLOCK_RATE_SHARE = 111
+CUS = 256
 
 
 class KeyRuns(NamedTuple):
@@ -109,7 +112,9 @@ def deal_key_runs(positions, window: int, waves_per_run: int, runs_out: np.ndarr
     wave_steps = int(steps.sum()) * wps
     mine = steps if live is None else steps[:max(1, int(live))]
     if blocks is None:
-        blocks = wants_blocks(mine.shape[0], wps) and int(mine.max()) * mine.shape[0] <= BLOCK_SPREAD * int(mine.sum())
+        pairs = mine.shape[0] * wps
+        spread = max(1.2, pairs / (BLOCK_RATE_SHARE * -(-pairs // CUS)))
+        blocks = wants_blocks(mine.shape[0], wps) and int(mine.max()) * mine.shape[0] <= spread * int(mine.sum())
     slots = RESIDENT_WAVES
     if blocks:
         # a run a row, unless a test asks for more
