@@ -1011,7 +1011,7 @@ def test_attention_decode_fused(nq, nkv, d, ps, window, splits, pairing, with_no
     assert ops.decode_fused_supported(qkv.to(DEV), d, ps, table, pr, batch)
     how = dict(splits=splits)
     if isinstance(splits, str):
-        from tffinfer_amd.engine.key_runs import deal_key_runs
+        from tffinfer_amd.kernels.key_runs import deal_key_runs
         runs, run_start, _, merge = deal_key_runs([P for P, _ in entries], window, nkv, target=int(splits.split()[1]), min_steps=1,
                                                   blocks=False)
         assert merge and run_start[-1] > R, "no entry has several runs"
@@ -1107,7 +1107,7 @@ def test_attention_decode_fused_keys_dealt_into_runs(nq, nkv, d, ps, window, wav
     the token's own key and value from registers and into their page.  Tables with runs that are
     not in use, and with a padding row's run, as a captured step has them."""
     ops = _ops()
-    from tffinfer_amd.engine.key_runs import deal_key_runs
+    from tffinfer_amd.kernels.key_runs import deal_key_runs
     far = 77
     entries = [(20000, 1), (40, 1), (0, 1), (95, 1), (96, 1), (3000, 1), (255, 1), (256, 1), (31, 1), (32, 1), (1023, 1)]
     batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=3 + d)
@@ -1150,7 +1150,8 @@ def test_attention_decode_fused_keys_dealt_into_runs(nq, nkv, d, ps, window, wav
 @pytest.mark.parametrize("nq,nkv,d,ps,window", [(32, 8, 128, 16, 0), (8, 2, 32, 8, 300), (40, 2, 96, 8, 0)])
 def test_attention_mfma_portions_beside_decoding_requests(nq, nkv, d, ps, window):
     """A step of long portions and of requests that bring one token with a long context: the
-    latter go to the split-key kernel, the former to the block kernel, into the same output."""
+    latter have their keys dealt into runs for single waves (the longest one into several, whose
+    partial results are merged), the former go to the block kernel, into the same output."""
     ops = _ops()
     entries = [(900, 1), (0, 300), (40, 1), (333, 150), (1500, 1), (7, 1)]
     batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=nq + d)
@@ -1159,9 +1160,16 @@ def test_attention_mfma_portions_beside_decoding_requests(nq, nkv, d, ps, window
     q = torch.randn(T, nq, d, generator=g).to(torch.bfloat16)
     scale = 1 / math.sqrt(d)
     out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale)
+    runs, run_start, tokens, merge = batch._attn_work[("single_runs", nkv, window)]
+    assert merge and run_start.tolist()[-1] > 4 and tokens.tolist() == [0, 301, 452, 453]
     gen = ops.attention_generic(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv.k_cache, kv.v_cache, kv.block_tables,
                                 batch.token_req, batch.positions, window, scale)
     _close(out, gen.double(), ATTN_TOL, "mixed step against the general kernel")
+    # every entry's keys split alike, as before the runs: the same to rounding
+    batch._attn_work.clear()
+    same = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale, splits=3)
+    assert "single_rows" in batch._attn_work
+    _close(same, gen.double(), ATTN_TOL, "mixed step with equal splits against the general kernel")
     cu = batch.host_cu_tokens
     for r, (P, n) in enumerate(entries):
         mine = torch.tensor([cu[r], cu[r + 1] - 1])
@@ -1172,8 +1180,8 @@ def test_attention_mfma_portions_beside_decoding_requests(nq, nkv, d, ps, window
 @pytest.mark.parametrize("nq,nkv,d,ps,window", [(32, 8, 128, 16, 0), (8, 2, 32, 8, 300), (40, 2, 96, 8, 0)])
 def test_attention_mfma_short_portions_beside_decoding_requests(nq, nkv, d, ps, window):
     """Portions of a few tokens (a wave of their own per 16 columns) beside requests that bring
-    one token with a long context: those go to the split-key kernel here too, not to a single
-    wave that walks all their keys."""
+    one token with a long context: those have their keys dealt into runs here too, and do not go
+    to a single wave that walks all their keys."""
     ops = _ops()
     entries = [(900, 1), (0, 3), (1500, 1), (44, 2), (300, 1), (9, 1)]
     batch, kv, ks, vs, positions, token_req = _fake_step(entries, ps, nkv, d, torch.bfloat16, seed=nq + d + 1)
@@ -1183,7 +1191,7 @@ def test_attention_mfma_short_portions_beside_decoding_requests(nq, nkv, d, ps, 
     q = torch.randn(T, nq, d, generator=g).to(torch.bfloat16)
     scale = 1 / math.sqrt(d)
     out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale)
-    assert "single_rows" in batch._attn_work, "the decoding requests did not get the split-key launch"
+    assert ("single_runs", nkv, window) in batch._attn_work, "the decoding requests' keys were not dealt into runs"
     for r in range(len(entries)):
         sel = (token_req == r).nonzero().flatten()
         ref = _attn_ref(q[sel], ks[r], vs[r], positions[sel], window, scale)

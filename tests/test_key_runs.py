@@ -7,7 +7,7 @@ import random
 import numpy as np
 import pytest
 
-from tffinfer_amd.engine.key_runs import (BLOCK_PAIRS, BUSY_WAVES, KEY_STEP, LONG_STEPS, MIN_STEPS, RESIDENT_WAVES,
+from tffinfer_amd.kernels.key_runs import (BLOCK_PAIRS, BUSY_WAVES, KEY_STEP, LONG_STEPS, MIN_STEPS, RESIDENT_WAVES,
                                           TARGET_WAVES, deal_key_runs, max_key_runs, wants_blocks)
 
 

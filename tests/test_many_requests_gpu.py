@@ -97,7 +97,8 @@ def test_twenty_eight_requests_shrinking_through_the_graph_buckets(model_dirs, n
     assert {28, 24, 16, 12, 8}.issubset(graphs), graphs
     assert standins, "no graph ever stood in for a smaller one"
     if dtype == "bfloat16":
-        assert seen["blocks"] == ({True, False} if even else {False}), "blocks of eight waves are for requests of about one length"
+        assert False in seen["blocks"] and (True in seen["blocks"] or not even), \
+            "single waves should have run, and blocks of eight waves for the requests of about one length"
         assert any(17 <= rows <= 64 and parts > 1 for rows, parts in seen["stacks"]), \
             "no product of 17 to 64 rows kept partial sums for the norm"
     for i in range(n):

@@ -191,7 +191,7 @@ __global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
     // has its place: strewn among the others they took places on half of the CUs and left the
     // waves with work crowded on the other half (a fifth slower at 64 entries of one run each).
     bool by_runs = false;
-    if constexpr (FUSED && (SPLIT || BW > 1)) by_runs = fz.key_runs != nullptr;
+    if constexpr (SPLIT || (FUSED && BW > 1)) by_runs = fz.key_runs != nullptr;
     int r, col0, g = blockIdx.y, run_index = 0;
     int4 run = make_int4(0, 0, 0, 0);
     if (by_runs) {
@@ -210,9 +210,10 @@ __global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
         col0 = (blockIdx.x % tiles_per_entry) * 16;
     }
     const int G = nq / nkv;
-    // (a run brings its entry's position with it, and its entry has one token: nothing to wait
-    // for between the run and the page numbers)
-    const int tok0 = by_runs ? r : cu_tokens[r];
+    // (a run brings its entry's position with it, and its entry has one token, which in a step of
+    // one token per entry, as the fused form takes it, is the entry's number: nothing to wait for
+    // between the run and the page numbers)
+    const int tok0 = (FUSED && by_runs) ? r : cu_tokens[r];
     const int n = by_runs ? 1 : cu_tokens[r + 1] - tok0;
     const int P = by_runs ? run.w : start_pos[r];
     const int ncols = n * G;
@@ -721,6 +722,7 @@ __global__ __launch_bounds__(256) void attn_run_merge_kernel(const float* __rest
                                                               const float* __restrict__ part_ml,
                                                               bf16_t* __restrict__ out,
                                                               const int32_t* __restrict__ run_start,
+                                                              const int32_t* __restrict__ tokens,
                                                               int R, int nq, int d) {
     const int lane = threadIdx.x & 63;
     const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);     // (entry, head), heads fastest
@@ -782,7 +784,7 @@ __global__ __launch_bounds__(256) void attn_run_merge_kernel(const float* __rest
             }
     }
     const float inv = 1.0f / l;
-    bf16_t* o = out + ((size_t)r * nq + h) * d;
+    bf16_t* o = out + ((size_t)(tokens ? tokens[r] : r) * nq + h) * d;   // (tokens: the row of out that entry r's token has)
     if (e0 < d) {
         o[e0] = (bf16_t)(acc[0].x * inv);
         o[e0 + 1] = (bf16_t)(acc[0].y * inv);
@@ -1160,7 +1162,8 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
                        const int32_t* work, int num_work, const int32_t* block_items, int num_blocks,
                        int tiles_per_entry, int cols_per_wave,
                        int splits, int nq, int nkv, int page_size, int window, float scale,
-                       int T_total, hipStream_t s, const AttnFuse* fuse = nullptr, int key_groups = 2) {
+                       int T_total, hipStream_t s, const AttnFuse* fuse = nullptr, int key_groups = 2,
+                       const AttnFuse* runs_only = nullptr) {
     int page_shift = 0;   // the page size is a power of two (tff_attention_mfma_supported)
     while ((1 << page_shift) < page_size) ++page_shift;
     if (cols_per_wave == 256) {
@@ -1197,7 +1200,9 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
         return tff_check_launch("attention_mfma_block");
     }
     const dim3 grid(num_work, nkv, max(splits, 1));
-    const AttnFuse fz = fuse ? *fuse : AttnFuse{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0, nullptr};
+    // (runs_only: nothing to fuse, q is finished and the pages hold the tokens; only the runs of keys are set)
+    const AttnFuse fz = fuse ? *fuse : runs_only ? *runs_only
+                                                 : AttnFuse{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0, nullptr};
 #define TFF_ATTN_ARGS                                                                              \
     q, q_stride, out, part_o, part_ml, k_cache, v_cache, block_tables, bt_stride, cu_tokens,       \
         start_pos, work, tiles_per_entry, nq, nkv, page_size, page_shift, window, scale, T_total
@@ -1220,6 +1225,9 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
             attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 1), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
         else
             attn_wave_kernel<DT, false, (DT <= 8 ? 4 : 1), true><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
+    } else if (fz.key_runs) {
+        // (the same for q, k and v that are finished and in their pages)
+        attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 2)><<<dim3(num_work * nkv, 1, tiles_per_entry), 64, 0, s>>>(TFF_ATTN_ARGS, fz);
     } else if (splits > 1) {
         attn_wave_kernel<DT, true, (DT <= 8 ? 4 : 2)><<<grid, 64, 0, s>>>(TFF_ATTN_ARGS, fz);
     } else {
@@ -1442,7 +1450,62 @@ TFF_API int tff_attention_decode_runs(const void* qkv, int qkv_stride, void* out
     }
 #undef TFF_ATTN_CASE
     if (rc || !merge) return rc;
-    attn_run_merge_kernel<<<(R * nq + 3) / 4, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, run_start, R, nq, d);
+    attn_run_merge_kernel<<<(R * nq + 3) / 4, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, run_start, nullptr, R, nq, d);
+    return tff_check_launch("attention_run_merge");
+}
+
+// Entries of one token among a step's entries (requests that decode beside prompt portions), q
+// finished and the tokens' keys and values in their pages (tff_qk_norm_rope_kv), their keys
+// dealt into runs by the caller as for tff_attention_decode_runs: key_runs [num_runs][4] = (the
+// entry's row in the step's tables, first key, end of keys, the entry's position); the runs of
+// the i-th such entry are run_start[i] .. run_start[i + 1] - 1 (run_start [num_entries + 1]) and
+// tokens[i] is its token's row in q and out.  Rows of out that belong to other entries are not
+// touched.  merge 0: the caller knows that every such entry is one run.
+TFF_API int tff_attention_mfma_runs(const void* q, int q_stride, void* out, float* part_o, float* part_ml,
+                                    const void* k_cache, const void* v_cache,
+                                    const int32_t* block_tables, int bt_stride,
+                                    const int32_t* cu_tokens, const int32_t* start_pos,
+                                    const int32_t* key_runs, const int32_t* run_start,
+                                    const int32_t* tokens, int num_runs, int num_entries, int merge,
+                                    int T, int nq, int nkv, int d, int page_size, int num_pages,
+                                    int window, float scale, tff_stream_t stream) {
+    TFF_REQUIRE(q && out && k_cache && v_cache && block_tables && cu_tokens && start_pos,
+                "attention_mfma_runs: null pointer");
+    TFF_REQUIRE(key_runs && run_start && tokens && part_o && part_ml,
+                "attention_mfma_runs: the runs, the tokens' rows and the workspace are needed");
+    TFF_REQUIRE(((uintptr_t)key_runs % 16) == 0, "attention_mfma_runs: key_runs must be 16-byte aligned");
+    TFF_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0,
+                "attention_mfma_runs: %d query heads are not a multiple of %d key heads", nq, nkv);
+    TFF_REQUIRE(tff_attention_mfma_supported(d, page_size),
+                "attention_mfma_runs: head size %d with pages of %d is not supported by the matrix-core kernel",
+                d, page_size);
+    TFF_REQUIRE(q_stride >= nq * d && q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0,
+                "attention_mfma_runs: q rows of %d elements must hold nq*d = %d and be 16-byte aligned", q_stride, nq * d);
+    const int tiles = (nq / nkv + 15) / 16;
+    TFF_REQUIRE(num_runs >= 0 && num_runs % 8 == 0 && (long)num_runs * nkv < (1L << 31) && tiles <= 65535 && d <= 256,
+                "attention_mfma_runs: %d runs (a multiple of eight is needed), %d kv heads, %d column tiles (at most "
+                "65,535), head size %d (at most 256)", num_runs, nkv, tiles, d);
+    TFF_REQUIRE(bt_stride > 0 && num_pages > 0 && window >= 0 && num_entries >= 0 && T >= 0, "attention_mfma_runs: bad geometry");
+    if (num_entries == 0 || num_runs == 0) return 0;
+    AttnFuse fz{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0, key_runs};
+    hipStream_t s = (hipStream_t)stream;
+    int rc = -1;
+#define TFF_ATTN_CASE(DTV)                                                                          \
+    case DTV * 16:                                                                                  \
+        rc = launch_attn<DTV>((const bf16_t*)q, q_stride, (bf16_t*)out, part_o, part_ml,            \
+                              (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,         \
+                              bt_stride, cu_tokens, start_pos, nullptr, num_runs, nullptr, 0,       \
+                              tiles, 16, 2, nq, nkv, page_size, window, scale, T, s, nullptr, 2, &fz); \
+        break;
+    switch (d) {
+        TFF_ATTN_CASE(1) TFF_ATTN_CASE(2) TFF_ATTN_CASE(3) TFF_ATTN_CASE(4) TFF_ATTN_CASE(5)
+        TFF_ATTN_CASE(6) TFF_ATTN_CASE(7) TFF_ATTN_CASE(8) TFF_ATTN_CASE(12) TFF_ATTN_CASE(16)
+        default: return tff_fail("attention_mfma_runs: head size %d", d);
+    }
+#undef TFF_ATTN_CASE
+    if (rc || !merge) return rc;
+    attn_run_merge_kernel<<<(num_entries * nq + 3) / 4, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, run_start, tokens,
+                                                                    num_entries, nq, d);
     return tff_check_launch("attention_run_merge");
 }
 

@@ -23,7 +23,7 @@ int tff_check_launch(const char* what) {
     return 0;
 }
 TFF_API const char* tff_last_error() { return g_error; }
-TFF_API int tff_abi_version() { return 20; }
+TFF_API int tff_abi_version() { return 21; }
 
 // ----------------------------------------------------------------- embed ---
 // x[t, :] = E[token[t], :]   (reference: src/kernel/cpu/embedding.cpp:34-49,

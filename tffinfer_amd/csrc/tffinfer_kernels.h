@@ -181,6 +181,23 @@ TFF_API int tff_attention_decode_runs(const void* qkv, int qkv_stride, void* out
                                       int block_waves, int merge, int R, int nq, int nkv, int d, int page_size,
                                       int num_pages, int window, float scale, tff_stream_t stream);
 
+// The entries of one token among a step's entries (requests that decode beside prompt portions),
+// with q finished and the tokens' keys and values in their pages (tff_qk_norm_rope_kv), and
+// their keys dealt into runs as for tff_attention_decode_runs: key_runs [num_runs][4] = (the
+// entry's row in the step's tables, first key, end of keys, the entry's position); the runs of
+// the i-th such entry are run_start[i] .. run_start[i + 1] - 1 (run_start [num_entries + 1]) and
+// tokens[i] is its token's row in q and out; other rows of out are not touched.  Workspace:
+// part_o [num_runs, nq, d], part_ml [num_runs, nq, 2].  num_runs is a multiple of eight; merge 0:
+// the caller knows that every such entry is one run.  T: rows of q.
+TFF_API int tff_attention_mfma_runs(const void* q, int q_stride, void* out, float* part_o, float* part_ml,
+                                    const void* k_cache, const void* v_cache,
+                                    const int32_t* block_tables, int bt_stride,
+                                    const int32_t* cu_tokens, const int32_t* start_pos,
+                                    const int32_t* key_runs, const int32_t* run_start,
+                                    const int32_t* tokens, int num_runs, int num_entries, int merge,
+                                    int T, int nq, int nkv, int d, int page_size, int num_pages,
+                                    int window, float scale, tff_stream_t stream);
+
 // tff_attention_decode_fused followed by tff_attention_split_reduce, for callers that cannot
 // allocate device memory: code under HIP graph capture, tight serving loops, harnesses that
 // forbid hipMalloc.  It has no counterpart in the reference.  The partial results of split keys

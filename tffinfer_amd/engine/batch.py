@@ -13,7 +13,7 @@ from dataclasses import dataclass, field
 
 import torch
 
-from .key_runs import deal_key_runs
+from ..kernels.key_runs import deal_key_runs
 
 
 @dataclass
@@ -39,7 +39,7 @@ class KVView:
         self.page_size = page_size
         self.group = group
         # a step of one token per request: the requests' visible keys dealt into runs of similar
-        # length (engine.key_runs), for a window of runs_window, for single waves or for blocks
+        # length (kernels.key_runs), for a window of runs_window, for single waves or for blocks
         # of eight; else None
         self.key_runs = key_runs
         self.run_start = run_start
@@ -57,7 +57,7 @@ class GroupTables:
         self.block_tables = block_tables        # int32 [R, max_blocks]
         self.slot_mapping = slot_mapping        # int32 [T]: page * page_size + offset of each new token
         self.no_slot_mapping = no_slot_mapping  # int32 [T] of -1: for calls that only read a cache
-        self.key_runs = key_runs                # int32 [runs, 4] or None (engine.key_runs)
+        self.key_runs = key_runs                # int32 [runs, 4] or None (kernels.key_runs)
         self.run_start = run_start              # int32 [R + 1] or None
         self.runs_window = runs_window
         self.runs_for_blocks = runs_for_blocks

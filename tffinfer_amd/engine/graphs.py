@@ -30,7 +30,7 @@ import numpy as np
 import torch
 
 from .batch import GroupTables, StepBatch
-from .key_runs import deal_key_runs, max_key_runs
+from ..kernels.key_runs import deal_key_runs, max_key_runs
 
 
 def _pad4(n: int) -> int:
@@ -229,7 +229,7 @@ class DecodeGraph:
         """The variants that steps in this bucket can ask for (for a warm-up that captures them
         all): single waves with and without the merge, and blocks of eight waves in the groups
         where some number of requests that runs in this bucket gets them."""
-        from .key_runs import wants_blocks
+        from ..kernels.key_runs import wants_blocks
         heads = [g.spec.num_kv_heads for g in self.runner.cache.groups]
         out = [(True, (False,) * len(heads)), (False, (False,) * len(heads))]
         for r in range(self.B // 2 + 1, self.B + 1):

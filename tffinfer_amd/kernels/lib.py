@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 20
+ABI_VERSION = 21
 
 
 class KernelLibraryError(RuntimeError):
@@ -41,6 +41,8 @@ _SIGNATURES = {
                                    _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "tff_attention_decode_runs": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _F, _P, _I, _I,
                                   _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
+    "tff_attention_mfma_runs": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I,
+                                _I, _F, _P],
     "tff_attention_decode_fused_static": [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _F, _P, _I, _I,
                                           _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "tff_attention_split_reduce": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _P],

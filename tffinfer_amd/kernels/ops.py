@@ -19,6 +19,7 @@ import numpy as np
 import torch
 
 from . import lib as _lib
+from .key_runs import deal_key_runs
 from . import staging as _staging
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
@@ -657,13 +658,36 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
         # contexts: they get the split-key kernel of their own rather than one block, or one
         # wave, each for all their keys.
         which = "multi"
-        work = _attention_work(batch, G, 16, q.device, "single")
-        cache = batch._attn_work
-        if "single_rows" not in cache:
-            cu = batch.host_cu_tokens
-            cache["single_rows"] = _staging.send(q.device, [np.asarray([(r, cu[r]) for r in single], dtype=np.int32)])[0]
-        sp = splits if splits is not None else pick_splits(work.shape[0] * nkv, batch.max_context)
-        launch(work, work.shape[0], None, 0, 1, 16, sp, cache["single_rows"])
+        cache = getattr(batch, "_attn_work", None)
+        if cache is None:
+            cache = batch._attn_work = {}
+        if splits is None and getattr(batch, "host_start_pos", None) is not None:
+            # their keys dealt into runs of similar length, whatever the requests' lengths
+            key = ("single_runs", nkv, int(window))
+            if key not in cache:
+                cu = batch.host_cu_tokens
+                dealt = deal_key_runs([batch.host_start_pos[r] for r in single], int(window), nkv, blocks=False)
+                runs = dealt.runs.copy()
+                used = int(dealt.run_start[-1])
+                runs[:used, 0] = np.asarray(single, dtype=np.int32)[runs[:used, 0]]     # rows of the step's tables
+                cache[key] = tuple(_staging.send(q.device, [runs, dealt.run_start.copy(),
+                                                            np.asarray([cu[r] for r in single], dtype=np.int32)])) \
+                    + (dealt.merge,)
+            runs, run_start, tokens, merge = cache[key]
+            part_o = torch.empty(runs.shape[0], nq, d, dtype=torch.float32, device=q.device)
+            part_ml = torch.empty(runs.shape[0], nq, 2, dtype=torch.float32, device=q.device)
+            _lib.check(L.tff_attention_mfma_runs(
+                q.data_ptr(), q.stride(0), out.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), k_cache.data_ptr(),
+                v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(), batch.start_pos.data_ptr(),
+                runs.data_ptr(), run_start.data_ptr(), tokens.data_ptr(), runs.shape[0], len(single), 1 if merge else 0,
+                T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale), stream))
+        else:
+            work = _attention_work(batch, G, 16, q.device, "single")
+            if "single_rows" not in cache:
+                cu = batch.host_cu_tokens
+                cache["single_rows"] = _staging.send(q.device, [np.asarray([(r, cu[r]) for r in single], dtype=np.int32)])[0]
+            sp = splits if splits is not None else pick_splits(work.shape[0] * nkv, batch.max_context)
+            launch(work, work.shape[0], None, 0, 1, 16, sp, cache["single_rows"])
     if cols == 128:
         bcols = block_cols or _pick_block_cols(batch, G, nkv, int(window), q.device, which, d)
         if bcols == 256:
@@ -708,7 +732,7 @@ def attention_decode_fused(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weigh
     position); None: no token's, the pages hold them already.  ``key_runs``
     (int32 [runs, 4]: row, first key, end of keys, the row's position) and ``run_start`` (int32
     [R + 1]): the rows' keys dealt into runs by the host, a wave per run and
-    kv head (``engine.key_runs``), or a block of eight waves if they were
+    kv head (``kernels.key_runs``), or a block of eight waves if they were
     dealt for that (``runs_for_blocks``) and the head size allows it;
     ``runs_merge`` False: the caller knows that every row is one run, and the
     kernel that merges partial results is left out.  Without runs every
