@@ -41,6 +41,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048)
+    ap.add_argument("--contexts", default=None,
+                    help="with --only decode: requests of these context lengths instead of --batch requests of --context, "
+                         "comma-separated, NxC for N requests of C tokens (32768,63x1024)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="8b",
                     help="layer sizes: the benchmark configuration (8b) or one of the smaller and larger shapes")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
@@ -208,6 +211,15 @@ def main():
         print(json.dumps({"ceilings": c,
                           "published": {"hbm_GBps": M.HBM_PEAK_GBS, "bf16_TFLOPs": M.MFMA_PEAK["bf16"] / 1e12}}))
         return
+    contexts = None
+    if args.contexts:
+        if args.only != "decode":
+            raise SystemExit("--contexts goes with --only decode")
+        contexts = []
+        for part in args.contexts.split(","):
+            n, _, c = part.rpartition("x")
+            contexts += [int(c)] * (int(n) if n else 1)
+        args.batch, args.context = len(contexts), max(contexts)
     shape_name, shape = SHAPES[args.shape]
     cfg = dict(shape)
     L_full = cfg["num_hidden_layers"]
@@ -240,6 +252,8 @@ def main():
     max_batch = args.batch if (args.no_points or args.only) else max(args.batch, 64)
     total_steps = args.steps + args.warmup + M.decode_slack(max_batch, args.context) + 16
     kv_tokens = max_batch * (args.context + total_steps + args.page_size) + args.prefill_tokens
+    if contexts:
+        kv_tokens = sum(contexts) + max_batch * (total_steps + args.page_size)
     opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=kv_tokens, max_num_seqs=max_batch,
                         max_num_batched_tokens=max(4096, max_batch), prefill_chunk=2048,
                         max_model_len=headline_limit, use_graphs=not args.no_graphs)
@@ -257,7 +271,7 @@ def main():
             k, p, t, *rest = args.sampling.split(",")
             sampling = SamplingConfig(type="top_p", top_k=int(k), top_p=float(p), temperature=float(t), seed=args.seed,
                                       repetition_penalty=float(rest[0]) if rest else 1.0)
-        dec = M.measure_decode(engine, gen, args.batch, args.context, args.steps, args.warmup, vocab, sampling)
+        dec = M.measure_decode(engine, gen, args.batch, contexts or args.context, args.steps, args.warmup, vocab, sampling)
     if args.only:
         part = ({"prefill_ms": round(1000 * pre["wall_s"], 3), "prefill_ms_device": round(1000 * pre["device_s"], 3)}
                 if pre else
@@ -265,7 +279,7 @@ def main():
                  "decode_ms_per_step_median": round(1000 * dec["step_median_s"], 4)})
         if args.sampling:
             part["sampling"] = args.sampling
-        print(json.dumps({"only": args.only, **part, "batch": args.batch, "context": args.context}))
+        print(json.dumps({"only": args.only, **part, "batch": args.batch, "context": args.contexts or args.context}))
         return
     points, detail = {}, {}
     if not args.no_points:
