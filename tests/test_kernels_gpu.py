@@ -926,6 +926,16 @@ def test_attention_mfma_decode_split_keys(nq, nkv, d, ps, window, splits):
                        for r in range(T)])
     out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale, splits=splits)
     _close(out.reshape(T, nq, d), ref, ATTN_TOL, "split-key decode attention")
+    if splits is None:
+        # with the keys dealt into runs by the step's tables, as the engine brings them
+        from tffinfer_amd.kernels.key_runs import deal_key_runs
+        for target in (None, 40):
+            dealt = deal_key_runs([P for P, _ in entries], window, nkv, blocks=False, target=target, min_steps=1 if target else None)
+            kv.key_runs, kv.run_start = torch.from_numpy(dealt.runs.copy()).to(DEV), torch.from_numpy(dealt.run_start.copy()).to(DEV)
+            kv.runs_window, kv.runs_merge, kv.runs_for_blocks = window, dealt.merge, False
+            assert dealt.merge or target is None
+            out = ops.attention_mfma(q.reshape(T, nq * d).to(DEV), nq, nkv, d, kv, batch, window, scale)
+            _close(out.reshape(T, nq, d), ref, ATTN_TOL, "decode attention over runs of keys, q finished")
 
 
 @pytest.mark.parametrize("with_norm,with_rope", [(True, True), (False, True), (True, False)])

@@ -644,6 +644,18 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
     if batch.max_new_tokens == 1:
         # decoding only: a wave per request, kv head and run of keys; sizes come from the tables
         tiles = -(-G // 16)
+        runs = getattr(kv, "key_runs", None)
+        if splits is None and runs is not None and kv.runs_window == int(window) and T == R:
+            # (the keys dealt into runs by the step's tables; entry i's token is row i)
+            part_o = torch.empty(runs.shape[0], nq, d, dtype=torch.float32, device=q.device)
+            part_ml = torch.empty(runs.shape[0], nq, 2, dtype=torch.float32, device=q.device)
+            _lib.check(L.tff_attention_mfma_runs(
+                q.data_ptr(), q.stride(0), out.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), k_cache.data_ptr(),
+                v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(), batch.start_pos.data_ptr(),
+                runs.data_ptr(), kv.run_start.data_ptr(), batch.cu_tokens.data_ptr(), runs.shape[0], R,
+                1 if kv.runs_merge else 0, T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale),
+                stream))
+            return out
         if splits is None:
             splits = pick_splits(R * tiles * nkv, batch.max_context)
         launch(None, R * tiles, None, 0, tiles, 16, splits)
