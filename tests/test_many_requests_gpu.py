@@ -210,3 +210,48 @@ def test_a_long_request_among_short_ones(tmp_path, n, graphs, monkeypatch):
         r = eng.pop_result(i)
         assert r.finish_reason == "length" and len(r.output) == news[i]
         check_choices(d, r, "bfloat16", None)
+
+
+@pytest.mark.parametrize("seed", range(2))
+def test_random_workloads_of_long_and_short_requests(tmp_path, seed, monkeypatch):
+    """Requests of twenty to twenty-five hundred tokens under continuous batching on a pool that
+    holds a third of them, with decode graphs and steps launched ahead: the runs of keys
+    change with every admission, end and preemption, the captured steps switch between their
+    variants, prompt portions run beside requests that decode over long contexts.  Every kept row
+    of logits against the plain implementation, every token the plain sampler's choice."""
+    import random
+    from helpers import TINY_E, make_model_dir
+    from tffinfer_amd import EngineOptions, LLMEngine, SamplingConfig
+    rng = random.Random(77 + seed)
+    cfg = dict(TINY_E, max_position_embeddings=4096)
+    d = make_model_dir(str(tmp_path / "E"), cfg, 62 + seed)
+    V = cfg["vocab_size"]
+    seen = _watch(monkeypatch)
+    n, ps = 12, 16
+    reqs, need = [], 0
+    for i in range(n):
+        plen = rng.choice([rng.randrange(20, 200), rng.randrange(300, 900), rng.randrange(1200, 2500)])
+        new = rng.randrange(6, 22)
+        sc = SamplingConfig("random", temperature=0.8, seed=rng.randrange(1 << 20)) if i % 4 == 1 else SamplingConfig()
+        reqs.append(dict(prompt_ids=random_tokens(plen, V, 4000 + 17 * seed + i), sampling=sc, max_new_tokens=new,
+                         ignore_eos=True, request_id=i))
+        need += -(-(plen + new) // ps)
+    biggest = max(-(-(len(r["prompt_ids"]) + r["max_new_tokens"]) // ps) for r in reqs)
+    opt = EngineOptions(dtype="bfloat16", page_size=ps, num_pages=max(biggest + 2, int(0.35 * need)), max_num_seqs=8,
+                        max_num_batched_tokens=512, prefill_chunk=384, max_model_len=2600, use_graphs=True, run_ahead=True)
+    eng = LLMEngine.from_model_dir(d, opt)
+    eng.keep_logits = True
+    arrivals = {}
+    for r in reqs:
+        arrivals.setdefault(rng.randrange(0, 10), []).append(r)
+    drive(eng, arrivals)
+    st = eng.scheduler.stats
+    variants = sorted({v for g in eng.runner._graphs.values() for v in g._variants})
+    print(f"seed {seed}: {st.steps} steps, {st.preemptions} preemptions, {eng.steps_ahead} launched ahead, "
+          f"graphs {sorted(eng.runner._graphs)}, variants {variants}")
+    assert True in seen["merge"], "no step cut a request's keys into several runs"
+    for r in reqs:
+        res = eng.pop_result(r["request_id"])
+        assert res.finish_reason == "length" and len(res.output) == r["max_new_tokens"]
+        check_choices(d, res, "bfloat16", r["sampling"])
+    assert all(g.pool.num_used == 0 for g in eng.runner.cache.groups)
