@@ -12,7 +12,10 @@ tensors that no request holds, and whose logits nobody reads.
 
 Nothing in a captured step clears memory with a memset node, and the kernels
 take every size from the tables, so one graph serves any mix of context
-lengths.
+lengths.  Among the tables are the runs of keys that the host deals the
+requests' keys into for the attention (``kernels.key_runs``); what the dealing
+finds (rows of several runs or none; single waves or blocks of eight) selects
+among a few captured variants of the step.
 
 A model may hold parts that cannot be captured (a mixer that loops on the host
 over the step's entries).  The step is then cut into pieces at those layer
@@ -255,8 +258,8 @@ class DecodeGraph:
         pieces = [_Piece(safe, items) for safe, items in rn.model.graph_pieces()]
         for gt, blocks in zip(self.batch.groups, variant[1]):
             gt.runs_merge, gt.runs_for_blocks = variant[0], blocks
-        # the decode attention sizes its key splits for the longest context the engine allows
-        # (batch.max_context), so the launch is the same whatever the requests hold
+        # (the decode attention's launch is sized by the tables of runs of keys, whose size depends
+        # on the bucket's rows only: the same launch whatever the requests hold)
         side = torch.cuda.Stream(device=rn.device)
         side.wait_stream(torch.cuda.current_stream(rn.device))
         # No collection of garbage may run while the stream records: the finaliser of an old

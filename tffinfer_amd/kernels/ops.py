@@ -576,6 +576,7 @@ def _pick_block_cols(batch, G: int, nkv: int, window: int, device, which: str, h
     return cache[key]
 
 
+#: (for a caller that brings no runs of keys, see ``kernels.key_runs``, which is how the engine's steps come)
 #: entries x kv heads from which a decode step gives every pair a block of eight waves that
 #: split its keys and merge in LDS, instead of splitting the keys over blocks of one wave and
 #: merging in a second kernel.  A block a pair keeps only as many CUs busy as there are pairs, and
