@@ -110,7 +110,9 @@ def large_points(args, gen) -> dict:
                             max_num_seqs=32, max_num_batched_tokens=1024, prefill_chunk=512,
                             max_model_len=cfg["max_position_embeddings"], use_graphs=not args.no_graphs)
         engine = LLMEngine(model, opt)
-        out["mixed32_14b_tokens_per_s"] = M.measure_mixed(engine, gen, 32, cfg["vocab_size"])["total_tokens_per_s"]
+        # (a generator of its own: the same 32 prompts whatever was measured before, those of `--mixed 32 --shape 14b`)
+        own = torch.Generator().manual_seed(args.seed)
+        out["mixed32_14b_tokens_per_s"] = M.measure_mixed(engine, own, 32, cfg["vocab_size"])["total_tokens_per_s"]
         del engine, model
     except Exception as e:      # the headline figures must not be lost to a side measurement
         print(f"bench: the 14B point failed: {e}", file=sys.stderr)
