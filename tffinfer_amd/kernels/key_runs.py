@@ -19,12 +19,12 @@ more as long as BUSY_WAVES waves have work, never under MIN_STEPS; with so many
 requests that the waves' fair share is most of a request, a run a request.
 
 With as many pairs of request and kv head as BLOCK_PAIRS says (most of a round
-of a block a CU, or of two), and requests of about one length (the longest no more than some two times the
-average, see BLOCK_RATE_SHARE), a block of eight waves per request and kv head, which merges its waves'
-results in LDS, is faster than single waves whose results a second kernel
-merges: every request is one run then, and ``blocks`` says so.  A CU holds one
-such block, and a block is as slow as its request is long, so uneven lengths
-go to single waves.
+of a block a CU, or of two), and requests of about one length (the longest no
+more than some two times the average, see BLOCK_RATE_SHARE), a block of eight
+waves per request and kv head, which merges its waves' results in LDS, is
+faster than single waves whose results a second kernel merges: every request
+is one run then, and ``blocks`` says so.  A CU holds one such block, and a
+block is as slow as its request is long, so uneven lengths go to single waves.
 
 Pure host code (numpy).  The reference has one sequence per forward and no such
 table (src/core/runtime/InferRuntime.cu:415-429).
@@ -85,8 +85,8 @@ def deal_key_runs(positions, window: int, waves_per_run: int, runs_out: np.ndarr
     ``waves_per_run``: waves (or blocks) that the kernel starts per run: the kv heads.  ``blocks``:
     whether a run gets a block of eight waves (None: by the number of rows and their lengths).
     ``live``: the first so many rows are requests, the others padding (a captured step's), which
-    does not count where the requests' number and lengths decide.  ``target`` and ``min_steps`` override the number of waves (or blocks) aimed at and the
-    shortest run (for tests).
+    does not count where the requests' number and lengths decide.  ``target`` and ``min_steps``
+    override the number of waves (or blocks) aimed at and the shortest run (for tests).
 
     The runs of row r are ``run_start[r] .. run_start[r + 1] - 1``, in the order of their keys,
     without gap or overlap, from the row's first visible key rounded down to a multiple of
@@ -115,7 +115,6 @@ def deal_key_runs(positions, window: int, waves_per_run: int, runs_out: np.ndarr
         pairs = mine.shape[0] * wps
         spread = max(1.2, pairs / (BLOCK_RATE_SHARE * -(-pairs // CUS)))
         blocks = wants_blocks(mine.shape[0], wps) and int(mine.max()) * mine.shape[0] <= spread * int(mine.sum())
-    slots = RESIDENT_WAVES
     if blocks:
         # a run a row, unless a test asks for more
         n = np.ones(R, dtype=np.int64)
@@ -140,7 +139,7 @@ def deal_key_runs(positions, window: int, waves_per_run: int, runs_out: np.ndarr
             chunk = floor
             n = np.maximum(1, steps // chunk)  # no run shorter than the floor
     # within what the GPU holds at once (and the tables), where longer runs can make it so
-    limit = min(slots, cap * wps)
+    limit = min(RESIDENT_WAVES, cap * wps)
     while wps * int(n.sum()) > limit and int(n.max()) > 1:
         chunk += max(1, chunk // 4)
         n = -(-steps // chunk)
