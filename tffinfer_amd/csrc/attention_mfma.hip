@@ -712,28 +712,30 @@ __global__ __launch_bounds__(256) void attn_split_reduce_few_kernel(const float*
 }
 
 // The same for runs of keys dealt by the host: entry r has the runs run_start[r] ..
-// run_start[r + 1] - 1, any number of them, their partial results one after the other.  One wave
-// per (entry, head), four to a block; an entry of one run has its result already.  The first
-// sixteen runs' elements are asked for together with the maxima and sums (lane s takes those of
-// run s, s + 64, ...), the weights of those runs then come from the lanes that hold them; further
-// runs are fetched sixteen at a time, every lane reading their maxima and sums itself (one address
-// for the whole wave).  Every lane adds up its own elements of the head in the order of the runs.
+// run_start[r + 1] - 1, any number of them, their partial results one after the other.  One block
+// of four waves per (entry, head); an entry of one run has its result already.  The runs go to the
+// waves sixteen at a time, in turn: up to sixteen runs are the first wave's alone (the others end
+// at once), a hundred are two rounds a wave instead of seven one after the other, each a round
+// trip to memory.  The first wave asks for its first sixteen runs' elements together with the
+// maxima and sums (lane s takes those of run s, s + 64, ...), the weights of those runs then come
+// from the lanes that hold them; in the other rounds every lane reads the runs' maxima and sums
+// itself (one address for the whole wave).  Every lane adds up its own elements of the head in the
+// order of its wave's runs, and the first wave adds the other waves' sums to its own in their order.
 __global__ __launch_bounds__(256) void attn_run_merge_kernel(const float* __restrict__ part_o,
                                                               const float* __restrict__ part_ml,
                                                               bf16_t* __restrict__ out,
                                                               const int32_t* __restrict__ run_start,
                                                               const int32_t* __restrict__ tokens,
                                                               int R, int nq, int d) {
-    const int lane = threadIdx.x & 63;
-    const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);     // (entry, head), heads fastest
-    if (pair >= R * nq) return;
+    constexpr int AHEAD = 16;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int pair = blockIdx.x;                              // (entry, head), heads fastest
     const int r = pair / nq, h = pair - r * nq;
     const int first = run_start[r], count = run_start[r + 1] - first;
-    if (count <= 1) return;
+    if (count <= 1 || (count <= AHEAD && wv > 0)) return;     // (with up to sixteen runs no wave waits for another below)
     const size_t stride_ml = (size_t)nq * 2, stride_o = (size_t)nq * d;
     const float* ml = part_ml + ((size_t)first * nq + h) * 2;
     const float* po = part_o + ((size_t)first * nq + h) * d;
-    constexpr int AHEAD = 16;
     const int e0 = 2 * lane, e1 = 128 + 2 * lane;             // d <= 256 and even: up to two pairs of elements a lane
     float ms0 = -INFINITY, ls0 = 0.f, m = -INFINITY;
     if (lane < count) {
@@ -742,29 +744,33 @@ __global__ __launch_bounds__(256) void attn_run_merge_kernel(const float* __rest
         m = ms0;
     }
     float2 v[AHEAD][2];
+    if (wv == 0) {
 #pragma unroll
-    for (int u = 0; u < AHEAD; ++u) {
-        const size_t o = (size_t)min(u, count - 1) * stride_o;
-        v[u][0] = e0 < d ? *reinterpret_cast<const float2*>(po + o + e0) : make_float2(0.f, 0.f);
-        v[u][1] = e1 < d ? *reinterpret_cast<const float2*>(po + o + e1) : make_float2(0.f, 0.f);
+        for (int u = 0; u < AHEAD; ++u) {
+            const size_t o = (size_t)min(u, count - 1) * stride_o;
+            v[u][0] = e0 < d ? *reinterpret_cast<const float2*>(po + o + e0) : make_float2(0.f, 0.f);
+            v[u][1] = e1 < d ? *reinterpret_cast<const float2*>(po + o + e1) : make_float2(0.f, 0.f);
+        }
     }
     for (int s = lane + 64; s < count; s += 64) m = fmaxf(m, ml[s * stride_ml]);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-    const float w0 = ms0 == -INFINITY ? 0.f : __expf(ms0 - m);   // (a lane past the last run: 0)
     float l = 0.f;
     float2 acc[2] = {make_float2(0.f, 0.f), make_float2(0.f, 0.f)};
+    if (wv == 0) {
+        const float w0 = ms0 == -INFINITY ? 0.f : __expf(ms0 - m);   // (a lane past the last run: 0)
 #pragma unroll
-    for (int u = 0; u < AHEAD; ++u) {
-        const float w = __shfl(w0, u, 64);
-        l = fmaf(__shfl(ls0, u, 64), w, l);
+        for (int u = 0; u < AHEAD; ++u) {
+            const float w = __shfl(w0, u, 64);
+            l = fmaf(__shfl(ls0, u, 64), w, l);
 #pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            acc[k].x = fmaf(v[u][k].x, w, acc[k].x);
-            acc[k].y = fmaf(v[u][k].y, w, acc[k].y);
+            for (int k = 0; k < 2; ++k) {
+                acc[k].x = fmaf(v[u][k].x, w, acc[k].x);
+                acc[k].y = fmaf(v[u][k].y, w, acc[k].y);
+            }
         }
     }
-    for (int s0 = AHEAD; s0 < count; s0 += AHEAD) {
+    for (int s0 = AHEAD * (wv == 0 ? 4 : wv); s0 < count; s0 += 4 * AHEAD) {
         float w[AHEAD];
 #pragma unroll
         for (int u = 0; u < AHEAD; ++u) {
@@ -782,6 +788,22 @@ __global__ __launch_bounds__(256) void attn_run_merge_kernel(const float* __rest
                 acc[k].x = fmaf(v[u][k].x, w[u], acc[k].x);
                 acc[k].y = fmaf(v[u][k].y, w[u], acc[k].y);
             }
+    }
+    if (count > AHEAD) {
+        // (all four waves are still here, one without runs with sums of zero)
+        __shared__ float4 sum_o[3][64];
+        __shared__ float sum_l[3];
+        if (wv > 0) {
+            sum_o[wv - 1][lane] = make_float4(acc[0].x, acc[0].y, acc[1].x, acc[1].y);
+            if (lane == 0) sum_l[wv - 1] = l;
+        }
+        __syncthreads();
+        if (wv > 0) return;
+        for (int o = 0; o < 3; ++o) {
+            const float4 t = sum_o[o][lane];
+            acc[0].x += t.x; acc[0].y += t.y; acc[1].x += t.z; acc[1].y += t.w;
+            l += sum_l[o];
+        }
     }
     const float inv = 1.0f / l;
     bf16_t* o = out + ((size_t)(tokens ? tokens[r] : r) * nq + h) * d;   // (tokens: the row of out that entry r's token has)
@@ -1450,7 +1472,7 @@ TFF_API int tff_attention_decode_runs(const void* qkv, int qkv_stride, void* out
     }
 #undef TFF_ATTN_CASE
     if (rc || !merge) return rc;
-    attn_run_merge_kernel<<<(R * nq + 3) / 4, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, run_start, nullptr, R, nq, d);
+    attn_run_merge_kernel<<<R * nq, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, run_start, nullptr, R, nq, d);
     return tff_check_launch("attention_run_merge");
 }
 
@@ -1504,7 +1526,7 @@ TFF_API int tff_attention_mfma_runs(const void* q, int q_stride, void* out, floa
     }
 #undef TFF_ATTN_CASE
     if (rc || !merge) return rc;
-    attn_run_merge_kernel<<<(num_entries * nq + 3) / 4, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, run_start, tokens,
+    attn_run_merge_kernel<<<num_entries * nq, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, run_start, tokens,
                                                                     num_entries, nq, d);
     return tff_check_launch("attention_run_merge");
 }
