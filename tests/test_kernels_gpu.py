@@ -335,7 +335,7 @@ ONE_BY_FOUR_CASES = [
     # M, N, K, gated: few rows and K in units of 64, so tiles of 128 rows on four waves side by side
     (100, 6150, 4096, False),      # 128 x 128, K split; rows of the result that are no multiple of 16 bytes
     (120, 24576, 4096, True),      # 128 x 128, gated
-    (40, 51184, 1024, True),       # 128 x 256, gated, a last column tile of a few columns
+    (70, 51184, 1024, True),       # 128 x 256, gated, a last column tile of a few columns
     (70, 40000, 512, False),       # 128 x 256
     (36, 66752, 640, False),       # 128 x 384
     (102, 73088, 1216, True),      # 128 x 384, gated
@@ -386,6 +386,62 @@ def test_cases_of_128_rows_cover_every_tile_width():
     assert {(128, False), (256, False), (384, False), (128, True), (256, True), (384, True)} <= widths, widths
 
 
+FEW_ROWS_CASES = [
+    # M, N, K, gated: 17 to 64 rows and K in units of 64, so tiles of 64 or 32 rows on four waves side by side
+    (40, 6150, 4096, False),       # 64 x 128, K split; handed on: 64 x 256; rows of the result that are no multiple of 16 bytes
+    (20, 24576, 4096, True),       # 32 x 128, gated
+    (64, 40000, 512, False),       # 64 x 256, every row of the tile
+    (17, 34816, 5120, True),       # 32 x 256, gated
+    (50, 34816, 320, True),        # 64 x 256, gated, an odd number of units of K
+    (33, 4096, 12288, False),      # 64 x 128, eight parts: added up, and handed on
+    (30, 5120, 5120, False),       # 32 x 128, four parts
+    (24, 10240, 5120, False),      # 32 x 256, four parts
+    (60, 24560, 192, True),        # 64 x 128, gated, a result whose rows are no multiple of 16 bytes
+    (18, 300, 64, False),          # 32 x 128, a single unit of K, a last column tile of a few columns
+    (32, 8200, 128, False),        # 32 x 128, every row of the tile
+]
+
+
+@pytest.mark.parametrize("M,N,K,glu", FEW_ROWS_CASES)
+def test_linear_on_tiles_of_64_and_32_rows(M, N, K, glu):
+    """The four-wave kernel with its waves side by side and four or two row groups a wave (17 to 64
+    rows: a decode step of so many requests): both heights and widths, gated or not, ragged edges, a
+    row stride beyond K, K split over blocks with the sums added or handed on."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(N + K)
+    wide = torch.randn(M, K + 72, generator=g).to(torch.bfloat16).to(DEV)
+    x = wide[:, :K].contiguous()
+    if glu:
+        I = N // 2
+        gate = (torch.randn(I, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+        up = (torch.randn(I, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+        assert _gemm_plan(M, 2 * I, K, 1)[0] == (32 if M <= 32 else 64)
+        a, b = ops.linear(x.float(), gate.float()), ops.linear(x.float(), up.float())
+        ref = a / (1 + torch.exp(-a)) * b
+        pw = ops.pack_gate_up(gate, up)
+        _close(ops.linear(x, pw, out_dtype=torch.float32), ref, 3e-5, "gated product")
+        _close(ops.linear(wide[:, :K], pw), ref, 8e-3, "gated product, strided rows, bfloat16 result")
+        return
+    w = (torch.randn(N, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+    pw = ops.pack_weight(w)
+    ref = ops.linear(x.float(), w.float())
+    for keep in (0, 1):
+        r, c, sp = _gemm_plan(M, N, K, 0, keep)
+        assert r in (32, 64) and r >= min(M, 33), (r, c, sp)
+        y = ops.linear(x, pw, out_dtype=torch.float32, partials=bool(keep))
+        if keep and sp > 1:
+            assert y.dim() == 3 and y.shape[0] == sp
+        _close(ops.as_tensor(y), ref, 3e-5, f"product (keep={keep}, {r} x {c}, {sp} parts)")
+        if K >= 4096:
+            assert sp > 1, "a case meant to split K"
+    _close(ops.linear(wide[:, :K], pw), ref, 8e-3, "strided rows, bfloat16 result")
+
+
+def test_cases_of_few_rows_cover_every_tile():
+    tiles = {(_gemm_plan(M, N, K, int(glu))[:2], glu) for M, N, K, glu in FEW_ROWS_CASES}
+    assert {((r, c), glu) for r in (32, 64) for c in (128, 256) for glu in (False, True)} <= tiles, tiles
+
+
 @pytest.mark.parametrize("M,N,K", [(2600, 6144, 264), (4500, 520, 200), (1100, 300, 96), (9000, 130, 64),
                                    (2304, 2100, 72)])
 def test_linear_with_many_row_tiles(M, N, K):
@@ -415,14 +471,16 @@ def test_gemm_plan():
     # 9 to 16 rows, 320 column groups (two rounds for 64 CUs, one for the rest), partial sums wanted
     # anyway and a weight large enough: tiles that split K instead of the streaming kernel; up to 8
     # rows, or with a weight that is not so large, the streaming kernel with two column groups a block
-    assert plan(12, 5120, 17408, keep=1)[0] in (64, 128) and plan(12, 5120, 17408, keep=1)[2] > 1
+    assert plan(12, 5120, 17408, keep=1)[0] in (32, 64, 128) and plan(12, 5120, 17408, keep=1)[2] > 1
     assert plan(8, 5120, 17408, keep=1) == (0, 0, 1) and plan(16, 5120, 8192, keep=1) == (0, 0, 1)
     assert plan(8, 5120, 8192) == (0, 0, 1) and plan(8, 5120, 5120, keep=1) == (0, 0, 1)
     assert plan(8, 4096, 12288, keep=1) == (0, 0, 1)
     assert plan(64, 4096, 12288) == (64, 128, 8)
     assert plan(64, 151936, 4096)[0] in (64, 128) and plan(64, 151936, 4096)[2] == 1
+    assert plan(32, 24576, 4096, 1) == (32, 128, 1) and plan(64, 34816, 5120, 1) == (64, 256, 1)   # up to 64 rows: tiles of so many
+    assert plan(65, 24576, 4096, 1)[0] == 128 and plan(33, 24576, 4096, 1)[0] == 64
     assert plan(128, 24576, 4096, 1) == (128, 128, 1)    # few rows: tiles of 128 rows, as many blocks as the columns give
-    assert plan(32, 51200, 5120, 1)[:2] == (128, 256)
+    assert plan(32, 51200, 5120, 1)[:2] == (32, 256)
     assert plan(2048, 24576, 4096, 1)[0] == 256 and plan(2048, 24576, 4096, 1)[2] == 1
     assert plan(2048, 24584, 4104, 1) == (256, 256, 1)  # K no multiple of 64: the sixteen-wave tiles, gated on 256 columns only
     assert plan(4096, 4096, 4096) == (256, 256, 1)

@@ -374,7 +374,7 @@ __device__ __forceinline__ int w4_lane() {
 // width that is no multiple of 8).  This is the kernel's only way out for its results on purpose:
 // with a second one beside it the compiler converts accumulators for both before the branch, runs
 // out of registers and spills, and a kernel that uses scratch memory pays some 15 us at its launch.
-template <int OW, int REGION, typename TO, typename F>
+template <int OW, int REGION, typename TO, int WTM = 8, typename F>
 __device__ __forceinline__ void w4_store_rows(char* region, F val, TO* out, size_t ld, int m_base, int n_base,
                                               int M, int ncols, int lane, bool vec) {
     constexpr int E = 16 / (int)sizeof(TO);           // columns in 16 bytes
@@ -382,15 +382,15 @@ __device__ __forceinline__ void w4_store_rows(char* region, F val, TO* out, size
     constexpr int LPR = CPR <= 4 ? 4 : CPR <= 8 ? 8 : CPR <= 16 ? 16 : 32;   // lanes a row
     static_assert(CPR <= LPR, "a row's pieces fit its lanes");
     constexpr int RPI = 64 / LPR;                     // rows a store instruction
-    constexpr int RC = 8 * 16 * RBP <= REGION ? 8 : 4;
-    static_assert(RC * 16 * RBP <= REGION, "the wave's region of LDS holds four row groups at least");
+    constexpr int RC = WTM * 16 * RBP <= REGION ? WTM : WTM / 2;   // row groups that go through the region at a time
+    static_assert(RC >= 1 && RC * 16 * RBP <= REGION, "the wave's region of LDS holds half its row groups at least");
     const int fr = lane & 15, fg = lane >> 4;
     const int srow = lane / LPR, sch = lane % LPR;    // this lane's row of an instruction's, and its piece
     const int n = n_base + sch * E;
     const bool mine = sch < CPR && n < ncols;
     const char* src = region + srow * RBP + sch * 16;
 #pragma unroll
-    for (int p = 0; p < 8 / RC; ++p) {
+    for (int p = 0; p < WTM / RC; ++p) {
 #pragma unroll
         for (int jj = 0; jj < RC; ++jj) {
             __builtin_amdgcn_sched_barrier(0);   // a row group at a time: all accumulators converted at once do not fit the registers
@@ -442,14 +442,16 @@ struct W4Scale {
     int stride, count;
     float inv_dim, eps;
 };
-template <int WTN, int NWS, bool GLU, typename TC, int WGM = 2, bool SCALE = false>
+template <int WTN, int NWS, bool GLU, typename TC, int WGM = 2, bool SCALE = false, int WTM = 8>
 __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, TC* __restrict__ C, int M, int N,
     int K, int lda, int KB, int n_out, W4Scale sc) {
     static_assert(!SCALE || WGM == 1, "rows that lack their norm's factor: up to 16, one row tile");
     // WGM: waves along the rows, 2 (a block tile of 256 rows, two waves side by side) or 1 (128 rows, four side by side)
-    constexpr int NW = 4, WTM = 8, NA = 3, WGN = NW / WGM;
+    // WTM: row groups of 16 a wave, 8, or with the waves side by side 4 or 2 (a block tile of 64 or 32 rows)
+    constexpr int NW = 4, NA = 3, WGN = NW / WGM;
     static_assert(WGM == 1 || WGM == 2, "four waves as 2 x 2 or 1 x 4");
+    static_assert(WTM == 8 || (WGM == 1 && (WTM == 4 || WTM == 2)), "fewer rows a wave only with the waves side by side");
     constexpr int BM = WGM * WTM * 16, BN = WGN * WTN * 16;
     constexpr int WF = BN / 16;                       // W fragments a k-tile, 1 KB each
     constexpr int ACP = BM / 8;                       // A copies a unit, 1 KB each
@@ -655,19 +657,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(
     };
     if constexpr (GLU) {
         static_assert(WTN % 2 == 0, "gate and up groups come in pairs");
-        w4_store_rows<WTN / 2, REGION, TC>(region, [&](int i, int jj) { return silu_mul(scaled(acc[2 * i][jj]), scaled(acc[2 * i + 1][jj])); },
+        w4_store_rows<WTN / 2, REGION, TC, WTM>(region, [&](int i, int jj) { return silu_mul(scaled(acc[2 * i][jj]), scaled(acc[2 * i + 1][jj])); },
                                            C, (size_t)n_out, mw, (n0 + wn * WTN * 16) / 2, M, n_out, lane_out,
                                            n_out % E == 0);
     } else {
         // (partial sums of a split K: plane blockIdx.z of the launcher's float32 workspace, which it passes as C)
         TC* out = C + (size_t)blockIdx.z * M * N;
-        w4_store_rows<WTN, REGION, TC>(region, [&](int i, int jj) { return scaled(acc[i][jj]); }, out, (size_t)N, mw,
+        w4_store_rows<WTN, REGION, TC, WTM>(region, [&](int i, int jj) { return scaled(acc[i][jj]); }, out, (size_t)N, mw,
                                        n0 + wn * WTN * 16, M, N, lane_out, N % E == 0);
     }
 }
 
 // splits > 1: the blocks of a tile split K among them in units of 64; part holds splits * M * N floats
-template <int WTN, int NWS, bool GLU = false, int WGM = 2, bool SCALE = false>
+template <int WTN, int NWS, bool GLU = false, int WGM = 2, bool SCALE = false, int WTM = 8>
 static int launch_w4(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int K, int lda, int c_dtype,
                      int n_out, hipStream_t s, int splits = 1, float* part = nullptr, bool reduce = true,
                      W4Scale sc = W4Scale{nullptr, 0, 0, 0.f, 0.f}) {
@@ -675,7 +677,7 @@ static int launch_w4(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, i
                 "gemm: rows that lack their norm's factor: up to 16 of them and K in one part");
     TFF_REQUIRE(K % 64 == 0, "gemm: the four-wave tiles take K in units of 64, not K=%d", K);
     const int KB = K / 32;
-    constexpr int BM = 128 * WGM, BN = (4 / WGM) * WTN * 16;
+    constexpr int BM = 16 * WTM * WGM, BN = (4 / WGM) * WTN * 16;
     if (splits <= 1 || !part) { splits = 1; part = nullptr; }
     TFF_REQUIRE(splits <= KB / 2, "gemm: %d parts of %d units of K", splits, KB / 2);
     const long TM = (M + BM - 1) / BM, TN = (N + BN - 1) / BN;
@@ -685,11 +687,11 @@ static int launch_w4(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, i
     const dim3 grid((unsigned)tiles, 1, splits);
     // the blocks of a split K leave plain float32 sums, plane by plane; a gate is applied when they are added up
     if (splits > 1)
-        gemm_bf16_w4_kernel<WTN, NWS, false, float, WGM><<<grid, 256, 0, s>>>(A, Wp, part, M, N, K, lda, KB, 0, sc);
+        gemm_bf16_w4_kernel<WTN, NWS, false, float, WGM, false, WTM><<<grid, 256, 0, s>>>(A, Wp, part, M, N, K, lda, KB, 0, sc);
     else if (c_dtype == TFF_F32)
-        gemm_bf16_w4_kernel<WTN, NWS, GLU, float, WGM, SCALE><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out, sc);
+        gemm_bf16_w4_kernel<WTN, NWS, GLU, float, WGM, SCALE, WTM><<<grid, 256, 0, s>>>(A, Wp, (float*)C, M, N, K, lda, KB, n_out, sc);
     else
-        gemm_bf16_w4_kernel<WTN, NWS, GLU, bf16_t, WGM, SCALE><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out, sc);
+        gemm_bf16_w4_kernel<WTN, NWS, GLU, bf16_t, WGM, SCALE, WTM><<<grid, 256, 0, s>>>(A, Wp, (bf16_t*)C, M, N, K, lda, KB, n_out, sc);
     if (int rc = tff_check_launch("gemm_bf16_w4")) return rc;
     if (splits > 1 && reduce) {
         const int No = GLU ? n_out : N;
@@ -1001,8 +1003,9 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
 
 // The tiled product's plan for M > 16: which tile, and into how many parts the blocks of a
 // tile split K, by a small cost model (see plan_for).  With K in units of 64: the four-wave
-// kernel's tiles of 256 rows (256, 192 or 128 columns) and of 128 rows (384, 256 or 128 columns),
-// and the sixteen-wave kernel's 64 x 128; otherwise the sixteen-wave kernel's tiles.
+// kernel's tiles of 256 rows (256, 192 or 128 columns), of 128 rows (384, 256 or 128 columns) and,
+// up to 64 and 32 rows, of 64 and 32 rows (256 or 128 columns), and from 65 to 512 rows the
+// sixteen-wave kernel's 64 x 128; otherwise the sixteen-wave kernel's tiles.
 struct GemmPlan { int tile; int bn; int splits; };   // tile = rows of a block tile
 // Compute units of the current device (256 on an MI355X, which the rates below were fitted on; a
 // device with another count gets plans for its own number of blocks a round).  256 if it cannot
@@ -1080,15 +1083,23 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
         // constants were fitted to measurements of the four products of the 8B, 14B and 32B shapes at
         // 17 .. 4,096 rows on an MI355X (weights in turn, so that none comes from a cache; every tile
         // with 1 .. 8 parts, 204 cases): the pick is 0.3 % from the best candidate on average, 6 % at worst.
+        // Up to 64 rows the four waves side by side take 64 or 32 rows: a product of so few rows is its
+        // weight's stream, and a block that does not work through 128 rows for 32 asks for its next
+        // columns sooner (3 to 10 % less time than the tiles of 128 rows and the sixteen-wave kernel's
+        // 64 x 128 on the four products of the three shapes at 17 to 64 rows; their rates fitted to
+        // those 88 cases stand for that, the pick 0.5 % from the best on average, 5 % at worst).
         struct Cand { int bm, bn, slots; double rate; };
-        static const Cand cands[7] = {{256, 256, 1, 6.01e6}, {256, 192, 1, 5.45e6}, {256, 128, 1, 5.04e6},
-                                      {128, 384, 1, 3.24e6}, {128, 256, 1, 4.61e6}, {128, 128, 1, 3.45e6},
-                                      {64, 128, 2, 2.18e6}};
+        static const Cand cands[11] = {{256, 256, 1, 6.01e6}, {256, 192, 1, 5.45e6}, {256, 128, 1, 5.04e6},
+                                       {128, 384, 1, 3.24e6}, {128, 256, 1, 4.61e6}, {128, 128, 1, 3.45e6},
+                                       {64, 256, 1, 2.4e6}, {64, 128, 1, 2.0e6}, {32, 256, 1, 1.4e6}, {32, 128, 1, 1.3e6},
+                                       {64, 128, 2, 2.18e6}};
         const double HBM = 7.72e6, CU_MAX = 6.0e4;       // bytes a microsecond: all CUs together, one alone
         GemmPlan best = {128, 128, 1};
         double best_t = 1e30;
         for (const Cand& c : cands) {
-            if ((c.bm == 256 && M <= 64) || (c.bm == 64 && M > 512)) continue;
+            if (c.bm == 256 && M <= 64) continue;
+            if (c.slots == 1 && c.bm <= 64 && M > c.bm) continue;         // (four waves side by side: one row tile)
+            if (c.slots == 2 && (M <= 64 || M > 512)) continue;            // (the sixteen-wave kernel)
             for (int S = 1; S <= ((glu && M > 64) ? 2 : 8); S *= 2) {
                 if (S > 1 && nk / S < 4) break;
                 const double blocks = (double)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * S;
@@ -1239,6 +1250,12 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
         TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
                     "gemm: a gated weight of %d rows does not fit %d output columns", N, glu_out);
         if (plan.tile == 0) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, nullptr);
+        if (plan.tile <= 64 && M <= 64 && K % 64 == 0) {     // the four waves side by side on 64 or 32 rows
+            if (plan.tile == 32 && plan.bn == 128) return launch_w4<2, 5, true, 1, false, 2>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+            if (plan.tile == 32) return launch_w4<4, 5, true, 1, false, 2>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+            if (plan.bn == 128) return launch_w4<2, 5, true, 1, false, 4>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+            return launch_w4<4, 5, true, 1, false, 4>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
+        }
         if (plan.tile == 64)
             return launch_async_g<2, 2, 2, 4, 3, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
         if (K % 64 == 0) {
@@ -1258,12 +1275,18 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
         return launch_async_g<4, 4, 4, 4, 5, true, 1, true>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
     }
     if (plan.tile == 0) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, nullptr);
-    if (plan.tile == 64) {
+    if (plan.tile == 64 || plan.tile == 32) {
         // few columns and no room for partial sums: the streaming kernel, whose blocks split K
         // among their waves
         if (S == 1 && planned_splits > 1 && M <= 64) {
             if (M <= 32) return launch_skinny<2, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
             return launch_skinny<4, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
+        }
+        if (M <= 64 && K % 64 == 0) {                        // the four waves side by side on 64 or 32 rows
+            if (plan.tile == 32 && plan.bn == 128) return launch_w4<2, 5, false, 1, false, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+            if (plan.tile == 32) return launch_w4<4, 5, false, 1, false, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+            if (plan.bn == 128) return launch_w4<2, 5, false, 1, false, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
+            return launch_w4<4, 5, false, 1, false, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
         }
         return launch_async_g<2, 2, 2, 4, 3>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
     }
