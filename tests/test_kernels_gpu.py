@@ -181,7 +181,7 @@ def test_norm_taken_into_the_products_on_either_side(M, H, K, N2, glu):
     multiplies by the row's factor.  Against the three steps done one after the other, in float64,
     with the norm's weights and a residual stream whose rows differ in size by orders of magnitude
     (a factor applied to the wrong row, or a norm left out, would show).  The last three cases, gated:
-    a weight so large (or so many rows) that the product after the norm runs on tiles of 128 rows
+    a weight so large (or so many rows) that the product after the norm runs on tiles of 32 rows
     of the four-wave kernel, which takes the rows' factors into its epilogue too."""
     ops = _ops()
     g = torch.Generator().manual_seed(M * 7 + H)
@@ -341,8 +341,6 @@ ONE_BY_FOUR_CASES = [
     (102, 73088, 1216, True),      # 128 x 384, gated
     (100, 4096, 12288, False),     # 128 x 128, eight parts: added up, and handed on
     (300, 34816, 320, False),      # three row tiles of 128, the last one ragged
-    (16, 51200, 5120, True),       # up to 16 rows, gated, a weight so large that the rows go on tiles, not the streaming kernel
-    (3, 49152, 5120, True),
 ]
 
 
@@ -399,6 +397,9 @@ FEW_ROWS_CASES = [
     (60, 24560, 192, True),        # 64 x 128, gated, a result whose rows are no multiple of 16 bytes
     (18, 300, 64, False),          # 32 x 128, a single unit of K, a last column tile of a few columns
     (32, 8200, 128, False),        # 32 x 128, every row of the tile
+    (16, 51200, 5120, True),       # up to 16 rows, gated, a weight so large that the rows go on tiles, not the streaming kernel
+    (3, 49152, 5120, True),
+    (14, 24576, 4096, True),       # (a smaller weight goes there with more rows)
 ]
 
 

@@ -1028,30 +1028,28 @@ static bool two_row_groups(int N) {
     const int nb = (N + 15) / 16, cus = device_cus();
     return nb > cus && nb * 10 <= cus * 16;
 }
-// Up to 16 rows, gated, a very large weight (the 32B shape's gate+up, 262M elements): the streaming
-// kernel's blocks each fetch all of A's rows, and with so many blocks that is traffic enough to show:
-// 94 us against 90 on tiles with one row, 115 against 90 with 16.  Then tiles of 128 rows of the
-// four-wave kernel, K in one part.  (At the 8B and 14B shapes' sizes tiles gain only with K in two
-// parts, which the rows' factors in the epilogue do not go with: the streaming kernel stays.)
-// The streaming kernel's time also grows with the rows (every block fetches them all), the tiles' does
-// not, so smaller weights cross over at more rows: gate+up of the 14B shape (1.8e8 elements) 67 / 71 /
-// 78 / 87 us at 1 / 8 / 12 / 16 rows against 75 on tiles, of the 8B shape (1.0e8) 37 / 38 / 40 / 44 us
-// against 43, of the 4B shape (5e7) 21 / 22 / 25 / 28 against 28.
+// Up to 16 rows, gated: the streaming kernel's blocks each fetch all of A's rows, so its time grows
+// with the rows, and with a very large weight (the 32B shape's gate+up, 262M elements, 3,200 blocks)
+// that traffic shows even with one row.  The four-wave kernel's tiles of 32 rows, K in one part, take
+// the same time whatever the rows, so each weight crosses over at its number of rows (us at 1 / 4 /
+// 8 / 12 / 16 rows, streaming against tiles): the 32B shape 94 / 96 / 100 / 107 / 120 against 91 to
+// 92; the 14B shape (1.8e8 elements) 67 / 69 / 71 / 77 / 89 against 68 to 70; the 8B shape (1.0e8)
+// 36 / 37 / 37 / 40 / 44 against 39; the 4B shape (5e7) 21 / 21 / 22 / 24 / 28 against 25.
 static bool few_rows_gated_on_tiles(int M, int N, int K) {
     const double w = (double)N * K;
-    return K % 64 == 0 && (w >= 2.4e8 || (w >= 1.6e8 && M >= 11) || (w >= 0.9e8 && M >= 15));
+    return K % 64 == 0 && (w >= 2.4e8 || (w >= 1.6e8 && M >= 5) || (w >= 0.9e8 && M >= 12) || (w >= 0.45e8 && M >= 14));
 }
-// One row tile of 128 rows, K in one part: the width (128, 256 or 384 columns) that plan_for's model prices lowest.
-static int plan_rows128(int N, int K) {
+// One row tile of 32 rows, K in one part: the width (128 or 256 columns) that plan_for's model prices lowest.
+static int plan_rows32(int N, int K) {
     const double CUS = (double)device_cus();
-    const int widths[3] = {128, 256, 384};
-    const double rates[3] = {3.45e6, 4.61e6, 3.24e6};
+    const int widths[2] = {128, 256};
+    const double rates[2] = {1.3e6, 1.4e6};
     int best = 256;
     double best_t = 1e30;
-    for (int i = 0; i < 3; ++i) {
+    for (int i = 0; i < 2; ++i) {
         const double blocks = (double)((N + widths[i] - 1) / widths[i]);
         const double bw = fmin(6.0e4, 7.72e6 / fmin(blocks, CUS));
-        const double unit = fmax(2.0 * 128 * widths[i] * 64.0 / rates[i], widths[i] * 128.0 / bw);
+        const double unit = fmax(2.0 * 32 * widths[i] * 64.0 / rates[i], widths[i] * 128.0 / bw);
         const double t = ceil(blocks / CUS) * (K / 64.0 * unit + 3.0);
         if (t < best_t) { best_t = t; best = widths[i]; }
     }
@@ -1065,7 +1063,7 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
     // partial sums anyway and the weight is large enough for the gain (three eighths of its
     // stream) to pay for the norm's own kernel, which the streaming kernel would have taken into
     // its epilogue: then the tiles below, whose blocks split K as finely as it takes.
-    if (M <= 16 && glu && few_rows_gated_on_tiles(M, N, K)) return {128, plan_rows128(N, K), 1};
+    if (M <= 16 && glu && few_rows_gated_on_tiles(M, N, K)) return {32, plan_rows32(N, K), 1};
     if (M <= 16) {
         const int nb = (N + 15) / 16;
         const double fill = (double)nb / (ceil(nb / CUS) * CUS);
@@ -1350,17 +1348,15 @@ TFF_API int tff_gemm_row_scaled(const void* A, const void* Wp, void* C, int M, i
     if (glu_out > 0)
         TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
                     "gemm_row_scaled: a gated weight of %d rows does not fit %d output columns", N, glu_out);
-    // (the four-wave kernel's tiles of 128 rows take the rows' factors into their epilogue too)
+    // (the four-wave kernel's tiles of 32 rows take the rows' factors into their epilogue too)
     if (glu_out > 0 && few_rows_gated_on_tiles(M, N, K)) {
         const W4Scale sc{ss, ss_stride, ss_count, 1.0f / (float)dim, eps};
         const bf16_t* a = (const bf16_t*)A;
         const bf16_t* w = (const bf16_t*)Wp;
         hipStream_t s = (hipStream_t)stream;
-        switch (plan_rows128(N, K)) {
-            case 128: return launch_w4<2, 5, true, 1, true>(a, w, C, M, N, K, lda, c_dtype, glu_out, s, 1, nullptr, true, sc);
-            case 256: return launch_w4<4, 5, true, 1, true>(a, w, C, M, N, K, lda, c_dtype, glu_out, s, 1, nullptr, true, sc);
-            default: return launch_w4<6, 4, true, 1, true>(a, w, C, M, N, K, lda, c_dtype, glu_out, s, 1, nullptr, true, sc);
-        }
+        if (plan_rows32(N, K) == 128)
+            return launch_w4<2, 5, true, 1, true, 2>(a, w, C, M, N, K, lda, c_dtype, glu_out, s, 1, nullptr, true, sc);
+        return launch_w4<4, 5, true, 1, true, 2>(a, w, C, M, N, K, lda, c_dtype, glu_out, s, 1, nullptr, true, sc);
     }
     SkinnyFuse fz{ss, ss_stride, ss_count, 1.0f / (float)dim, eps, nullptr, nullptr, nullptr, nullptr, 0};
     return skinny_for<1>((const bf16_t*)A, (const bf16_t*)Wp, C, M, N, K, lda, c_dtype, glu_out, (hipStream_t)stream, &fz);
