@@ -58,7 +58,8 @@ def parse_args():
                          "prompt portions of --chunk tokens beside decoding requests, 256 tokens generated each")
     ap.add_argument("--chunk", type=int, default=512, help="prompt portion of the --mixed workload")
     ap.add_argument("--budget", type=int, default=0,
-                    help="tokens of a step of the --mixed workload (default: a portion beside every decoding request, at least 1,024)")
+                    help="tokens of a step of the --mixed workload (default: the engine's own default, 2,048: four portions, "
+                         "or fewer beside the requests that decode)")
     ap.add_argument("--token-quantum", type=int, default=None,
                     help="with --mixed: the scheduler cuts steps a little over a multiple of this many tokens down "
                          "to the multiple (default: the engine's own, 256; 0: off)")
@@ -107,7 +108,7 @@ def large_points(args, gen) -> dict:
         cfg = dict(SHAPES["14b"][1])
         model = build_model(cfg, args.seed)
         opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=32 * (4096 + 256 + args.page_size),
-                            max_num_seqs=32, max_num_batched_tokens=1024, prefill_chunk=512,
+                            max_num_seqs=32, prefill_chunk=512,      # (the token budget of a step: the engine's default)
                             max_model_len=cfg["max_position_embeddings"], use_graphs=not args.no_graphs)
         engine = LLMEngine(model, opt)
         # (a generator of its own: the same 32 prompts whatever was measured before, those of `--mixed 32 --shape 14b`)
@@ -243,13 +244,14 @@ def main():
     model = build_model(cfg, args.seed)
     if args.mixed:
         kv_tokens = args.mixed * (4096 + 256 + args.page_size)
+        budget = {"max_num_batched_tokens": max(args.budget, args.chunk, args.mixed)} if args.budget else {}
         opt = EngineOptions(dtype="bfloat16", page_size=args.page_size, kv_tokens=kv_tokens,
-                            max_num_seqs=args.mixed, max_num_batched_tokens=args.budget or max(args.chunk + args.mixed, 1024),
-                            prefill_chunk=args.chunk, max_model_len=cfg["max_position_embeddings"],
-                            use_graphs=not args.no_graphs, token_quantum=args.token_quantum)
+                            max_num_seqs=args.mixed, prefill_chunk=args.chunk, max_model_len=cfg["max_position_embeddings"],
+                            use_graphs=not args.no_graphs, token_quantum=args.token_quantum, **budget)
         engine = LLMEngine(model, opt)
         res = M.measure_mixed(engine, gen, args.mixed, vocab)
-        print(json.dumps({"workload": "mixed", "model": shape_name, "layers_run": L, "chunk": args.chunk, **res}))
+        print(json.dumps({"workload": "mixed", "model": shape_name, "layers_run": L, "chunk": args.chunk,
+                          "budget": opt.max_num_batched_tokens, **res}))
         return
     max_batch = args.batch if (args.no_points or args.only) else max(args.batch, 64)
     total_steps = args.steps + args.warmup + M.decode_slack(max_batch, args.context) + 16
