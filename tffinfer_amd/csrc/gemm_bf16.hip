@@ -1004,8 +1004,8 @@ static int launch_skinny(const bf16_t* A, const bf16_t* Wp, void* C, int M, int 
 // The tiled product's plan for M > 16: which tile, and into how many parts the blocks of a
 // tile split K, by a small cost model (see plan_for).  With K in units of 64: the four-wave
 // kernel's tiles of 256 rows (256, 192 or 128 columns), of 128 rows (384, 256 or 128 columns) and,
-// up to 64 and 32 rows, of 64 and 32 rows (256 or 128 columns), and from 65 to 512 rows the
-// sixteen-wave kernel's 64 x 128; otherwise the sixteen-wave kernel's tiles.
+// up to 64 and 32 rows, of 64 and 32 rows (256 or 128 columns), and from 65 to 512 rows also
+// 64 x 128 with several row tiles; otherwise the sixteen-wave kernel's tiles.
 struct GemmPlan { int tile; int bn; int splits; };   // tile = rows of a block tile
 // Compute units of the current device (256 on an MI355X, which the rates below were fitted on; a
 // device with another count gets plans for its own number of blocks a round).  256 if it cannot
@@ -1074,7 +1074,9 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
     const int nk = (K + 63) / 64;
     if (K % 64 == 0) {
         // The four-wave kernel's tiles (256 rows on 2 x 2 waves, 128 rows on 1 x 4) and, up to 512 rows,
-        // the sixteen-wave kernel's 64 x 128, two blocks to a CU.  A block goes through its part of K in
+        // its 64 x 128, two blocks to a CU (the last candidate; its rate is that of the sixteen-wave
+        // kernel's 64 x 128, which it replaced and is 8 to 17 % faster than at 128 to 512 rows, so
+        // the model picks it rather too seldom).  A block goes through its part of K in
         // units of 64; a unit takes what its MFMAs take at the tile's rate or what its columns of W take
         // to arrive, whichever is longer: a block's share of the HBM stream, at most what one CU pulls.
         // Blocks go round the CUs; each round ends with the pipeline filled and the tile stored.  The
@@ -1097,7 +1099,7 @@ static GemmPlan plan_for(int M, int N, int K, bool glu, bool keep) {
         for (const Cand& c : cands) {
             if (c.bm == 256 && M <= 64) continue;
             if (c.slots == 1 && c.bm <= 64 && M > c.bm) continue;         // (four waves side by side: one row tile)
-            if (c.slots == 2 && (M <= 64 || M > 512)) continue;            // (the sixteen-wave kernel)
+            if (c.slots == 2 && (M <= 64 || M > 512)) continue;            // (64 x 128 with several row tiles)
             for (int S = 1; S <= ((glu && M > 64) ? 2 : 8); S *= 2) {
                 if (S > 1 && nk / S < 4) break;
                 const double blocks = (double)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * S;
@@ -1248,7 +1250,7 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
         TFF_REQUIRE(N % 32 == 0 && glu_out <= N / 2 && glu_out > N / 2 - 16,
                     "gemm: a gated weight of %d rows does not fit %d output columns", N, glu_out);
         if (plan.tile == 0) return skinny_for<0>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, nullptr);
-        if (plan.tile <= 64 && M <= 64 && K % 64 == 0) {     // the four waves side by side on 64 or 32 rows
+        if (plan.tile <= 64 && K % 64 == 0) {                // the four waves side by side on 64 or 32 rows
             if (plan.tile == 32 && plan.bn == 128) return launch_w4<2, 5, true, 1, false, 2>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
             if (plan.tile == 32) return launch_w4<4, 5, true, 1, false, 2>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
             if (plan.bn == 128) return launch_w4<2, 5, true, 1, false, 4>(A, Wp, C, M, N, K, lda, c_dtype, glu_out, s, S, workspace);
@@ -1280,7 +1282,7 @@ int tff_gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* C, int M, int N, int 
             if (M <= 32) return launch_skinny<2, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
             return launch_skinny<4, 2, 4, 8>(A, Wp, C, M, N, K, lda, c_dtype, 0, s);
         }
-        if (M <= 64 && K % 64 == 0) {                        // the four waves side by side on 64 or 32 rows
+        if (K % 64 == 0) {                                   // the four waves side by side on 64 or 32 rows
             if (plan.tile == 32 && plan.bn == 128) return launch_w4<2, 5, false, 1, false, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
             if (plan.tile == 32) return launch_w4<4, 5, false, 1, false, 2>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
             if (plan.bn == 128) return launch_w4<2, 5, false, 1, false, 4>(A, Wp, C, M, N, K, lda, c_dtype, 0, s, S, workspace, red);
